@@ -1,0 +1,148 @@
+/*
+ * pccl_hip.h -- C ABI of the MI355X (gfx950) reduce-copy plugin, libpccl_hip.so.
+ *
+ * This is the boundary the reference's host code binds for its local
+ * reduce-copy / copy path.  In the reference that path is declared but empty:
+ *   - include/plugins/cuda_executor/executor.h   (0 bytes; device executor)
+ *   - include/plugins/cpu_executor/executor.h    (0 bytes; CPU executor)
+ *   - csrc/engine.cc:102-104 Engine::regOp, include/engine.h:19 Engine::exeOp
+ * so each entry point below cites the reference declaration whose role it
+ * fills.  Plain pointers and sizes only; no C++ or torch types; no exception
+ * crosses this boundary.  Every function returns PCCL_OK (0) or a negative
+ * PCCL_ERR_* code; pccl_hip_last_error() gives the text for the calling thread.
+ */
+#ifndef PCCL_HIP_H
+#define PCCL_HIP_H
+
+#include "pccl_op_layout.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- return codes -------------------------------------------------------- */
+#define PCCL_OK 0
+#define PCCL_ERR_INVALID_ARG (-1) /* null pointer, count < 0, n_in/n_out out of range ...  */
+#define PCCL_ERR_UNSUPPORTED (-2) /* unknown dtype / compute / primitive code               */
+#define PCCL_ERR_HIP (-3)         /* a HIP runtime call failed; text in last_error          */
+#define PCCL_ERR_NO_DEVICE (-4)   /* no gfx950 device visible                               */
+#define PCCL_ERR_NOMEM (-5)       /* device allocation failed                               */
+#define PCCL_ERR_MISALIGNED (-6)  /* operand address not a multiple of its element size     */
+#define PCCL_ERR_GRAPH (-7)       /* op graph malformed: cycle, bad uid, too many edges ... */
+
+/* ---- fixed codes used on the wire ---------------------------------------- */
+/* The host layer maps TypeRegistry ids (include/base/registry.h:12-43, ids are
+ * handed out at run time from one shared counter) onto these stable codes. */
+enum pccl_dtype {   /* element types with 16-byte packs in                         */
+  PCCL_F32 = 0,     /* include/plugins/cuda_executor/utils/vector_datatype.h:66    */
+  PCCL_I32 = 1,     /* :64                                                         */
+  PCCL_BF16 = 2,    /* :71 (bf16x8)                                                */
+  PCCL_F16 = 3      /* :70 (f16x8)                                                 */
+};
+enum pccl_compute { /* multimem.h:12-59 only has .add; min/max/prod complete the   */
+  PCCL_SUM = 0,     /* set of ComputeType names the registry is meant to hold      */
+  PCCL_PROD = 1,
+  PCCL_MIN = 2,
+  PCCL_MAX = 3
+};
+enum pccl_primitive { /* PrimitiveOpType, pccl/lang/chunk.py:6-10 */
+  PCCL_COPY = 0,
+  PCCL_REDUCE = 1,
+  PCCL_NOTIFY = 2,
+  PCCL_GET_NOTIFIED = 3
+};
+
+#define PCCL_MAX_INPUTS 8
+#define PCCL_MAX_OUTPUTS 8
+
+/* ---- device + allocator --------------------------------------------------- */
+
+/* Number of usable devices.  Role: CudaDevice::allocatorAvailable,
+ * csrc/plugins/cuda_executor/device.cc:53-57 (cudaGetDeviceCount > 0). */
+int pccl_hip_device_count(int *n);
+
+/* Compute units and HBM bytes of the current device (launch sizing and
+ * reporting; the reference has no counterpart because it has no launches). */
+int pccl_hip_device_info(int *compute_units, long *hbm_bytes, char *name, int name_len);
+
+/* Device memory, size rounded up to 2 MiB, tracked until freed.  nbytes <= 0
+ * yields PCCL_ERR_INVALID_ARG and *p == NULL.  Role: CudaDevice::allocate /
+ * deallocate, csrc/plugins/cuda_executor/device.cc:59-144 (2 MiB granularity
+ * :60,70; nullptr for nbytes <= 0 :61; pointer-keyed bookkeeping :121-144). */
+int pccl_hip_alloc(void **p, long nbytes);
+int pccl_hip_free(void *p);
+
+/* ---- the hot path: one reduce-copy ---------------------------------------- */
+
+/* out[j][i] = cvt(fold_op(up(in[0][i]) ... up(in[n_in-1][i]))) for j < n_out,
+ * i < count.  Strict left fold in input order; float accumulator for
+ * f32/bf16/f16 with one round-to-nearest-even at the end; uint32 wraparound
+ * for i32; n_in == 1 copies bytes.  Any element-aligned addresses; an output
+ * may be the same buffer as an input (in place), other overlaps are undefined.
+ * One kernel launch on `stream` (a hipStream_t; NULL = the default stream);
+ * returns without waiting.
+ * Role: the N-pointer form of multimem_ld_reduce + multimemStore,
+ * include/plugins/cuda_executor/utils/multimem.h:12-102, over operands
+ * described like ChunkMeta, include/base/chunk.h:10-14. */
+int pccl_hip_reduce_copy(int dtype, int compute, const void *const *ins, int n_in,
+                         void *const *outs, int n_out, long count, void *stream);
+
+/* Launch-shape overrides for tuning runs: workgroups per compute unit
+ * (0 = built-in choice) and non-temporal access hint (0/1, -1 = built-in). */
+int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);
+
+/* ---- the op-batching path: a DAG of ops drained by one persistent kernel -- */
+
+/* One IR operation as the host hands it over: the C++ payload level of
+ * PrimitiveOp (pccl/lang/chunk.py:46-55): op kind, operands, dependencies. */
+typedef struct pccl_op_desc {
+  int op_uid;                          /* dense 0..n_ops-1, chunk.py:82-83           */
+  unsigned char primitive;             /* enum pccl_primitive (COPY or REDUCE)        */
+  unsigned char dtype;                 /* enum pccl_dtype                             */
+  unsigned char compute;               /* enum pccl_compute                           */
+  unsigned char n_in;                  /* 1..8                                        */
+  unsigned char n_out;                 /* 1..8                                        */
+  unsigned char reserved[3];
+  const void *ins[PCCL_MAX_INPUTS];
+  void *outs[PCCL_MAX_OUTPUTS];
+  long count;                          /* elements per operand                        */
+  int n_deps;                          /* PrimitiveOp.dependencies, chunk.py:54       */
+  const int *deps;                     /* op_uids that must complete first            */
+} pccl_op_desc;
+
+/* Builds the device-resident GraphBufferLayout (include/base/operator.h:31-38):
+ * one OperationLayoutHeader per op (:19-29) with payload and successor list,
+ * one ready queue (RingBuffer, :7-17).  Role: Engine::regOp,
+ * csrc/engine.cc:102-104.  tile_bytes = bytes of output one workgroup handles
+ * per queue entry (0 = built-in choice); it fixes required_executors_. */
+int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
+
+/* Drains the whole DAG with ONE persistent-kernel launch on `stream`; returns
+ * without waiting.  The graph re-arms itself, so it can be run again.
+ * Role: Engine::exeOp, include/engine.h:19. */
+int pccl_hip_graph_run(void *graph, void *stream);
+
+/* Waits for `stream`, then reports *completed_operator and *total_operator
+ * (operator.h:32-33); after a successful run they are equal. */
+int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
+                          unsigned int *total);
+
+/* Replaces operand addresses: every operand that lies in [old_base,
+ * old_base+nbytes) moves to new_base + the same offset.  Lets exeOp bind a
+ * new input / output tensor without rebuilding the graph. */
+int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,
+                          void *stream);
+
+/* Device address of the GraphBufferLayout and launch facts, for inspection. */
+int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
+
+int pccl_hip_graph_destroy(void *graph);
+
+/* ---- errors ---------------------------------------------------------------- */
+const char *pccl_hip_last_error(void);
+const char *pccl_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,36 @@
+// plugin_common.h -- host-side helpers shared by the translation units of
+// libpccl_hip.so: thread-local error text and HIP call checking.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "pccl_hip.h"
+
+namespace pccl_host {
+
+// Sets the calling thread's error text and returns `code` so that call sites
+// can write `return fail(PCCL_ERR_..., "...")`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// Compute units of the current device (cached per device index).
+int compute_units();
+
+struct Tuning {
+  int workgroups_per_cu;  // 0 = built-in choice
+  int nontemporal;        // -1 = built-in choice, else 0/1
+};
+Tuning tuning();
+
+}  // namespace pccl_host
+
+#define PCCL_HIP_CHECK(expr)                                                              \
+  do {                                                                                    \
+    hipError_t _e = (expr);                                                               \
+    if (_e != hipSuccess)                                                                 \
+      return ::pccl_host::fail(PCCL_ERR_HIP, "%s failed: %s (%s:%d)", #expr,              \
+                               hipGetErrorString(_e), __FILE__, __LINE__);                \
+  } while (0)

@@ -1,0 +1,88 @@
+// reduce_copy.hip -- pccl_hip_reduce_copy: argument checks, alignment analysis,
+// launch shape, dispatch to the typed kernels.
+#include <cstring>
+
+#include "reduce_copy_kernel.h"
+
+namespace pccl_dev {
+
+int launch_copy(int elem_bytes, bool aligned, bool nt, unsigned grid, hipStream_t stream,
+                const RcLaunch &p) {
+  // the dtype only selects the alignment the unaligned pack type may assume
+  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(aligned, nt, grid, stream, p);
+  return launch_nin<PCCL_BF16, OpSum, 1>(aligned, nt, grid, stream, p);
+}
+
+}  // namespace pccl_dev
+
+using namespace pccl_dev;
+using pccl_host::fail;
+
+namespace pccl_host {
+
+// Shared with the graph builder: validates one op's operands and fills the
+// launch record.  Returns PCCL_OK or an error code (text set).
+int plan_reduce_copy(int dtype, int compute, const void *const *ins, int n_in, void *const *outs,
+                     int n_out, long count, RcLaunch *out, bool *aligned) {
+  if (dtype < PCCL_F32 || dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+  if (compute < PCCL_SUM || compute > PCCL_MAX)
+    return fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute);
+  if (n_in < 1 || n_in > PCCL_MAX_INPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_in %d outside [1, 8]", n_in);
+  if (n_out < 1 || n_out > PCCL_MAX_OUTPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_out %d outside [1, 8]", n_out);
+  if (count < 0) return fail(PCCL_ERR_INVALID_ARG, "count %ld < 0", count);
+  if (!ins || !outs) return fail(PCCL_ERR_INVALID_ARG, "operand array is null");
+  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  RcLaunch p;
+  memset(&p, 0, sizeof(p));
+  for (int k = 0; k < n_in; ++k) {
+    if (!ins[k] && count) return fail(PCCL_ERR_INVALID_ARG, "input %d is null", k);
+    if ((uintptr_t)ins[k] % es) return fail(PCCL_ERR_MISALIGNED, "input %d (%p) not %d-byte aligned", k, ins[k], es);
+    p.ops.in[k] = (const char *)ins[k];
+  }
+  for (int j = 0; j < n_out; ++j) {
+    if (!outs[j] && count) return fail(PCCL_ERR_INVALID_ARG, "output %d is null", j);
+    if ((uintptr_t)outs[j] % es) return fail(PCCL_ERR_MISALIGNED, "output %d (%p) not %d-byte aligned", j, outs[j], es);
+    p.ops.out[j] = (char *)outs[j];
+  }
+  p.ops.n_out = n_out;
+  p.count = count;
+  // peel a head so that output 0 starts its body on a 16-byte boundary
+  long head = (long)((16 - ((uintptr_t)outs[0] & 15)) & 15) / es;
+  if (head > count) head = count;
+  p.head = head;
+  p.n_packs = (count - head) / (16 / es);
+  bool al = true;  // do all other streams land on 16 bytes after the same peel?
+  for (int k = 0; k < n_in; ++k) al = al && (((uintptr_t)ins[k] + (uintptr_t)head * es) & 15) == 0;
+  for (int j = 0; j < n_out; ++j) al = al && (((uintptr_t)outs[j] + (uintptr_t)head * es) & 15) == 0;
+  *aligned = al;
+  *out = p;
+  return PCCL_OK;
+}
+
+}  // namespace pccl_host
+
+extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *ins, int n_in,
+                                    void *const *outs, int n_out, long count, void *stream) {
+  pccl_host::clear_error();
+  RcLaunch p;
+  bool aligned = false;
+  int rc = pccl_host::plan_reduce_copy(dtype, compute, ins, n_in, outs, n_out, count, &p, &aligned);
+  if (rc != PCCL_OK) return rc;
+  if (count == 0) return PCCL_OK;
+  const pccl_host::Tuning t = pccl_host::tuning();
+  const int wpc = t.workgroups_per_cu > 0 ? t.workgroups_per_cu : 8;
+  const bool nt = t.nontemporal < 0 ? false : t.nontemporal != 0;
+  const long chunk = (long)kBlock * unroll_for(n_in);
+  long chunks = (p.n_packs + chunk - 1) / chunk;
+  if (chunks < 1) chunks = 1;
+  const long cap = (long)pccl_host::compute_units() * wpc;
+  const unsigned grid = (unsigned)(chunks < cap ? chunks : cap);
+  hipStream_t s = (hipStream_t)stream;
+  if (n_in == 1) return launch_copy(dtype == PCCL_F32 || dtype == PCCL_I32 ? 4 : 2, aligned, nt, grid, s, p);
+  switch (dtype) {
+    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, aligned, nt, grid, s, p);
+    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, aligned, nt, grid, s, p);
+    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, aligned, nt, grid, s, p);
+    default: return launch_typed<PCCL_F16>(compute, n_in, aligned, nt, grid, s, p);
+  }
+}

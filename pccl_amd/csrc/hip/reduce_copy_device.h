@@ -1,0 +1,254 @@
+// reduce_copy_device.h -- gfx950 device code shared by the direct-launch kernels
+// and the persistent work-queue kernel.
+//
+// One lane moves 16-byte packs (the widest packs of the reference's
+// include/plugins/cuda_executor/utils/vector_datatype.h:64-71: i32x4, f32x4,
+// f16x8, bf16x8), so a 64-lane wavefront covers 1 KiB of every stream per
+// load/store instruction.  The N-input fold replaces the switch-side
+// multimem.ld_reduce of include/plugins/cuda_executor/utils/multimem.h:12-59
+// with N explicit loads and a left fold in registers; the store to every
+// output replaces multimem.st (multimem.h:61-102).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "pccl_hip.h"
+
+namespace pccl_dev {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// Same 16 bytes, but the compiler may only assume the stated alignment.  The
+// HSA ABI runs gfx9 in unaligned access mode, so these still compile to one
+// global_load_dwordx4 / global_store_dwordx4.
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;  // 4 wavefronts, one per SIMD of a compute unit
+
+__device__ __forceinline__ float as_f32(unsigned int u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ unsigned int as_u32(float f) { return __builtin_bit_cast(unsigned int, f); }
+
+// ---- fold operators: a is the accumulator, b the next input ----------------
+struct OpSum {
+  static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+  static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) { return a + b; }
+};
+struct OpProd {
+  static __device__ __forceinline__ float f(float a, float b) { return a * b; }
+  static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) { return a * b; }
+};
+struct OpMin {
+  static __device__ __forceinline__ float f(float a, float b) { return b < a ? b : a; }
+  static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) {
+    return (int)b < (int)a ? b : a;
+  }
+};
+struct OpMax {
+  static __device__ __forceinline__ float f(float a, float b) { return a < b ? b : a; }
+  static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) {
+    return (int)a < (int)b ? b : a;
+  }
+};
+
+// ---- per-dtype: fold one 32-bit word of every input ------------------------
+template <int DT> struct Dtype;
+
+template <> struct Dtype<PCCL_F32> {
+  static constexpr int kElemBytes = 4;
+  typedef unsigned int elem_t;
+  typedef u32x4_a4 pack_unaligned;
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    float acc = as_f32(w[0]);
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::f(acc, as_f32(w[k]));
+    return as_u32(acc);
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    return word<Op, N>(e);
+  }
+};
+
+template <> struct Dtype<PCCL_I32> {
+  static constexpr int kElemBytes = 4;
+  typedef unsigned int elem_t;
+  typedef u32x4_a4 pack_unaligned;
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    unsigned int acc = w[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::i(acc, w[k]);
+    return acc;
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    return word<Op, N>(e);
+  }
+};
+
+template <> struct Dtype<PCCL_BF16> {
+  static constexpr int kElemBytes = 2;
+  typedef unsigned short elem_t;
+  typedef u32x4_a2 pack_unaligned;
+  // two bf16 per word: widen by shifting into the top half of a binary32,
+  // fold both halves in float, round once (v_cvt_pk_bf16_f32: nearest even)
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    float lo = as_f32(w[0] << 16), hi = as_f32(w[0] & 0xffff0000u);
+#pragma unroll
+    for (int k = 1; k < N; ++k) {
+      lo = Op::f(lo, as_f32(w[k] << 16));
+      hi = Op::f(hi, as_f32(w[k] & 0xffff0000u));
+    }
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    float acc = as_f32((unsigned int)e[0] << 16);
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::f(acc, as_f32((unsigned int)e[k] << 16));
+    return __builtin_bit_cast(unsigned short, (__bf16)acc);
+  }
+};
+
+template <> struct Dtype<PCCL_F16> {
+  static constexpr int kElemBytes = 2;
+  typedef unsigned short elem_t;
+  typedef u32x4_a2 pack_unaligned;
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    f32x2 acc = __builtin_convertvector(__builtin_bit_cast(f16x2, w[0]), f32x2);
+#pragma unroll
+    for (int k = 1; k < N; ++k) {
+      f32x2 x = __builtin_convertvector(__builtin_bit_cast(f16x2, w[k]), f32x2);
+      acc.x = Op::f(acc.x, x.x);
+      acc.y = Op::f(acc.y, x.y);
+    }
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(acc, f16x2));
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    float acc = (float)__builtin_bit_cast(_Float16, e[0]);
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::f(acc, (float)__builtin_bit_cast(_Float16, e[k]));
+    return __builtin_bit_cast(unsigned short, (_Float16)acc);
+  }
+};
+
+// ---- pack load / store -------------------------------------------------------
+// ALIGNED: every stream is 16-byte aligned.  Otherwise only output 0 is (the
+// host peels a head so that it is) and the others are element-aligned.
+template <class D, bool ALIGNED, bool NT>
+__device__ __forceinline__ u32x4 load_pack(const char *p) {
+  if constexpr (ALIGNED) {
+    if constexpr (NT) return __builtin_nontemporal_load((const u32x4 *)p);
+    else return *(const u32x4 *)p;
+  } else {
+    typedef typename D::pack_unaligned P;
+    if constexpr (NT) return __builtin_nontemporal_load((const P *)p);
+    else return *(const P *)p;
+  }
+}
+
+template <class D, bool ALIGNED, bool NT>
+__device__ __forceinline__ void store_pack(char *p, u32x4 v) {
+  if constexpr (ALIGNED) {
+    if constexpr (NT) __builtin_nontemporal_store(v, (u32x4 *)p);
+    else *(u32x4 *)p = v;
+  } else {
+    typedef typename D::pack_unaligned P;
+    if constexpr (NT) __builtin_nontemporal_store(v, (P *)p);
+    else *(P *)p = v;
+  }
+}
+
+template <class D, class Op, int NIN>
+__device__ __forceinline__ u32x4 fold_pack(const u32x4 (&v)[NIN]) {
+  if constexpr (NIN == 1) {
+    return v[0];  // COPY: bytes unchanged
+  } else {
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      unsigned int w[NIN];
+#pragma unroll
+      for (int k = 0; k < NIN; ++k) w[k] = v[k][j];
+      r[j] = D::template word<Op, NIN>(w);
+    }
+    return r;
+  }
+}
+
+// Operands of one reduce-copy (or of one part of it), as the kernels see them.
+struct RcOperands {
+  const char *in[PCCL_MAX_INPUTS];
+  char *out[PCCL_MAX_OUTPUTS];
+  int n_out;
+};
+
+// Body: packs [0, n_packs) of every stream, stream pointers already at the
+// first pack.  Workgroup `wg` of `n_wg` takes chunks wg, wg+n_wg, ... of
+// kBlock*UNROLL packs; inside a chunk lane t takes packs t, t+kBlock, ... so
+// every load and store instruction of a wavefront covers 1 KiB contiguously.
+template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, bool NT>
+__device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, long wg, long n_wg) {
+  constexpr long kChunk = (long)kBlock * UNROLL;
+  for (long base = wg * kChunk; base < n_packs; base += n_wg * kChunk) {
+    const long p0 = base + threadIdx.x;
+    if (base + kChunk <= n_packs) {
+      u32x4 v[UNROLL][NIN];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+        for (int k = 0; k < NIN; ++k)
+          v[u][k] = load_pack<D, ALIGNED, NT>(a.in[k] + (p0 + (long)u * kBlock) * 16);
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const u32x4 r = fold_pack<D, Op, NIN>(v[u]);
+        const long off = (p0 + (long)u * kBlock) * 16;
+        store_pack<D, true, NT>(a.out[0] + off, r);
+#pragma unroll
+        for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
+          if (j < a.n_out) store_pack<D, ALIGNED, NT>(a.out[j] + off, r);
+      }
+    } else {  // last, partial chunk: same shape, every pack guarded
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const long p = p0 + (long)u * kBlock;
+        if (p < n_packs) {
+          u32x4 v[NIN];
+#pragma unroll
+          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, NT>(a.in[k] + p * 16);
+          const u32x4 r = fold_pack<D, Op, NIN>(v);
+          store_pack<D, true, NT>(a.out[0] + p * 16, r);
+#pragma unroll
+          for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
+            if (j < a.n_out) store_pack<D, ALIGNED, NT>(a.out[j] + p * 16, r);
+        }
+      }
+    }
+  }
+}
+
+// Edge elements, one per lane of a single wavefront: elements [0, head) and
+// [tail_begin, count) of the ORIGINAL (un-advanced) streams.
+template <class D, class Op, int NIN>
+__device__ __forceinline__ void edge_elems(const RcOperands &a, long head, long tail_begin,
+                                           long count, int lane) {
+  typedef typename D::elem_t E;
+  const long n_edge = head + (count - tail_begin);
+  for (long e = lane; e < n_edge; e += kWave) {
+    const long i = e < head ? e : tail_begin + (e - head);
+    E x[NIN];
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) x[k] = ((const E *)a.in[k])[i];
+    E r;
+    if constexpr (NIN == 1) r = x[0];
+    else r = D::template elem<Op, NIN>(x);
+#pragma unroll
+    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
+      if (j < a.n_out) ((E *)a.out[j])[i] = r;
+  }
+}
+
+}  // namespace pccl_dev

@@ -1,0 +1,7 @@
+// reduce_copy_inst_i32.hip -- instantiates the i32 reduce-copy kernels
+// (4 compute ops x n_in 2..8 x aligned/unaligned x temporal/non-temporal).
+#include "reduce_copy_kernel.h"
+
+namespace pccl_dev {
+PCCL_DEFINE_LAUNCH_TYPED(PCCL_I32)
+}  // namespace pccl_dev

@@ -1,0 +1,195 @@
+"""ctypes binding of ``libpccl_hip.so`` (C ABI declared in ``include/pccl_hip.h``).
+
+Operands are raw device addresses; anything with ``data_ptr()`` (a torch tensor) is
+accepted in their place.  Every call raises :class:`PcclError` on a non-zero return
+code, carrying the library's error text.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpccl_hip.so")
+
+# codes of include/pccl_hip.h
+F32, I32, BF16, F16 = 0, 1, 2, 3
+SUM, PROD, MIN, MAX = 0, 1, 2, 3
+COPY, REDUCE, NOTIFY, GET_NOTIFIED = 0, 1, 2, 3
+DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16}
+COMPUTES = {"sum": SUM, "prod": PROD, "min": MIN, "max": MAX}
+ELEM_BYTES = {F32: 4, I32: 4, BF16: 2, F16: 2}
+
+OK = 0
+ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = -1, -2, -3, -4
+ERR_NOMEM, ERR_MISALIGNED, ERR_GRAPH = -5, -6, -7
+
+MAX_INPUTS = 8
+MAX_OUTPUTS = 8
+
+
+class PcclError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("pccl_hip error %d: %s" % (code, text))
+        self.code = code
+
+
+class OpDesc(ctypes.Structure):
+    """struct pccl_op_desc"""
+    _fields_ = [
+        ("op_uid", ctypes.c_int),
+        ("primitive", ctypes.c_ubyte),
+        ("dtype", ctypes.c_ubyte),
+        ("compute", ctypes.c_ubyte),
+        ("n_in", ctypes.c_ubyte),
+        ("n_out", ctypes.c_ubyte),
+        ("reserved", ctypes.c_ubyte * 3),
+        ("ins", ctypes.c_void_p * MAX_INPUTS),
+        ("outs", ctypes.c_void_p * MAX_OUTPUTS),
+        ("count", ctypes.c_long),
+        ("n_deps", ctypes.c_int),
+        ("deps", ctypes.POINTER(ctypes.c_int)),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    """Loads the library on first use; no fallback when it is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+        vp, ci, cl = ctypes.c_void_p, ctypes.c_int, ctypes.c_long
+        L.pccl_hip_device_count.argtypes = [ctypes.POINTER(ci)]
+        L.pccl_hip_device_info.argtypes = [ctypes.POINTER(ci), ctypes.POINTER(cl), ctypes.c_char_p, ci]
+        L.pccl_hip_alloc.argtypes = [ctypes.POINTER(vp), cl]
+        L.pccl_hip_free.argtypes = [vp]
+        L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
+        L.pccl_hip_set_tuning.argtypes = [ci, ci]
+        L.pccl_hip_graph_create.argtypes = [ctypes.POINTER(OpDesc), ci, cl, ctypes.POINTER(vp)]
+        L.pccl_hip_graph_run.argtypes = [vp, vp]
+        L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
+        L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
+        L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.pccl_hip_graph_destroy.argtypes = [vp]
+        for name in ("pccl_hip_last_error", "pccl_hip_version"):
+            getattr(L, name).restype = ctypes.c_char_p
+            getattr(L, name).argtypes = []
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != OK:
+        raise PcclError(rc, lib().pccl_hip_last_error().decode())
+
+
+def _addr(x):
+    if x is None:
+        return None
+    return int(x.data_ptr()) if hasattr(x, "data_ptr") else int(x)
+
+
+def _code(table, x):
+    return table[x] if isinstance(x, str) else int(x)
+
+
+def version():
+    return lib().pccl_hip_version().decode()
+
+
+def device_count():
+    n = ctypes.c_int(0)
+    _check(lib().pccl_hip_device_count(ctypes.byref(n)))
+    return n.value
+
+
+def device_info():
+    cus, mem = ctypes.c_int(0), ctypes.c_long(0)
+    name = ctypes.create_string_buffer(256)
+    _check(lib().pccl_hip_device_info(ctypes.byref(cus), ctypes.byref(mem), name, 256))
+    return {"compute_units": cus.value, "hbm_bytes": mem.value, "name": name.value.decode()}
+
+
+def alloc(nbytes):
+    p = ctypes.c_void_p(None)
+    _check(lib().pccl_hip_alloc(ctypes.byref(p), nbytes))
+    return p.value
+
+
+def free(ptr):
+    _check(lib().pccl_hip_free(ctypes.c_void_p(ptr)))
+
+
+def set_tuning(workgroups_per_cu=0, nontemporal=-1):
+    _check(lib().pccl_hip_set_tuning(workgroups_per_cu, nontemporal))
+
+
+def reduce_copy(dtype, compute, ins, outs, count, stream=None):
+    """One reduce-copy launch: outs[j][:count] = fold(compute, ins[0][:count], ...)."""
+    n_in, n_out = len(ins), len(outs)
+    a_in = (ctypes.c_void_p * max(n_in, 1))(*[_addr(x) for x in ins])
+    a_out = (ctypes.c_void_p * max(n_out, 1))(*[_addr(x) for x in outs])
+    _check(lib().pccl_hip_reduce_copy(_code(DTYPES, dtype), _code(COMPUTES, compute), a_in, n_in,
+                                      a_out, n_out, count, ctypes.c_void_p(_addr(stream))))
+
+
+class Graph:
+    """A DAG of COPY / REDUCE ops resident on the device, drained by one launch."""
+
+    def __init__(self, ops, tile_bytes=0):
+        """ops: list of dicts with keys dtype, compute, ins, outs, count, deps (op index list)."""
+        n = len(ops)
+        arr = (OpDesc * max(n, 1))()
+        self._keep = []
+        for i, o in enumerate(ops):
+            d = arr[i]
+            d.op_uid = i
+            n_in, n_out = len(o["ins"]), len(o["outs"])
+            d.primitive = o.get("primitive", COPY if n_in == 1 else REDUCE)
+            d.dtype = _code(DTYPES, o["dtype"])
+            d.compute = _code(COMPUTES, o.get("compute", "sum"))
+            d.n_in, d.n_out = n_in, n_out
+            for k in range(min(n_in, MAX_INPUTS)):
+                d.ins[k] = _addr(o["ins"][k])
+            for k in range(min(n_out, MAX_OUTPUTS)):
+                d.outs[k] = _addr(o["outs"][k])
+            d.count = o["count"]
+            deps = list(o.get("deps", ()))
+            d.n_deps = len(deps)
+            buf = (ctypes.c_int * max(len(deps), 1))(*deps)
+            self._keep.append(buf)
+            d.deps = ctypes.cast(buf, ctypes.POINTER(ctypes.c_int))
+        self._h = ctypes.c_void_p(None)
+        _check(lib().pccl_hip_graph_create(arr, n, tile_bytes, ctypes.byref(self._h)))
+
+    def run(self, stream=None):
+        _check(lib().pccl_hip_graph_run(self._h, ctypes.c_void_p(_addr(stream))))
+
+    def status(self, stream=None):
+        c, t = ctypes.c_uint(0), ctypes.c_uint(0)
+        _check(lib().pccl_hip_graph_status(self._h, ctypes.c_void_p(_addr(stream)), ctypes.byref(c), ctypes.byref(t)))
+        return c.value, t.value
+
+    def rebind(self, old_base, new_base, nbytes, stream=None):
+        _check(lib().pccl_hip_graph_rebind(self._h, ctypes.c_void_p(_addr(old_base)), ctypes.c_void_p(_addr(new_base)),
+                                           nbytes, ctypes.c_void_p(_addr(stream))))
+
+    def info(self):
+        lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)
+        _check(lib().pccl_hip_graph_info(self._h, ctypes.byref(lay), ctypes.byref(nt), ctypes.byref(nw)))
+        return {"device_layout": lay.value, "n_tiles": nt.value, "n_workgroups": nw.value}
+
+    def destroy(self):
+        if self._h:
+            _check(lib().pccl_hip_graph_destroy(self._h))
+            self._h = ctypes.c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

@@ -1,0 +1,140 @@
+"""GPU parity: pccl_hip_reduce_copy (through the C ABI) against the CPU checker."""
+import itertools
+
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+COUNTS_SMALL = [1, 2, 3, 7, 8, 15, 16, 17, 63, 64, 65, 127, 255, 256, 257, 1023, 1024, 1025, 4099, 65537]
+
+
+def _inputs(dtype, compute, n_in, count, seed):
+    if compute == "prod":
+        return [H.gen(dtype, count, seed, k, kind="uniform", lo=0.5, hi=2.0) if dtype != "i32"
+                else H.gen(dtype, count, seed, k, lo=-7, hi=7) for k in range(n_in)]
+    if dtype == "i32":
+        return [H.gen(dtype, count, seed, k) for k in range(n_in)]
+    return [H.gen(dtype, count, seed, k, kind="normal") for k in range(n_in)]
+
+
+def test_config1_f32_sum_2in(hip, oracle):
+    """fp32 sum of 2 inputs, 1,048,576 elements, uniform[-1,1) seed 0, aligned; bit-exact."""
+    import torch
+    n = 1 << 20
+    ins = [oracle.fill_uniform_f32(n, 0, k, -1.0, 1.0) for k in range(2)]
+    want = oracle.reduce("f32", "sum", ins)
+    (got,) = H.hip_reduce(torch, hip, "f32", "sum", ins)
+    H.assert_bits_equal(got, want, "config 1")
+    # and the checker itself agrees with numpy's IEEE add on this case
+    H.assert_bits_equal(want, ins[0] + ins[1], "oracle vs numpy")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "i32", "bf16", "f16"])
+@pytest.mark.parametrize("compute", ["sum", "prod", "min", "max"])
+def test_all_dtype_op_nin(hip, oracle, dtype, compute):
+    """Every (dtype, compute, n_in) instantiation on ragged counts, aligned buffers."""
+    import torch
+    for n_in in range(1, 9):
+        for count in (1, 5, 257, 4099, 70001):
+            ins = _inputs(dtype, compute, n_in, count, seed=100 + n_in)
+            want = oracle.reduce(dtype, compute, ins)
+            (got,) = H.hip_reduce(torch, hip, dtype, compute, ins)
+            H.assert_bits_equal(got, want, "%s %s n_in=%d count=%d" % (dtype, compute, n_in, count))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_small_counts_every_offset(hip, oracle, dtype):
+    """Counts around pack / wavefront / workgroup boundaries at every element offset of output 0."""
+    import torch
+    es = H.ELEM_BYTES[dtype]
+    for count in COUNTS_SMALL:
+        ins = _inputs(dtype, "sum", 3, count, seed=7)
+        want = oracle.reduce(dtype, "sum", ins)
+        for off in range(0, 64, es):
+            in_offs = [(off + 4 * k * es) % 64 for k in range(3)]
+            (got,) = H.hip_reduce(torch, hip, dtype, "sum", ins, in_offsets=in_offs, out_offsets=[off])
+            H.assert_bits_equal(got, want, "%s count=%d off=%d" % (dtype, count, off))
+
+
+@pytest.mark.parametrize("n_out", [1, 2, 3, 8])
+def test_multi_output(hip, oracle, n_out):
+    import torch
+    count = 100003
+    for dtype in ("bf16", "f16", "f32"):
+        ins = _inputs(dtype, "sum", 4, count, seed=11)
+        want = oracle.reduce(dtype, "sum", ins)
+        outs = H.hip_reduce(torch, hip, dtype, "sum", ins, n_out=n_out,
+                            out_offsets=[(2 * j * H.ELEM_BYTES[dtype]) % 64 for j in range(n_out)])
+        for j, got in enumerate(outs):
+            H.assert_bits_equal(got, want, "%s out %d of %d" % (dtype, j, n_out))
+
+
+def test_in_place_ring_step(hip, oracle):
+    """Output 0 is also input 1 (the in-place form a ring step uses)."""
+    import torch
+    count = 300007
+    a = H.gen("bf16", count, 21, 0)
+    b = H.gen("bf16", count, 21, 1)
+    want = oracle.reduce("bf16", "sum", [a, b])
+    d_a = H.DevBuf(torch, "bf16", count, 6, src=a)
+    d_b = H.DevBuf(torch, "bf16", count, 10, src=b)
+    d_send = H.DevBuf(torch, "bf16", count, 0)
+    hip.reduce_copy("bf16", "sum", [d_a.ptr, d_b.ptr], [d_b.ptr, d_send.ptr], count,
+                    torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    H.assert_bits_equal(d_b.download(), want, "in-place output")
+    H.assert_bits_equal(d_send.download(), want, "send buffer")
+    H.assert_bits_equal(d_a.download(), a, "input untouched")
+    assert d_b.guards_intact() and d_send.guards_intact()
+
+
+def test_special_values(hip, oracle):
+    """inf, NaN, signed zero, subnormals and rounding ties through the bf16 / f16 / f32 paths."""
+    import torch
+    f = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-40, -1e-40, 3.0e38, -3.0e38, 65504.0,
+                  65520.0, 1.00390625, 1.01171875, 5.9604645e-8, 2.98e-8, 6.1e-5, 1e-45], dtype=np.float32)
+    pairs = np.array(list(itertools.product(f, f)), dtype=np.float32)
+    for dtype in ("f32", "bf16", "f16"):
+        x = pairs[:, 0].copy() if dtype == "f32" else oracle.narrow(dtype, pairs[:, 0])
+        y = pairs[:, 1].copy() if dtype == "f32" else oracle.narrow(dtype, pairs[:, 1])
+        for compute in ("sum", "prod", "min", "max"):
+            want = oracle.reduce(dtype, compute, [x, y])
+            (got,) = H.hip_reduce(torch, hip, dtype, compute, [x, y])
+            if dtype == "f32":
+                wn, gn = np.isnan(want), np.isnan(got)
+            else:
+                wn, gn = np.isnan(oracle.widen(dtype, want)), np.isnan(oracle.widen(dtype, got))
+            assert np.array_equal(wn, gn), "%s %s: NaN positions differ" % (dtype, compute)
+            H.assert_bits_equal(np.where(wn, 0, H.bits(got)), np.where(wn, 0, H.bits(want)),
+                                "%s %s specials" % (dtype, compute))
+
+
+def test_argument_errors(hip):
+    import torch
+    t = torch.zeros(1024, dtype=torch.float32, device="cuda")
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy(9, "sum", [t], [t], 4)
+    assert e.value.code == hip.ERR_UNSUPPORTED
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", 7, [t, t], [t], 4)
+    assert e.value.code == hip.ERR_UNSUPPORTED
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", "sum", [t] * 9, [t], 4)
+    assert e.value.code == hip.ERR_INVALID_ARG
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", "sum", [t], [], 4)
+    assert e.value.code == hip.ERR_INVALID_ARG
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", "sum", [t], [t], -1)
+    assert e.value.code == hip.ERR_INVALID_ARG
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", "sum", [t.data_ptr() + 2], [t], 4)
+    assert e.value.code == hip.ERR_MISALIGNED
+    with pytest.raises(hip.PcclError) as e:
+        hip.reduce_copy("f32", "sum", [0], [t], 4)
+    assert e.value.code == hip.ERR_INVALID_ARG
+    hip.reduce_copy("f32", "sum", [t], [t], 0)  # empty op is a no-op
+    torch.cuda.synchronize()
