@@ -136,6 +136,12 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
 /* Device address of the GraphBufferLayout and launch facts, for inspection. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 
+/* Bounds every wait inside the drain kernel to `polls` polls of a queue slot
+ * (default about 2 million, a few seconds).  When a wait gives up the kernel
+ * raises its abort flag, every workgroup leaves, and pccl_hip_graph_status
+ * returns PCCL_ERR_GRAPH after restoring the graph's pristine state. */
+int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls);
+
 int pccl_hip_graph_destroy(void *graph);
 
 /* ---- errors ---------------------------------------------------------------- */

@@ -1,0 +1,70 @@
+"""Test-side builders of op DAGs (ring all-reduce over virtual ranks resident on one GPU).
+
+An op is a dict: dtype, compute, ins, outs, count, deps.  Operands are named symbolically as
+(buffer, rank, element_offset); `materialise` turns them into addresses (device) or numpy views
+(CPU checker).  The ring follows the textbook schedule: at reduce-scatter step s rank r folds
+the partial sum of chunk (r - s) mod W coming from rank r-1 with its own copy of that chunk; at
+all-gather step s it copies chunk (r - s + 1) mod W from rank r-1.  An op of (rank r, step l)
+depends on the op of (rank r-1, step l-1), which also covers every write-after-read hazard
+because going back W-1 steps along that rule reaches the reader of the overwritten chunk.
+"""
+import math
+
+
+def ring_allreduce_ops(world, slice_sizes, dtype="bf16", compute="sum", base_elem=0):
+    """slice_sizes[k] = elements per chunk of independent all-reduce k.
+    Returns (ops, elems_per_rank).  Buffers: "in" (per-rank input), "out" (per-rank output)."""
+    ops = []
+    off = base_elem
+    for size in slice_sizes:
+        prev = {}
+        for step in range(1, world):  # reduce-scatter
+            cur = {}
+            for r in range(world):
+                c = (r - step) % world
+                src_rank = (r - 1) % world
+                incoming = ("in" if step == 1 else "out", src_rank, off + c * size)
+                local = ("in", r, off + c * size)
+                deps = [prev[src_rank]] if step > 1 else []
+                ops.append(dict(dtype=dtype, compute=compute, ins=[incoming, local],
+                                outs=[("out", r, off + c * size)], count=size, deps=deps))
+                cur[r] = len(ops) - 1
+            prev = cur
+        for step in range(1, world):  # all-gather
+            cur = {}
+            for r in range(world):
+                c = (r - step + 1) % world
+                src_rank = (r - 1) % world
+                ops.append(dict(dtype=dtype, compute=compute, ins=[("out", src_rank, off + c * size)],
+                                outs=[("out", r, off + c * size)], count=size, deps=[prev[src_rank]]))
+                cur[r] = len(ops) - 1
+            prev = cur
+        off += world * size
+    return ops, off
+
+
+def log_uniform_sizes(orc, n, seed, stream, lo_bytes, hi_bytes, elem_bytes):
+    """n sizes in elements, log-uniform in [lo_bytes, hi_bytes], rounded down to whole elements."""
+    out = []
+    for i in range(n):
+        u = (orc.rng_u64(seed, stream, i) >> 11) / float(1 << 53)
+        b = lo_bytes * math.exp(u * math.log(hi_bytes / lo_bytes))
+        out.append(max(1, int(b) // elem_bytes))
+    return out
+
+
+def materialise(ops, resolve):
+    """resolve(buffer, rank, elem_offset, count) -> address or numpy view."""
+    done = []
+    for o in ops:
+        d = dict(o)
+        d["ins"] = [resolve(b, r, e, o["count"]) for (b, r, e) in o["ins"]]
+        d["outs"] = [resolve(b, r, e, o["count"]) for (b, r, e) in o["outs"]]
+        done.append(d)
+    return done
+
+
+def edges_of(ops):
+    """(src, dst) pairs in the order CollectiveIR.create_operation adds them
+    (reference pccl/lang/chunk.py:104-106: for each op, one edge per dependency)."""
+    return [(d, i) for i, o in enumerate(ops) for d in o["deps"]]

@@ -1,0 +1,221 @@
+"""GPU parity of the op-batching path: DAGs drained by one persistent kernel (C ABI
+pccl_hip_graph_*) against the CPU checker executing the same ops in topological order."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import helpers as H
+import schedules as S
+
+pytestmark = pytest.mark.gpu
+
+
+def _stream(torch):
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _run_and_check(torch, hip, g, n_ops):
+    g.run(_stream(torch))
+    done, total = g.status(_stream(torch))
+    assert (done, total) == (n_ops, n_ops)
+
+
+def test_single_op_graph(hip, oracle):
+    import torch
+    for dtype, count in (("bf16", 32768), ("f32", 70001), ("i32", 5), ("f16", 1 << 20)):
+        ins = [H.gen(dtype, count, 31, k) for k in range(2)]
+        want = oracle.reduce(dtype, "sum", ins)
+        d_in = [H.DevBuf(torch, dtype, count, 0, src=a) for a in ins]
+        d_out = H.DevBuf(torch, dtype, count, 0)
+        g = hip.Graph([dict(dtype=dtype, compute="sum", ins=[b.ptr for b in d_in], outs=[d_out.ptr], count=count)])
+        _run_and_check(torch, hip, g, 1)
+        H.assert_bits_equal(d_out.download(), want, "single-op graph %s" % dtype)
+        assert d_out.guards_intact()
+        g.destroy()
+
+
+def test_dependent_chain_in_place(hip, oracle):
+    """t = a+b; u = t+c; t = u+t (in place); v = copy(t) -- wrong order gives wrong bits."""
+    import torch
+    count = 200003
+    a, b, c = (H.gen("f32", count, 41, k, kind="uniform", lo=-1e3, hi=1e3) for k in range(3))
+    t = oracle.reduce("f32", "sum", [a, b])
+    u = oracle.reduce("f32", "sum", [t, c])
+    t2 = oracle.reduce("f32", "sum", [u, t])
+    da, db, dc = (H.DevBuf(torch, "f32", count, 4 * k, src=x) for k, x in enumerate((a, b, c)))
+    dt, du, dv = (H.DevBuf(torch, "f32", count, 8 * k) for k in range(3))
+    ops = [
+        dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+        dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0]),
+        dict(dtype="f32", compute="sum", ins=[du.ptr, dt.ptr], outs=[dt.ptr], count=count, deps=[1]),
+        dict(dtype="f32", compute="sum", ins=[dt.ptr], outs=[dv.ptr], count=count, deps=[2]),
+    ]
+    g = hip.Graph(ops, tile_bytes=16384)
+    assert g.info()["n_tiles"] > 4
+    _run_and_check(torch, hip, g, 4)
+    H.assert_bits_equal(du.download(), u, "u")
+    H.assert_bits_equal(dt.download(), t2, "t (in place)")
+    H.assert_bits_equal(dv.download(), t2, "v (copy)")
+    g.destroy()
+
+
+def _ring_case(torch, hip, oracle, world, sizes, dtype, seed, offsets=(0, 0), tile_bytes=0, runs=1):
+    es = H.ELEM_BYTES[dtype]
+    ops, per_rank = S.ring_allreduce_ops(world, sizes, dtype=dtype)
+    host_in = [H.gen(dtype, per_rank, seed, r, sigma=1.0) for r in range(world)]
+    host_out = [np.zeros(per_rank, dtype=H.STORAGE[dtype]) for _ in range(world)]
+    # CPU checker: same ops, order restated from the reference's topological_sort
+    order = oracle.topo_sort(len(ops), S.edges_of(ops))
+    assert order is not None
+    bufs = {"in": host_in, "out": host_out}
+    oracle.run_ops(S.materialise(ops, lambda b, r, e, n: bufs[b][r][e:e + n]), order)
+    # every rank ends with the same bytes: the all-reduce invariant
+    for r in range(1, world):
+        H.assert_bits_equal(host_out[r], host_out[0], "oracle: rank %d vs rank 0" % r)
+    d_in = [H.DevBuf(torch, dtype, per_rank, offsets[0], src=host_in[r]) for r in range(world)]
+    d_out = [H.DevBuf(torch, dtype, per_rank, offsets[1]) for r in range(world)]
+    dev = {"in": d_in, "out": d_out}
+    g = hip.Graph(S.materialise(ops, lambda b, r, e, n: dev[b][r].ptr + e * es), tile_bytes=tile_bytes)
+    for it in range(runs):
+        if it:
+            for b in d_out:
+                b.view().fill_(0xFF)
+        _run_and_check(torch, hip, g, len(ops))
+        for r in range(world):
+            H.assert_bits_equal(d_out[r].download(), host_out[r], "run %d rank %d" % (it, r))
+            assert d_out[r].guards_intact()
+    info = g.info()
+    g.destroy()
+    return info
+
+
+def test_ring_allreduce_small(hip, oracle):
+    import torch
+    _ring_case(torch, hip, oracle, 8, [1000, 37, 4096], "bf16", seed=4)
+
+
+def test_ring_allreduce_world_sizes(hip, oracle):
+    import torch
+    for world in (2, 3, 5, 8):
+        _ring_case(torch, hip, oracle, world, [2049, 64], "f32", seed=5)
+
+
+def test_ring_allreduce_unaligned_and_rerun(hip, oracle):
+    """Operands 6 and 10 bytes off 16-byte alignment; graph run three times (self re-arming)."""
+    import torch
+    _ring_case(torch, hip, oracle, 8, [5001, 12345, 3], "bf16", seed=6, offsets=(6, 10), tile_bytes=4096, runs=3)
+
+
+def test_config5_shape_reduced(hip, oracle):
+    """The 4096-op construction at reduced byte sizes: 36 ring slices x 112 ops + 64 copies."""
+    import torch
+    sizes = S.log_uniform_sizes(oracle, 36, 4, 0, 512, 16384, 2)
+    world = 8
+    ops, per_rank = S.ring_allreduce_ops(world, sizes, dtype="bf16")
+    extra = S.log_uniform_sizes(oracle, 64, 4, 1, 512, 16384, 2)
+    off = per_rank
+    for i, n in enumerate(extra):  # 64 independent level-1 copies, 8 per rank
+        r = i % world
+        ops.append(dict(dtype="bf16", compute="sum", ins=[("in", r, off)], outs=[("out", r, off)], count=n, deps=[]))
+        if r == world - 1:
+            off += max(extra[i - 7:i + 1])
+    per_rank = off + max(extra)
+    assert len(ops) == 4096
+    host_in = [H.gen("bf16", per_rank, 4, 10 + r, sigma=1.0) for r in range(world)]
+    host_out = [np.zeros(per_rank, dtype=np.uint16) for _ in range(world)]
+    bufs = {"in": host_in, "out": host_out}
+    order = oracle.topo_sort(len(ops), S.edges_of(ops))
+    oracle.run_ops(S.materialise(ops, lambda b, r, e, n: bufs[b][r][e:e + n]), order)
+    d_in = [H.DevBuf(torch, "bf16", per_rank, 0, src=host_in[r]) for r in range(world)]
+    d_out = [H.DevBuf(torch, "bf16", per_rank, 0, fill=0) for r in range(world)]
+    dev = {"in": d_in, "out": d_out}
+    g = hip.Graph(S.materialise(ops, lambda b, r, e, n: dev[b][r].ptr + e * 2))
+    for it in range(2):
+        _run_and_check(torch, hip, g, 4096)
+        for r in range(world):
+            H.assert_bits_equal(d_out[r].download(), host_out[r], "run %d rank %d" % (it, r))
+    g.destroy()
+
+
+def test_rebind(hip, oracle):
+    import torch
+    count = 40000
+    a, b, a2 = (H.gen("bf16", count, 51, k) for k in range(3))
+    da, db, da2 = (H.DevBuf(torch, "bf16", count, 0, src=x) for x in (a, b, a2))
+    do, do2 = H.DevBuf(torch, "bf16", count, 0), H.DevBuf(torch, "bf16", count, 0)
+    g = hip.Graph([dict(dtype="bf16", compute="sum", ins=[da.ptr, db.ptr], outs=[do.ptr], count=count)])
+    _run_and_check(torch, hip, g, 1)
+    H.assert_bits_equal(do.download(), oracle.reduce("bf16", "sum", [a, b]), "before rebind")
+    g.rebind(da.ptr, da2.ptr, da.nbytes, _stream(torch))
+    g.rebind(do.ptr, do2.ptr, do.nbytes, _stream(torch))
+    _run_and_check(torch, hip, g, 1)
+    H.assert_bits_equal(do2.download(), oracle.reduce("bf16", "sum", [a2, b]), "after rebind")
+    g.destroy()
+
+
+def test_graph_errors(hip):
+    import torch
+    t = torch.zeros(4096, dtype=torch.float32, device="cuda")
+    op = dict(dtype="f32", compute="sum", ins=[t, t], outs=[t], count=16, deps=[])
+    with pytest.raises(hip.PcclError) as e:  # cycle
+        hip.Graph([dict(op, deps=[1]), dict(op, deps=[0])])
+    assert e.value.code == hip.ERR_GRAPH
+    with pytest.raises(hip.PcclError) as e:  # dependency outside the graph
+        hip.Graph([dict(op, deps=[5])])
+    assert e.value.code == hip.ERR_GRAPH
+    with pytest.raises(hip.PcclError) as e:  # self dependency
+        hip.Graph([dict(op, deps=[0])])
+    assert e.value.code == hip.ERR_GRAPH
+    with pytest.raises(hip.PcclError) as e:  # two (dtype, compute) pairs
+        hip.Graph([op, dict(op, compute="max")])
+    assert e.value.code == hip.ERR_UNSUPPORTED
+    with pytest.raises(hip.PcclError) as e:  # NOTIFY is not executable here
+        hip.Graph([dict(op, primitive=hip.NOTIFY)])
+    assert e.value.code == hip.ERR_UNSUPPORTED
+    with pytest.raises(hip.PcclError) as e:
+        hip.Graph([dict(op, ins=[t.data_ptr() + 1, t])])
+    assert e.value.code == hip.ERR_MISALIGNED
+    g = hip.Graph([])  # empty graph runs and reports 0 of 0
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (0, 0)
+    g.destroy()
+
+
+def test_bounded_wait_aborts_cleanly(hip, oracle):
+    """A dependency that is never satisfied (forced from the host by inflating one op's
+    pre_dependencies_ on the device) must end in PCCL_ERR_GRAPH, not in a hang, and the
+    graph must work again afterwards."""
+    import torch
+    count = 1024
+    a, b = H.gen("f32", count, 61, 0), H.gen("f32", count, 61, 1)
+    da, db = H.DevBuf(torch, "f32", count, 0, src=a), H.DevBuf(torch, "f32", count, 0, src=b)
+    dt, du = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[dt.ptr, db.ptr], outs=[du.ptr], count=count, deps=[0])]
+    g = hip.Graph(ops)
+    L = hip.lib()
+    L.pccl_hip_graph_set_spin_limit.argtypes = [ctypes.c_void_p, ctypes.c_uint]
+    assert L.pccl_hip_graph_set_spin_limit(g._h, 256) == 0
+    # GraphBufferLayout.operators (offset 16) -> headers; op 1's byte 12 is pre_dependencies_
+    lay = g.info()["device_layout"]
+    host = torch.empty(48, dtype=torch.uint8)
+    import ctypes as C
+    hipmemcpy = C.CDLL("libamdhip64.so").hipMemcpy
+    hipmemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    assert hipmemcpy(host.data_ptr(), lay, 48, 2) == 0
+    operators = int(host.numpy()[16:24].view(np.uint64)[0])
+    ptrs = torch.empty(16, dtype=torch.uint8)
+    assert hipmemcpy(ptrs.data_ptr(), operators, 16, 2) == 0
+    hdr1 = int(ptrs.numpy()[8:16].view(np.uint64)[0])
+    two = torch.tensor([2], dtype=torch.uint8)
+    assert hipmemcpy(hdr1 + 12, two.data_ptr(), 1, 1) == 0  # needs 2 predecessors, has 1
+    g.run(_stream(torch))
+    with pytest.raises(hip.PcclError) as e:
+        g.status(_stream(torch))
+    assert e.value.code == hip.ERR_GRAPH
+    # status restored the pristine graph: it runs correctly now
+    assert L.pccl_hip_graph_set_spin_limit(g._h, 1 << 21) == 0
+    _run_and_check(torch, hip, g, 2)
+    H.assert_bits_equal(du.download(), oracle.reduce("f32", "sum", [oracle.reduce("f32", "sum", [a, b]), b]), "after reset")
+    g.destroy()
