@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the reduce-copy hot path on one MI355X.
+
+A step is one pass of the hot path over one batch: one pccl_hip_reduce_copy launch of the
+headline workload (bf16, 8 inputs -> 1 output, 256 MiB per buffer).  Inputs are resident in
+HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# scaled by what the same counters read for a plain copy of known size (figures and commands in
+# profiles/reduce_copy_bf16_8in_256MiB.pmc.txt).  None until that profile has been taken.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def event_times_us(torch, fn, iters, warm):
+    """Per-launch durations from HIP events recorded on the stream fn launches on."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+
+
+def stats(ts):
+    return {"min_us": round(ts[0], 2), "median_us": round(ts[len(ts) // 2], 2), "mean_us": round(sum(ts) / len(ts), 2)}
+
+
+def gbps(nbytes, us):
+    return round(nbytes / us / 1e3, 1)
+
+
+def randn(torch, n, kind, sigma=1.0):
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[kind]
+    # generated in slices to bound the fp32 temporary
+    out = torch.empty(n, dtype=dt, device="cuda")
+    step = 1 << 26
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        out[lo:hi] = (torch.randn(hi - lo, device="cuda") * sigma).to(dt)
+    return out
+
+
+def cpu_baseline(count_sample):
+    """The CPU checker's reduce-copy (a port: the reference has no CPU reduce code) on a
+    bounded sample of the headline workload, timed on this box's host cores."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import pccl_oracle as orc
+    cores = min(16, os.cpu_count() or 1)
+    ins = [np.random.default_rng(k).integers(0x3c00, 0x4000, size=count_sample, dtype=np.uint16) for k in range(8)]
+    out = np.empty(count_sample, dtype=np.uint16)
+    nbytes = 9 * count_sample * 2
+    best = {}
+    for threads in (1, cores):
+        ts = []
+        reps = 2 if threads == 1 else 5
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            orc.reduce_copy("bf16", "sum", ins, [out], count_sample, nthreads=threads)
+            ts.append(time.perf_counter() - t0)
+        best[threads] = nbytes / min(ts) / 1e9
+    return {"value": round(best[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "bf16 8->1 sum, %d elements per buffer (1/%d of the headline buffers), best of 5; "
+                      "single thread: %.2f GB/s" % (count_sample, (1 << 27) // count_sample, best[1]),
+            "host_cpus_visible": os.cpu_count()}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (peers are HBM buffers on the "
+              "same device); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from pccl_amd import hip
+    from pccl_amd import lang
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    hip.lib()
+    info = hip.device_info()
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.manual_seed(2)
+
+    # ---- headline: bf16 8 -> 1, 256 MiB per buffer --------------------------------------
+    count = 1 << 27
+    ins = [randn(torch, count, "bf16") for _ in range(8)]
+    out = torch.empty(count, dtype=torch.bfloat16, device="cuda")
+    step_bytes = 9 * count * 2
+
+    def step():
+        hip.reduce_copy("bf16", "sum", ins, [out], count, stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = step_bytes * args.steps / wall / 1e9
+
+    ts = event_times_us(torch, step, max(20, min(args.steps, 100)), 3)
+    mean_us = sum(ts) / len(ts)
+    achieved = step_bytes / mean_us / 1e3
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                "kernel": "reduce_copy_kernel<bf16, sum, n_in=8>", "algorithmic_bytes_per_launch": step_bytes,
+                "launch_us": stats(ts)}
+
+    # quick self-check of the timed buffers against torch's fp32 accumulate (same fold order)
+    ref = ins[0][:1 << 20].float()
+    for k in range(1, 8):
+        ref = ref + ins[k][:1 << 20].float()
+    assert torch.equal(ref.to(torch.bfloat16), out[:1 << 20]), "headline output differs from fp32-accumulated fold"
+
+    extras = {}
+    if not args.no_extras:
+        # ---- 128 MiB variants: bf16 8->1 and fp16 8->2 ------------------------------------
+        c3 = 1 << 26
+        t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x[:c3] for x in ins], [out[:c3]], c3, stream), 30, 5)
+        extras["nvls_bf16_8in_1out_128MiB"] = dict(stats(t), GBps_median=gbps(9 * c3 * 2, t[len(t) // 2]))
+        ins16 = [randn(torch, c3, "f16") for _ in range(8)]
+        o16 = [torch.empty(c3, dtype=torch.float16, device="cuda") for _ in range(2)]
+        t = event_times_us(torch, lambda: hip.reduce_copy("f16", "sum", ins16, o16, c3, stream), 30, 5)
+        extras["nvls_f16_8in_2out_128MiB"] = dict(stats(t), GBps_median=gbps(10 * c3 * 2, t[len(t) // 2]))
+        assert torch.equal(o16[0], o16[1])
+        del ins16, o16
+
+        # ---- ring all-reduce, one rank's share at world 8: 7 reduce-copy + 7 copy steps ----
+        W, ce = 8, 1 << 24  # 32 MiB chunks of a 256 MiB gradient
+        grad = randn(torch, W * ce, "bf16", 1e-2)
+        peers = [randn(torch, ce, "bf16", 1e-2) for _ in range(W - 1)]
+        result = torch.empty(W * ce, dtype=torch.bfloat16, device="cuda")
+        send = torch.empty(ce, dtype=torch.bfloat16, device="cuda")
+
+        def ring():
+            for s in range(W - 1):  # local chunk + incoming -> output chunk + send buffer
+                c = (W - 1 - s) % W
+                hip.reduce_copy("bf16", "sum", [peers[s], grad[c * ce:(c + 1) * ce]],
+                                [result[c * ce:(c + 1) * ce], send], ce, stream)
+            for s in range(W - 1):  # incoming reduced chunk -> output chunk
+                c = (W - s) % W
+                hip.reduce_copy("bf16", "sum", [peers[s]], [result[c * ce:(c + 1) * ce]], ce, stream)
+
+        t = event_times_us(torch, ring, 20, 3)
+        ring_bytes = 7 * 4 * ce * 2 + 7 * 2 * ce * 2
+        tr = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[0], grad[:ce]], [result[:ce], send], ce, stream), 50, 5)
+        tc = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[1]], [result[ce:2 * ce]], ce, stream), 50, 5)
+        extras["ring_allreduce_rank_share"] = {
+            "all_14_steps": dict(stats(t), GBps_median=gbps(ring_bytes, t[len(t) // 2])),
+            "reduce_step_2in_2out_32MiB": dict(stats(tr), GBps_median=gbps(4 * ce * 2, tr[len(tr) // 2])),
+            "copy_step_1in_1out_32MiB": dict(stats(tc), GBps_median=gbps(2 * ce * 2, tc[len(tc) // 2])),
+            "note": "single steps re-touch 128/64 MiB and are helped by the 256 MB Infinity Cache; "
+                    "the 14-step figure walks 1.3 GiB of distinct data"}
+        del grad, peers, result, send
+
+        # ---- plumbing config: f32 2 -> 1, 4 MiB ---------------------------------------------
+        a, b = randn(torch, 1 << 20, "f32"), randn(torch, 1 << 20, "f32")
+        o = torch.empty_like(a)
+        t = event_times_us(torch, lambda: hip.reduce_copy("f32", "sum", [a, b], [o], 1 << 20, stream), 100, 10)
+        assert torch.equal(o, a + b)
+        extras["f32_2in_1out_4MiB"] = stats(t)
+
+        # ---- small ops: 64 KiB direct launch and through the queue --------------------------
+        n64 = 32768
+        x, y = randn(torch, n64, "bf16"), randn(torch, n64, "bf16")
+        z = torch.empty_like(x)
+        t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x, y], [z], n64, stream), 200, 20)
+        extras["op_64KiB_direct_launch"] = stats(t)
+        g1 = hip.Graph([dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)])
+        t = event_times_us(torch, lambda: g1.run(stream), 200, 20)
+        extras["op_64KiB_via_queue"] = stats(t)
+        g1.destroy()
+
+        # ---- the 4096-op small-message schedule: one persistent launch ----------------------
+        ir, per_rank = lang.small_message_allreduce()
+        low = ir.lower()
+        bufs = {"in": [randn(torch, per_rank, "bf16") for _ in range(8)],
+                "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
+        bound = lang.bind(low, lambda b, r, e: bufs[b][r].data_ptr() + 2 * e)
+        sched_bytes = sum((len(o["ins"]) + len(o["outs"])) * o["count"] * 2 for o in low)
+        g = hip.Graph(bound)
+        t = event_times_us(torch, lambda: g.run(stream), 30, 5)
+        done, total = g.status(stream)
+        assert done == total == len(low)
+        for r in range(1, 8):  # all-reduce invariant on the ring part
+            assert torch.equal(bufs["out"][r][:per_rank // 2], bufs["out"][0][:per_rank // 2])
+        ginfo = g.info()
+        med = t[len(t) // 2]
+
+        def individually():
+            for o in bound:
+                hip.reduce_copy("bf16", "sum", o["ins"], o["outs"], o["count"], stream)
+
+        t2 = event_times_us(torch, individually, 5, 1)
+        extras["schedule_4096_ops"] = {
+            "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med)),
+            "as_4096_launches": dict(stats(t2), us_per_op=round(t2[len(t2) // 2] / len(low), 4)),
+            "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
+            "algorithmic_bytes": sched_bytes}
+        g.destroy()
+
+    result = {
+        "metric": "reduce_copy_hbm_bandwidth", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 sum of 8 inputs -> 1 output, 134217728 elements (256 MiB) per buffer, "
+                               "N(0,1) from torch seed 2, fp32 accumulate, one launch per step",
+                   "n_in": 8, "n_out": 1, "count": count, "bytes_per_step": step_bytes},
+        "pct_of_peak_hbm": round(100.0 * value / PEAK_HBM_GBPS, 2),
+        "roofline": roofline,
+        "device": info,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(1 << 24)
+    if extras:
+        result["extras"] = extras
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

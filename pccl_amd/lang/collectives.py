@@ -1,0 +1,109 @@
+"""Schedule emitters: collectives written against :class:`CollectiveIR`.
+
+The reference reserves ``pccl/lang/operator.py`` and ``example/collective/allreduce.py`` for
+this and leaves both empty, so the schedules are this build's.
+"""
+import math
+
+from .ir import Chunk, CollectiveIR, Device, DeviceType, Link, PrimitiveOpType
+
+
+def _ring_ir(name, world, dtype, compute):
+    ir = CollectiveIR(name, dtype=dtype, compute=compute)
+    for r in range(world):
+        ir.add_device(Device(r, DeviceType.ROCM, memory_bandwidth=8.0e12, compute_capability=9.5))
+    for r in range(world):
+        if world > 1 and (world > 2 or r == 0):
+            ir.add_link(Link(r, (r + 1) % world, bandwidth=153.0e9, latency=1.0e-6))
+    return ir
+
+
+def ring_allreduce(world, chunk_elems, dtype="bf16", compute="sum", name="ring_allreduce", ir=None, base=0):
+    """Out-of-place ring all-reduce of `world` chunks of `chunk_elems` elements per rank.
+
+    Buffers: "in" (each rank's contribution) and "out" (each rank's result), chunk c of a rank
+    at element offset base + c*chunk_elems.  Reduce-scatter step s (1..W-1): rank r folds the
+    partial sum of chunk (r-s) mod W held by rank r-1 with its own contribution.  All-gather
+    step s: rank r copies chunk (r-s+1) mod W from rank r-1.  The op of (rank r, level l)
+    depends on the op of (rank r-1, level l-1); following that rule back W-1 levels reaches the
+    last reader of every location an op overwrites, so no other edges are needed.
+    Returns (ir, elements_per_rank_used)."""
+    W = world
+    ir = ir or _ring_ir(name, W, dtype, compute)
+    prev = {}
+    for step in range(1, W):
+        cur = {}
+        for r in range(W):
+            c, p = (r - step) % W, (r - 1) % W
+            off = base + c * chunk_elems
+            incoming = ("in" if step == 1 else "out", p, off)
+            ranks = {(c + i) % W for i in range(step + 1)}
+            cur[r] = ir.create_operation(
+                PrimitiveOpType.REDUCE,
+                src_chunk=Chunk(ranks - {r}, p, chunk_elems, off), tgt_chunk=Chunk(ranks, r, chunk_elems, off),
+                src_device=p, tgt_device=r, dependencies=[prev[p]] if step > 1 else [],
+                metadata={"srcs": [incoming, ("in", r, off)], "tgt_buffer": "out", "level": step})
+        prev = cur
+    full = set(range(W))
+    for step in range(1, W):
+        cur = {}
+        for r in range(W):
+            c, p = (r - step + 1) % W, (r - 1) % W
+            off = base + c * chunk_elems
+            cur[r] = ir.create_operation(
+                PrimitiveOpType.COPY,
+                src_chunk=Chunk(full, p, chunk_elems, off), tgt_chunk=Chunk(full, r, chunk_elems, off),
+                src_device=p, tgt_device=r, dependencies=[prev[p]],
+                metadata={"src_buffer": "out", "tgt_buffer": "out", "level": W - 1 + step})
+        prev = cur
+    return ir, base + W * chunk_elems
+
+
+def log_uniform_sizes(n, seed, lo_bytes, hi_bytes, elem_bytes):
+    """n sizes in elements, log-uniform in [lo_bytes, hi_bytes] (splitmix64 stream of `seed`)."""
+    def mix(z):
+        z &= (1 << 64) - 1
+        z = ((z ^ (z >> 30)) * 0xbf58476d1ce4e5b9) & ((1 << 64) - 1)
+        z = ((z ^ (z >> 27)) * 0x94d049bb133111eb) & ((1 << 64) - 1)
+        return z ^ (z >> 31)
+    sizes = []
+    for i in range(n):
+        u = (mix(seed * 0x9e3779b97f4a7c15 + (i + 1) * 0x9e3779b97f4a7c15) >> 11) / float(1 << 53)
+        sizes.append(max(1, int(lo_bytes * math.exp(u * math.log(hi_bytes / lo_bytes))) // elem_bytes))
+    return sizes
+
+
+def small_message_allreduce(world=8, n_slices=36, n_extra=64, seed=4, lo_bytes=8 << 10, hi_bytes=256 << 10,
+                            dtype="bf16", compute="sum"):
+    """The small-message program: `n_slices` independent ring all-reduces whose chunk sizes
+    are log-uniform in [lo_bytes, hi_bytes] (one draw per slice: the 2*(W-1)*W ops of a slice
+    share it), plus `n_extra` independent level-1 COPY ops in -> out with sizes drawn the same
+    way.  world=8, 36 slices, 64 extras: 36*112 + 64 = 4096 ops, DAG depth 14.
+    Returns (ir, elements_per_rank)."""
+    es = 4 if dtype in ("f32", "i32") else 2
+    sizes = log_uniform_sizes(n_slices + n_extra, seed, lo_bytes, hi_bytes, es)
+    ir = _ring_ir("small_message_allreduce", world, dtype, compute)
+    base = 0
+    for k in range(n_slices):
+        ir, base = ring_allreduce(world, sizes[k], dtype, compute, ir=ir, base=base)
+    # extras: rank i % W copies a private region; regions of one round share an offset
+    for i in range(n_extra):
+        r, n = i % world, sizes[n_slices + i]
+        full = {r}
+        ir.create_operation(PrimitiveOpType.COPY, src_chunk=Chunk(full, r, n, base), tgt_chunk=Chunk(full, r, n, base),
+                            src_device=r, tgt_device=r, dependencies=[],
+                            metadata={"src_buffer": "in", "tgt_buffer": "out", "level": 1})
+        if r == world - 1 or i == n_extra - 1:
+            base += max(sizes[n_slices + i - r:n_slices + i + 1])
+    return ir, base
+
+
+def bind(lowered, resolve):
+    """Replaces symbolic operands: resolve(buffer, device, element_offset) -> address."""
+    out = []
+    for o in lowered:
+        d = dict(o)
+        d["ins"] = [resolve(*x) for x in o["ins"]]
+        d["outs"] = [resolve(*x) for x in o["outs"]]
+        out.append(d)
+    return out
