@@ -77,7 +77,7 @@ __device__ __forceinline__ void run_part_body(const RcOperands &a, long head, lo
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < a.n_out) body.out[j] = a.out[j] + head * D::kElemBytes;
     constexpr int kUnroll = NIN >= 4 ? 1 : NIN >= 2 ? 2 : 4;
-    body_packs<D, Op, NIN, kUnroll, ALIGNED, false>(body, n_packs, 0, 1);
+    body_packs<D, Op, NIN, kUnroll, ALIGNED, false, false>(body, n_packs, 0, 1);
   }
   if (threadIdx.x >= kBlock - kWave)
     edge_elems<D, Op, NIN>(a, head, head + n_packs * kEpp, count, (int)threadIdx.x - (kBlock - kWave));

@@ -1,16 +1,17 @@
 // reduce_copy.hip -- pccl_hip_reduce_copy: argument checks, alignment analysis,
 // launch shape, dispatch to the typed kernels.
+#include <algorithm>
 #include <cstring>
 
 #include "reduce_copy_kernel.h"
 
 namespace pccl_dev {
 
-int launch_copy(int elem_bytes, bool aligned, bool nt, unsigned grid, hipStream_t stream,
+int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream,
                 const RcLaunch &p) {
   // the dtype only selects the alignment the unaligned pack type may assume
-  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(aligned, nt, grid, stream, p);
-  return launch_nin<PCCL_BF16, OpSum, 1>(aligned, nt, grid, stream, p);
+  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, nt, grid, stream, p);
+  return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, stream, p);
 }
 
 }  // namespace pccl_dev
@@ -70,19 +71,26 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   if (rc != PCCL_OK) return rc;
   if (count == 0) return PCCL_OK;
   const pccl_host::Tuning t = pccl_host::tuning();
-  const int wpc = t.workgroups_per_cu > 0 ? t.workgroups_per_cu : 8;
-  const bool nt = t.nontemporal < 0 ? false : t.nontemporal != 0;
-  const long chunk = (long)kBlock * unroll_for(n_in);
+  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  // Streams that together exceed what the 256 MB Infinity Cache can hold are
+  // streamed (non-temporal) one pack per lane; smaller ones stay cacheable.
+  const long total_bytes = (long)(n_in + n_out) * count * es;
+  const bool big = total_bytes > (192l << 20);
+  const bool nt = t.nontemporal < 0 ? big : t.nontemporal != 0;
+  const int unroll = big ? 1 : small_unroll_for(n_in);
+  const long chunk = (long)kBlock * unroll;
   long chunks = (p.n_packs + chunk - 1) / chunk;
   if (chunks < 1) chunks = 1;
-  const long cap = (long)pccl_host::compute_units() * wpc;
-  const unsigned grid = (unsigned)(chunks < cap ? chunks : cap);
+  // default: one workgroup per chunk; a tuning run may cap it to a persistent grid
+  long grid = chunks;
+  if (t.workgroups_per_cu > 0) grid = std::min<long>(chunks, (long)pccl_host::compute_units() * t.workgroups_per_cu);
+  if (grid > 0x7fffffffl) grid = 0x7fffffffl;  // the kernel's chunk loop covers the rest
   hipStream_t s = (hipStream_t)stream;
-  if (n_in == 1) return launch_copy(dtype == PCCL_F32 || dtype == PCCL_I32 ? 4 : 2, aligned, nt, grid, s, p);
+  if (n_in == 1) return launch_copy(es, unroll, aligned, nt, (unsigned)grid, s, p);
   switch (dtype) {
-    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, aligned, nt, grid, s, p);
-    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, aligned, nt, grid, s, p);
-    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, aligned, nt, grid, s, p);
-    default: return launch_typed<PCCL_F16>(compute, n_in, aligned, nt, grid, s, p);
+    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
+    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
+    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
+    default: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
   }
 }

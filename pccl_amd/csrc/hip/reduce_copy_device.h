@@ -190,7 +190,11 @@ struct RcOperands {
 // first pack.  Workgroup `wg` of `n_wg` takes chunks wg, wg+n_wg, ... of
 // kBlock*UNROLL packs; inside a chunk lane t takes packs t, t+kBlock, ... so
 // every load and store instruction of a wavefront covers 1 KiB contiguously.
-template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, bool NT>
+//
+// NTL / NTS mark loads / stores non-temporal (streaming).  Measured on MI355X with
+// buffers far larger than the 256 MB Infinity Cache: reductions want both, a plain
+// copy wants only the stores; cache-resident sizes want neither.
+template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, bool NTL, bool NTS>
 __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, long wg, long n_wg) {
   constexpr long kChunk = (long)kBlock * UNROLL;
   for (long base = wg * kChunk; base < n_packs; base += n_wg * kChunk) {
@@ -201,15 +205,15 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
       for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
         for (int k = 0; k < NIN; ++k)
-          v[u][k] = load_pack<D, ALIGNED, NT>(a.in[k] + (p0 + (long)u * kBlock) * 16);
+          v[u][k] = load_pack<D, ALIGNED, NTL>(a.in[k] + (p0 + (long)u * kBlock) * 16);
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const u32x4 r = fold_pack<D, Op, NIN>(v[u]);
         const long off = (p0 + (long)u * kBlock) * 16;
-        store_pack<D, true, NT>(a.out[0] + off, r);
+        store_pack<D, true, NTS>(a.out[0] + off, r);
 #pragma unroll
         for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-          if (j < a.n_out) store_pack<D, ALIGNED, NT>(a.out[j] + off, r);
+          if (j < a.n_out) store_pack<D, ALIGNED, NTS>(a.out[j] + off, r);
       }
     } else {  // last, partial chunk: same shape, every pack guarded
 #pragma unroll
@@ -218,12 +222,12 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
         if (p < n_packs) {
           u32x4 v[NIN];
 #pragma unroll
-          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, NT>(a.in[k] + p * 16);
+          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, NTL>(a.in[k] + p * 16);
           const u32x4 r = fold_pack<D, Op, NIN>(v);
-          store_pack<D, true, NT>(a.out[0] + p * 16, r);
+          store_pack<D, true, NTS>(a.out[0] + p * 16, r);
 #pragma unroll
           for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-            if (j < a.n_out) store_pack<D, ALIGNED, NT>(a.out[j] + p * 16, r);
+            if (j < a.n_out) store_pack<D, ALIGNED, NTS>(a.out[j] + p * 16, r);
         }
       }
     }

@@ -15,10 +15,16 @@ struct RcLaunch {
   long count;      // elements in all
 };
 
-// Loads a lane keeps in flight per chunk: n_in * unroll packs of 16 bytes.
-__host__ __device__ constexpr int unroll_for(int n_in) { return n_in >= 5 ? 1 : n_in >= 3 ? 2 : 8 / n_in; }
+// Packs per lane per workgroup.  Measured on MI355X: with streams larger than
+// the Infinity Cache one pack per lane and one workgroup per 4 KiB of every stream
+// (the hardware dispatcher then walks memory in address order) beats every
+// persistent / grid-stride shape for all n_in; only cache-resident copies and
+// 2-input reductions gain (about 5 %) from 4 packs per lane.
+__host__ __device__ constexpr int small_unroll_for(int n_in) { return n_in <= 2 ? 4 : 1; }
 
-template <int DT, class Op, int NIN, bool ALIGNED, bool NT>
+// NT: streaming hint.  Reductions apply it to loads and stores, a copy to its
+// stores only.
+template <int DT, class Op, int NIN, int UNROLL, bool ALIGNED, bool NT>
 __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
   typedef Dtype<DT> D;
   constexpr int kEpp = 16 / D::kElemBytes;  // elements per pack
@@ -30,7 +36,7 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.ops.n_out) body.out[j] = p.ops.out[j] + p.head * D::kElemBytes;
-    body_packs<D, Op, NIN, unroll_for(NIN), ALIGNED, NT>(body, p.n_packs, blockIdx.x, gridDim.x);
+    body_packs<D, Op, NIN, UNROLL, ALIGNED, (NT && NIN > 1), NT>(body, p.n_packs, blockIdx.x, gridDim.x);
   }
   // head and tail elements: the last wavefront of the last workgroup
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x >= kBlock - kWave) {
@@ -39,14 +45,14 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
   }
 }
 
-template <int DT, class Op, int NIN>
-int launch_nin(bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+template <int DT, class Op, int NIN, int UNROLL>
+int launch_shape(bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
   if (aligned) {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, true, true>), dim3(grid), dim3(kBlock), 0, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, true, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, true>), dim3(grid), dim3(kBlock), 0, stream, p);
+    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, false>), dim3(grid), dim3(kBlock), 0, stream, p);
   } else {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, false, true>), dim3(grid), dim3(kBlock), 0, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, false, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, true>), dim3(grid), dim3(kBlock), 0, stream, p);
+    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, false>), dim3(grid), dim3(kBlock), 0, stream, p);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
@@ -54,38 +60,47 @@ int launch_nin(bool aligned, bool nt, unsigned grid, hipStream_t stream, const R
   return PCCL_OK;
 }
 
+// unroll is 1 or small_unroll_for(NIN); the two coincide for n_in >= 3
+template <int DT, class Op, int NIN>
+int launch_nin(int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+  if constexpr (small_unroll_for(NIN) != 1) {
+    if (unroll != 1) return launch_shape<DT, Op, NIN, small_unroll_for(NIN)>(aligned, nt, grid, stream, p);
+  }
+  return launch_shape<DT, Op, NIN, 1>(aligned, nt, grid, stream, p);
+}
+
 template <int DT, class Op>
-int launch_op(int n_in, bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+int launch_op(int n_in, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
   switch (n_in) {
-    case 2: return launch_nin<DT, Op, 2>(aligned, nt, grid, stream, p);
-    case 3: return launch_nin<DT, Op, 3>(aligned, nt, grid, stream, p);
-    case 4: return launch_nin<DT, Op, 4>(aligned, nt, grid, stream, p);
-    case 5: return launch_nin<DT, Op, 5>(aligned, nt, grid, stream, p);
-    case 6: return launch_nin<DT, Op, 6>(aligned, nt, grid, stream, p);
-    case 7: return launch_nin<DT, Op, 7>(aligned, nt, grid, stream, p);
-    case 8: return launch_nin<DT, Op, 8>(aligned, nt, grid, stream, p);
+    case 2: return launch_nin<DT, Op, 2>(unroll, aligned, nt, grid, stream, p);
+    case 3: return launch_nin<DT, Op, 3>(unroll, aligned, nt, grid, stream, p);
+    case 4: return launch_nin<DT, Op, 4>(unroll, aligned, nt, grid, stream, p);
+    case 5: return launch_nin<DT, Op, 5>(unroll, aligned, nt, grid, stream, p);
+    case 6: return launch_nin<DT, Op, 6>(unroll, aligned, nt, grid, stream, p);
+    case 7: return launch_nin<DT, Op, 7>(unroll, aligned, nt, grid, stream, p);
+    case 8: return launch_nin<DT, Op, 8>(unroll, aligned, nt, grid, stream, p);
     default: return pccl_host::fail(PCCL_ERR_INVALID_ARG, "n_in %d outside [1, 8]", n_in);
   }
 }
 
 // n_in >= 2.  Defined once per dtype (reduce_copy_inst_*.hip).
 template <int DT>
-int launch_typed(int compute, int n_in, bool aligned, bool nt, unsigned grid, hipStream_t stream,
-                 const RcLaunch &p);
+int launch_typed(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid,
+                 hipStream_t stream, const RcLaunch &p);
 
 // n_in == 1: bytes move unchanged, so only the element size matters.
-int launch_copy(int elem_bytes, bool aligned, bool nt, unsigned grid, hipStream_t stream,
+int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream,
                 const RcLaunch &p);
 
 #define PCCL_DEFINE_LAUNCH_TYPED(DT)                                                            \
   template <>                                                                                   \
-  int launch_typed<DT>(int compute, int n_in, bool aligned, bool nt, unsigned grid,             \
+  int launch_typed<DT>(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid, \
                        hipStream_t stream, const RcLaunch &p) {                                 \
     switch (compute) {                                                                          \
-      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, aligned, nt, grid, stream, p);           \
-      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, aligned, nt, grid, stream, p);         \
-      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, aligned, nt, grid, stream, p);           \
-      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, aligned, nt, grid, stream, p);           \
+      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, unroll, aligned, nt, grid, stream, p);           \
+      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, unroll, aligned, nt, grid, stream, p);         \
+      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, unroll, aligned, nt, grid, stream, p);           \
+      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, unroll, aligned, nt, grid, stream, p);           \
       default: return pccl_host::fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute); \
     }                                                                                           \
   }
