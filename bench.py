@@ -18,8 +18,8 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size (figures and commands in
-# profiles/reduce_copy_bf16_8in_256MiB.pmc.txt).  None until that profile has been taken.
-MEASURED_TRAFFIC_BYTES = None
+# profiles/reduce_copy_bf16_8in_256MiB.md).
+MEASURED_TRAFFIC_BYTES = 2414675968
 
 
 def parse():
@@ -29,6 +29,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibration-copy", type=int, default=0, metavar="N",
+                    help="also launch N plain copies (1 input -> 1 output) of the same 256 MiB buffers: the "
+                         "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     return ap.parse_args()
 
 
@@ -139,6 +142,9 @@ def main():
     for k in range(1, 8):
         ref = ref + ins[k][:1 << 20].float()
     assert torch.equal(ref.to(torch.bfloat16), out[:1 << 20]), "headline output differs from fp32-accumulated fold"
+    for _ in range(args.calibration_copy):
+        hip.reduce_copy("bf16", "sum", [ins[0]], [out], count, stream)
+    torch.cuda.synchronize()
 
     extras = {}
     if not args.no_extras:
