@@ -1,0 +1,152 @@
+#include "engine.h"
+
+#include <stdexcept>
+
+#include "device_plugin.h"
+#include "executor.h"
+#include "launch_env.h"
+
+namespace engine_c {
+
+Engine::Engine(int rank, int world_size) : rank_(rank), world_size_(world_size) {
+  if (world_size < 1 || rank < 0 || rank >= world_size)
+    throw std::runtime_error("Engine: rank " + std::to_string(rank) + " outside world of " + std::to_string(world_size));
+}
+
+Engine::~Engine() {
+  operators_.reset();  // graphs first: they hold device memory of their own
+  for (auto &[type, ptr] : owned_) {
+    try {
+      getDev(type)->deallocate(ptr);
+    } catch (const std::exception &e) {
+      PCCL_LOG_WARN("Engine: releasing a workspace failed: %s", e.what());
+    }
+  }
+}
+
+void Engine::initEngine() {
+  if (buffers_) throw std::runtime_error("Engine::initEngine(): already initialised");
+  buffers_ = std::make_unique<BufferManager>();
+  operators_ = std::make_unique<OperatorManager>();
+  available_remote_devices_.clear();
+  available_memory_devices_.clear();
+  for (DeviceType device : TypeRegistry::getDeviceTypes()) {
+    const std::string device_name(TypeRegistry::getTypeName(device));
+    auto dev = getDev(device);
+    // No plugin of this build offers remote communication or IPC, so the
+    // reference's first two branches (csrc/engine.cc:56-73) are never taken.
+    if (dev->remoteCommAvailable()) available_remote_devices_.push_back(device_name);
+    if (!dev->allocatorAvailable()) continue;
+    void *buffer = dev->allocate(TOTAL_SIZE);
+    if (!buffer) {
+      PCCL_LOG_WARN("Engine::initEngine(): device '%s' could not allocate its workspace", device_name.c_str());
+      continue;
+    }
+    owned_.push_back({device, buffer});
+    int *signal_buffer = reinterpret_cast<int *>(static_cast<char *>(buffer) + WORKSPACE_SIZE);
+    buffers_->regBuffer(buffer, WORKSPACE_SIZE, signal_buffer, SLOT, rank_, device);
+    available_memory_devices_.push_back(device_name);
+  }
+}
+
+void Engine::regOp(const std::string &name, const std::string &filepath) { regOp(name, Schedule::load(filepath)); }
+
+void Engine::regOp(const std::string &name, Schedule schedule) {
+  if (!operators_) throw std::runtime_error("Engine::regOp(): call initEngine() first");
+  schedule.validate();
+  // every name the schedule uses must be known to the registry and runnable by the hip executor
+  const ExecutorType hip = TypeRegistry::getTypeId("hip");
+  const auto &ok = TypeRegistry::getCompatibleTypes(hip);
+  for (const std::string &n : {schedule.dtype, schedule.compute})
+    if (!TypeRegistry::hasType(n) || !ok.count(TypeRegistry::getTypeId(n)))
+      throw std::runtime_error("Engine::regOp(): executor 'hip' does not support '" + n + "'");
+  auto op = operators_->add(name, std::move(schedule));
+  op->executor = getExecutor(hip);
+}
+
+void Engine::exeOp(const std::string &name, const void *input, void *output, long input_bytes, long output_bytes,
+                   void *stream) {
+  if (!operators_) throw std::runtime_error("Engine::exeOp(): call initEngine() first");
+  auto op = operators_->get(name);
+  const Schedule &s = op->schedule;
+  const long es = s.elemBytes();
+  const long need = (long)s.devices * s.elems_per_device * es;
+  if (!input || !output) throw std::runtime_error("Engine::exeOp(): null tensor");
+  if (input_bytes < need || output_bytes < need)
+    throw std::runtime_error("Engine::exeOp(): '" + name + "' needs " + std::to_string(need) +
+                             " bytes per tensor, got " + std::to_string(input_bytes) + " / " + std::to_string(output_bytes));
+  if (!op->graph) {
+    const DeviceType rocm = TypeRegistry::getTypeId("rocm");
+    char *ws = nullptr;
+    long ws_bytes = 0;
+    if (buffers_->hasDevBuffer(rocm)) {
+      ws = static_cast<char *>(std::get<0>(buffers_->getDevBuffer(rocm)));
+      ws_bytes = buffers_->getDevBufferSize(rocm);
+    }
+    const DataType dt = TypeRegistry::getTypeId(s.dtype);
+    const ComputeType compute = TypeRegistry::getTypeId(s.compute);
+    const PrimitiveType copy = TypeRegistry::getTypeId("copy"), reduce = TypeRegistry::getTypeId("reduce");
+    auto resolve = [&](const ScheduleOperand &x, long count) -> void * {
+      if (x.buffer == "ws") {
+        const long per_device = ws_bytes / s.devices / es;
+        if (!ws || x.offset + count > per_device)
+          throw std::runtime_error("Engine::exeOp(): workspace operand does not fit the device workspace");
+        return ws + ((long)x.device * per_device + x.offset) * es;
+      }
+      const char *base = x.buffer == "in" ? static_cast<const char *>(input) : static_cast<char *>(output);
+      return const_cast<char *>(base) + ((long)x.device * s.elems_per_device + x.offset) * es;
+    };
+    std::vector<BoundOp> bound(s.ops.size());
+    for (size_t i = 0; i < s.ops.size(); ++i) {
+      const ScheduleOp &o = s.ops[i];
+      BoundOp &b = bound[i];
+      b.primitive = o.reduce ? reduce : copy;
+      b.compute = compute;
+      b.deps = o.deps;
+      for (const auto &x : o.srcs) b.ins.push_back(ChunkMeta{dt, resolve(x, o.count), o.count});
+      for (const auto &x : o.dsts) b.outs.push_back(ChunkMeta{dt, resolve(x, o.count), o.count});
+    }
+    op->graph = op->executor->createGraph(bound);
+    op->bound_in = input;
+    op->bound_out = output;
+  } else if (op->bound_in != input || op->bound_out != output) {
+    // New tensors.  Moving operands range by range is only safe when no new range
+    // touches an old one (an operand must not be moved twice); otherwise rebuild.
+    auto apart = [need](const void *a, const void *b) {
+      const char *x = static_cast<const char *>(a), *y = static_cast<const char *>(b);
+      return x + need <= y || y + need <= x;
+    };
+    const bool in_moves = op->bound_in != input, out_moves = op->bound_out != output;
+    const bool safe = apart(op->bound_in, op->bound_out) && apart(input, output) &&
+                      (!in_moves || (apart(input, op->bound_in) && apart(input, op->bound_out))) &&
+                      (!out_moves || (apart(output, op->bound_out) && apart(output, op->bound_in)));
+    if (safe) {
+      if (in_moves) op->executor->rebindGraph(op->graph, op->bound_in, input, need, stream);
+      if (out_moves) op->executor->rebindGraph(op->graph, op->bound_out, output, need, stream);
+      op->bound_in = input;
+      op->bound_out = output;
+    } else {
+      op->executor->waitGraph(op->graph, stream);
+      op->executor->destroyGraph(op->graph);
+      op->graph = nullptr;
+      exeOp(name, input, output, input_bytes, output_bytes, stream);
+      return;
+    }
+  }
+  op->executor->runGraph(op->graph, stream);
+}
+
+void Engine::waitOp(const std::string &name, void *stream) {
+  auto op = operators_->get(name);
+  if (!op->graph) return;
+  const auto [done, total] = op->executor->waitGraph(op->graph, stream);
+  if (done != total)
+    throw std::runtime_error("Engine::waitOp(): '" + name + "' completed " + std::to_string(done) + " of " +
+                             std::to_string(total) + " operators");
+}
+
+std::string Engine::exportEndpoint() { throw std::runtime_error("Engine::exportEndpoint(): no cluster control plane in this build"); }
+void Engine::joinCluster(const std::string &) { throw std::runtime_error("Engine::joinCluster(): no cluster control plane in this build"); }
+void Engine::exitCluster() { throw std::runtime_error("Engine::exitCluster(): no cluster control plane in this build"); }
+
+}  // namespace engine_c

@@ -1,0 +1,79 @@
+// schedule.h -- a compiled collective: the op list Engine::regOp(name, filepath)
+// loads, its on-disk text format, and native generators.
+//
+// The reference passes a file path to regOp (include/engine.h:18) but defines
+// neither the format nor a producer (csrc/engine.cc:102-104 is empty,
+// pccl/lang/operator.py and example/collective/allreduce.py are empty files).
+// An op record carries what a PrimitiveOp of pccl/lang/chunk.py:46-55 carries:
+// kind, id (= position), source / target chunks as (buffer, device, element
+// offset), element count, dependencies.
+//
+// File format, one token stream, '#' starts a comment line:
+//   pccl-schedule 1
+//   name <word>
+//   dtype <f32|i32|bf16|f16>
+//   compute <sum|prod|min|max>
+//   devices <W>
+//   elems_per_device <N>          elements of every device's "in" and "out" region
+//   ops <n>
+//   op <id> <COPY|REDUCE> <count> deps <k> <id>*k  src <s> (<buffer> <device> <offset>)*s
+//                                                  dst <d> (<buffer> <device> <offset>)*d
+// Buffers: "in" and "out" are the tensors given to exeOp, laid out as W consecutive
+// per-device regions of elems_per_device elements; "ws" is the device workspace.
+#pragma once
+
+#include <string>
+#include <vector>
+
+namespace engine_c {
+
+struct ScheduleOperand {
+  std::string buffer;  // "in", "out" or "ws"
+  int device = 0;
+  long offset = 0;     // elements, inside the device's region
+};
+
+struct ScheduleOp {
+  bool reduce = false;  // false: COPY
+  long count = 0;
+  std::vector<int> deps;
+  std::vector<ScheduleOperand> srcs;
+  std::vector<ScheduleOperand> dsts;
+};
+
+struct Schedule {
+  std::string name;
+  std::string dtype = "bf16";
+  std::string compute = "sum";
+  int devices = 1;
+  long elems_per_device = 0;
+  std::vector<ScheduleOp> ops;
+
+  int elemBytes() const;
+  // Structural checks: operand ranges, dependency ids, acyclicity.  Throws std::runtime_error.
+  void validate() const;
+  // Op ids in the order DirectedGraph.topological_sort of pccl/lang/utils/graph.py:94-112
+  // produces for this DAG (reverse DFS post-order, nodes in id order, successors in
+  // edge-insertion order).
+  std::vector<int> topologicalOrder() const;
+
+  std::string serialize() const;
+  static Schedule parse(const std::string &text);
+  static Schedule load(const std::string &path);
+  void save(const std::string &path) const;
+};
+
+// Appends an out-of-place ring all-reduce over `devices` virtual ranks, `chunk_elems`
+// elements per chunk, regions starting at element `base`; returns the new base.
+long appendRingAllReduce(Schedule &s, long chunk_elems, long base);
+
+// Direct ("NVLS-style") all-reduce: device d reduces slice d of all W inputs in one
+// W-input op and writes it to every device's output (W outputs), W ops, no dependencies.
+long appendDirectAllReduce(Schedule &s, long slice_elems, long base);
+
+// The small-message program: n_slices ring all-reduces with log-uniform chunk sizes in
+// [lo_bytes, hi_bytes] plus n_extra independent copies; seed selects the sizes.
+Schedule makeSmallMessageSchedule(int devices, int n_slices, int n_extra, unsigned long seed,
+                                  long lo_bytes, long hi_bytes, const std::string &dtype);
+
+}  // namespace engine_c

@@ -89,10 +89,11 @@ class CollectiveIR:
     def add_device(self, device: Device):
         # the topology graph numbers nodes densely in insertion order (graph.py:23-27), so
         # device ids must be 0, 1, 2, ... in the order they are added
-        node = self.device_topology.add_node(device.device_id)
-        if node != device.device_id:
+        expected = self.device_topology.num_nodes()
+        if device.device_id != expected:
             raise ValueError("device ids must be dense and added in order (got %d, expected %d)"
-                             % (device.device_id, node))
+                             % (device.device_id, expected))
+        self.device_topology.add_node(device.device_id)
         self.devices[device.device_id] = device
 
     def add_link(self, link: Link):
@@ -137,6 +138,29 @@ class CollectiveIR:
             return [self.ops[i] for i in self.op_dag.topological_sort()]
         except ValueError:
             return []
+
+    # -- the engine's schedule file -------------------------------------------------------
+    def serialize(self, elems_per_device=None):
+        """Text of the schedule file ``Engine.regOp(name, filepath)`` loads (format documented
+        in ``pccl_amd/csrc/host/schedule.h``)."""
+        low = self.lower()
+        if elems_per_device is None:
+            elems_per_device = max([x[2] + o["count"] for o in low for x in o["ins"] + o["outs"] if x[0] != "ws"] or [0])
+        lines = ["pccl-schedule 1", "name %s" % (self.name.replace(" ", "_") or "unnamed"), "dtype %s" % self.dtype,
+                 "compute %s" % self.compute, "devices %d" % max(len(self.devices), 1),
+                 "elems_per_device %d" % elems_per_device, "ops %d" % len(low)]
+        for i, o in enumerate(low):
+            parts = ["op %d %s %d deps %d" % (i, "REDUCE" if o["primitive"] == 1 else "COPY", o["count"], len(o["deps"]))]
+            parts += [str(d) for d in o["deps"]]
+            for key, ops in (("src", o["ins"]), ("dst", o["outs"])):
+                parts.append("%s %d" % (key, len(ops)))
+                parts += ["%s %d %d" % (b, dev, off) for (b, dev, off) in ops]
+            lines.append(" ".join(parts))
+        return "\n".join(lines) + "\n"
+
+    def save(self, path, elems_per_device=None):
+        with open(path, "w") as f:
+            f.write(self.serialize(elems_per_device))
 
     # -- lowering to operand level --------------------------------------------------------
     def lower(self):

@@ -68,3 +68,38 @@ def edges_of(ops):
     """(src, dst) pairs in the order CollectiveIR.create_operation adds them
     (reference pccl/lang/chunk.py:104-106: for each op, one edge per dependency)."""
     return [(d, i) for i, o in enumerate(ops) for d in o["deps"]]
+
+
+def parse_schedule_text(text):
+    """Test-side reader of the engine's schedule file (independent of the product parser).
+    Returns (header dict, ops) with ops in the symbolic form used by `materialise`."""
+    toks = []
+    for line in text.splitlines():
+        line = line.strip()
+        if line and not line.startswith("#"):
+            toks += line.split()
+    it = iter(toks)
+
+    def nxt():
+        return next(it)
+
+    assert nxt() == "pccl-schedule" and nxt() == "1"
+    hdr = {}
+    for key in ("name", "dtype", "compute", "devices", "elems_per_device", "ops"):
+        assert nxt() == key
+        hdr[key] = nxt()
+    for key in ("devices", "elems_per_device", "ops"):
+        hdr[key] = int(hdr[key])
+    ops = []
+    for i in range(hdr["ops"]):
+        assert nxt() == "op" and int(nxt()) == i
+        kind, count = nxt(), int(nxt())
+        assert nxt() == "deps"
+        deps = [int(nxt()) for _ in range(int(nxt()))]
+        sides = []
+        for key in ("src", "dst"):
+            assert nxt() == key
+            sides.append([(nxt(), int(nxt()), int(nxt())) for _ in range(int(nxt()))])
+        assert kind in ("COPY", "REDUCE")
+        ops.append(dict(dtype=hdr["dtype"], compute=hdr["compute"], ins=sides[0], outs=sides[1], count=count, deps=deps))
+    return hdr, ops

@@ -1,0 +1,271 @@
+"""CPU-side tests of the host layer and the C ABI surface (no GPU needed): exported symbols,
+TypeRegistry, device plugins, schedule format and generators, the Python collective IR."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import schedules as S
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def E():
+    from pccl_amd import engine
+    engine.lib()
+    return engine
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pccl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    from pccl_amd import hip, engine
+    for header, path in (("pccl_hip.h", hip.LIB_PATH), ("pccl_engine.h", engine.LIB_PATH)):
+        names = _declared(header)
+        assert len(names) >= 15, names
+        L = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+        for n in names:
+            assert hasattr(L, n), "%s declares %s but %s does not export it" % (header, n, os.path.basename(path))
+
+
+def test_layout_header_compiles_as_c_and_matches_reference_offsets(tmp_path):
+    """pccl_op_layout.h is plain C; offsets are those of the reference's operator.h / chunk.h (LP64)."""
+    src = tmp_path / "t.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include "pccl_op_layout.h"
+int main(void) {
+  printf("%zu %zu %zu\n", sizeof(pccl_chunk_meta), offsetof(pccl_chunk_meta, addr_), offsetof(pccl_chunk_meta, num_elems_));
+  printf("%zu %zu %zu %zu %zu\n", sizeof(pccl_ring_buffer), offsetof(pccl_ring_buffer, elem_size_), offsetof(pccl_ring_buffer, tail_), offsetof(pccl_ring_buffer, head_), offsetof(pccl_ring_buffer, consumer_buffer_));
+  printf("%zu %zu %zu %zu %zu %zu\n", sizeof(pccl_operation_layout_header), offsetof(pccl_operation_layout_header, remaining_executors_), offsetof(pccl_operation_layout_header, pre_dependencies_), offsetof(pccl_operation_layout_header, num_next_ops_), offsetof(pccl_operation_layout_header, op_buffer_), offsetof(pccl_operation_layout_header, next_op_uids_head_));
+  printf("%zu %zu %zu %zu\n", sizeof(pccl_graph_buffer_layout), offsetof(pccl_graph_buffer_layout, operators), offsetof(pccl_graph_buffer_layout, ready_queues), offsetof(pccl_graph_buffer_layout, num_queues));
+  return 0;
+}''')
+    exe = tmp_path / "t"
+    import subprocess
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    assert out[0] == "24 8 16"
+    assert out[1] == "40 4 16 20 32"
+    assert out[2] == "32 8 12 15 16 24"
+    assert out[3] == "48 16 32 40"
+
+
+# ---- TypeRegistry ------------------------------------------------------------------------------
+
+def test_registry_plugins_registered_at_load(E):
+    assert set(E.device_types()) == {"cpu", "rocm"}
+    for n in ("copy", "reduce", "notify", "get_notified", "f32", "i32", "bf16", "f16", "sum", "prod", "min", "max", "hip"):
+        assert E.type_name(E.type_id(n)) == n
+    ids = [E.type_id(n) for n in ("cpu", "rocm", "hip", "copy", "f32", "sum")]
+    assert len(set(ids)) == len(ids), "all kinds share one id space"
+    for n in ("copy", "reduce", "f32", "i32", "bf16", "f16", "sum", "prod", "min", "max"):
+        assert E.is_compatible("hip", n)
+    assert not E.is_compatible("hip", "notify") and not E.is_compatible("hip", "get_notified")
+
+
+def test_registry_register_and_errors(E):
+    a = E.register_type("data", "test_dtype_x")
+    assert E.register_type("data", "test_dtype_x") == a, "same name, same id"
+    b = E.register_type("compute", "test_compute_y")
+    assert b == a + 1, "one shared counter"
+    with pytest.raises(E.EngineError):
+        E.register_type("device", "test_dtype_x")  # already a data type
+    with pytest.raises(E.EngineError):
+        E.type_id("no_such_type")
+    with pytest.raises(E.EngineError):
+        E.type_name(250)
+    with pytest.raises(E.EngineError):
+        E.register_compatibility("no_such_executor", "f32")
+    with pytest.raises(E.EngineError):
+        E.register_compatibility("hip", "no_such_type")
+    E.register_compatibility("hip", "test_dtype_x")
+    assert E.is_compatible("hip", "test_dtype_x")
+
+
+# ---- device plugins ----------------------------------------------------------------------------
+
+def test_cpu_plugin_allocator(E):
+    assert E.allocator_available("cpu")
+    assert not E.ipc_available("cpu") and not E.ipc_available("rocm")
+    p = E.allocate("cpu", 1 << 20)
+    assert p
+    buf = (ctypes.c_ubyte * (1 << 20)).from_address(p)
+    buf[0], buf[(1 << 20) - 1] = 7, 9
+    assert (buf[0], buf[(1 << 20) - 1]) == (7, 9)
+    E.deallocate("cpu", p)
+    assert E.allocate("cpu", 0) is None and E.allocate("cpu", -5) is None
+    with pytest.raises(E.EngineError):
+        E.allocator_available("hip")  # an executor, not a device
+
+
+def test_launch_options_listed(E):
+    assert {"PCCL_HIP_WG_PER_CU", "PCCL_HIP_NT", "PCCL_HIP_TILE_BYTES"} <= set(E.LaunchEnvironments.listOpt())
+    assert E.LaunchEnvironments.getEnv("PCCL_SURELY_UNSET_VARIABLE") == ""
+    assert E.LaunchEnvironments.getEnv("PATH") == os.environ["PATH"]
+
+
+# ---- schedules ----------------------------------------------------------------------------------
+
+def test_native_and_python_emitters_agree(E, tmp_path):
+    from pccl_amd import lang
+    p = str(tmp_path / "a.sched")
+    E.write_small_message(p)
+    ir, per = lang.small_message_allreduce()
+    assert open(p).read() == ir.serialize(per)
+    for world, n, dt, op in ((8, 1000, "f32", "max"), (2, 5, "bf16", "sum"), (3, 77, "i32", "prod"), (1, 4, "f16", "min")):
+        E.write_ring_allreduce(p, dt, op, world, n)
+        ir, per = lang.ring_allreduce(world, n, dt, op)
+        assert open(p).read() == ir.serialize(per)
+
+
+def test_schedule_order_matches_reference_rule(E, oracle, tmp_path):
+    """Schedule::topologicalOrder, the Python DirectedGraph and the CPU checker's restatement of
+    pccl/lang/utils/graph.py:94-112 give the same order, and it respects every dependency."""
+    from pccl_amd import lang
+    p = str(tmp_path / "a.sched")
+    E.write_small_message(p, n_slices=3, n_extra=5)
+    info = E.inspect_schedule(p)
+    hdr, ops = S.parse_schedule_text(open(p).read())
+    assert info["n_ops"] == len(ops) == 3 * 112 + 5 and info["devices"] == 8
+    assert info["order"] == oracle.topo_sort(len(ops), S.edges_of(ops))
+    ir, _ = lang.small_message_allreduce(n_slices=3, n_extra=5)
+    assert info["order"] == [o.op_id for o in ir.get_operation_sequence()]
+    pos = {op: i for i, op in enumerate(info["order"])}
+    assert all(pos[d] < pos[i] for i, o in enumerate(ops) for d in o["deps"])
+
+
+def test_direct_allreduce_schedule_shape(E, tmp_path):
+    p = str(tmp_path / "d.sched")
+    E.write_direct_allreduce(p, "bf16", "sum", 8, 4096)
+    hdr, ops = S.parse_schedule_text(open(p).read())
+    assert hdr["elems_per_device"] == 8 * 4096 and len(ops) == 16
+    red, bc = ops[0], ops[1]
+    assert [x[1] for x in red["ins"]] == list(range(8)) and len(red["outs"]) == 1
+    assert len(bc["ins"]) == 1 and len(bc["outs"]) == 7 and bc["deps"] == [0]
+
+
+@pytest.mark.parametrize("text, why", [
+    ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "version"),
+    ("pccl-schedule 1\nname x\ndtype f64\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "dtype"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute xor\ndevices 1\nelems_per_device 4\nops 0\n", "compute"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 NOTIFY 4 deps 0 src 1 in 0 0 dst 1 out 0 0\n", "NOTIFY"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 COPY 8 deps 0 src 1 in 0 0 dst 1 out 0 0\n", "past elems_per_device"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 COPY 4 deps 0 src 1 in 0 0 dst 1 in 0 0\n", "read-only"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 2\n"
+     "op 0 COPY 4 deps 1 1 src 1 in 0 0 dst 1 out 0 0\nop 1 COPY 4 deps 1 0 src 1 in 0 0 dst 1 out 0 0\n", "cycle"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 COPY 4 deps 0 src 2 in 0 0 in 0 0 dst 1 out 0 0\n", "one source"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 2\nelems_per_device 4\nops 1\n"
+     "op 0 COPY 4 deps 0 src 1 in 2 0 dst 1 out 0 0\n", "device"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n", "end of file"),
+])
+def test_schedule_parser_rejects(E, text, why):
+    eng = E.Engine(0, 1)
+    eng.initEngine()
+    with pytest.raises(E.EngineError) as e:
+        eng.regOpText("bad", text)
+    assert why.lower() in str(e.value).lower(), str(e.value)
+    eng.close()
+
+
+def test_engine_without_gpu_fails_loudly(E, tmp_path):
+    """On a box without a GPU the engine initialises (cpu workspace only), registers schedules, and
+    exeOp raises instead of computing anything on the CPU."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("this check is for boxes without a GPU")
+    eng = E.Engine(0, 1)
+    eng.initEngine()
+    ws, sig, nbytes = eng.getDevBuffer("cpu")
+    assert nbytes == 1 << 28 and sig == ws + (1 << 28)
+    with pytest.raises(E.EngineError):
+        eng.getDevBuffer("rocm")
+    p = str(tmp_path / "r.sched")
+    E.write_ring_allreduce(p, "f32", "sum", 2, 16)
+    eng.regOp("ar", p)
+    assert eng.opInfo("ar") == {"n_ops": 4, "devices": 2, "elems_per_device": 32, "elem_bytes": 4}
+    a, b = torch.zeros(64), torch.zeros(64)
+    with pytest.raises(E.EngineError):
+        eng.exeOp("ar", a, b)
+    with pytest.raises(E.EngineError):
+        eng.exeOp("unknown_name", a, b)
+    for call in (eng.exportEndpoint, eng.exitCluster, lambda: eng.joinCluster("127.0.0.1:1")):
+        with pytest.raises(E.EngineError) as e:
+            call()
+        assert "control plane" in str(e.value)
+    with pytest.raises(E.EngineError):
+        E.Engine(3, 2)
+    eng.close()
+
+
+# ---- Python collective IR (reference pccl/lang) -----------------------------------------------------
+
+def test_directed_graph_follows_reference_rules():
+    from pccl_amd.lang import DirectedGraph
+    g = DirectedGraph()
+    assert [g.add_node(data=100 + i) for i in range(4)] == [0, 1, 2, 3]  # ids are dense; data is not the id
+    with pytest.raises(ValueError):
+        g.add_edge(0, 4)
+    for e in ((0, 1), (0, 2), (1, 3), (2, 3)):
+        g.add_edge(*e)
+    assert g.get_successors(0) == [1, 2] and g.get_predecessors(3) == [1, 2]
+    assert g.is_acyclic() and g.topological_sort() == [0, 2, 1, 3]
+    g.add_edge(3, 0)
+    assert not g.is_acyclic()
+    with pytest.raises(ValueError):
+        g.topological_sort()
+    g.remove_edge(3, 0)
+    assert g.is_acyclic()
+    h = DirectedGraph()
+    for _ in range(5):
+        h.add_node()
+    h.add_edge(0, 1)
+    h.add_edge(3, 4)
+    assert sorted(map(sorted, h.get_connected_components())) == [[0, 1], [2], [3, 4]]
+    deep = DirectedGraph()
+    for i in range(5000):  # deeper than the interpreter's recursion limit
+        deep.add_node()
+        if i:
+            deep.add_edge(i - 1, i)
+    assert deep.topological_sort() == list(range(5000))
+
+
+def test_collective_ir_container():
+    from pccl_amd.lang import Chunk, CollectiveIR, Device, DeviceType, Link, PrimitiveOpType
+    ir = CollectiveIR("t", dtype="f32")
+    for d in range(3):
+        ir.add_device(Device(d, DeviceType.ROCM, 8e12, 9.5))
+    with pytest.raises(ValueError):
+        ir.add_device(Device(7, DeviceType.ROCM, 8e12, 9.5))  # ids must be dense, in order
+    ir.add_link(Link(0, 1, 1e11, 1e-6))
+    assert not ir.validate_topology()
+    ir.add_link(Link(1, 2, 1e11, 1e-6))
+    assert ir.validate_topology()
+    assert ir.get_device_bandwidth_matrix()[(2, 1)] == 1e11
+    c = Chunk({0}, 0, 16, 0)
+    c2 = c.copy()
+    c2.reduced_ranks.add(1)
+    assert c.reduced_ranks == {0}
+    a = ir.create_operation(PrimitiveOpType.COPY, c, Chunk({0}, 1, 16, 0), 0, 1)
+    b = ir.create_operation(PrimitiveOpType.REDUCE, Chunk({0}, 1, 16, 0), Chunk({0, 2}, 2, 16, 0), 1, 2, dependencies=[a])
+    assert (a, b) == (0, 1) and ir.validate_dag()
+    assert [o.op_id for o in ir.get_operation_sequence()] == [0, 1]
+    low = ir.lower()
+    assert low[1]["ins"] == [("out", 1, 0), ("out", 2, 0)] and low[1]["outs"] == [("out", 2, 0)]  # reduce src into tgt
+    ir.create_operation(PrimitiveOpType.NOTIFY, c, c, 0, 1)
+    with pytest.raises(NotImplementedError):
+        ir.lower()
+    bad = CollectiveIR("cyc")
+    x = bad.create_operation(PrimitiveOpType.COPY, c, c, 0, 0)
+    bad.op_dag.add_edge(x, x)
+    assert not bad.validate_dag() and bad.get_operation_sequence() == []
