@@ -1,0 +1,165 @@
+"""GPU parity at the full sizes of the five baseline configurations.  Inputs are seeded on the
+device, downloaded once, and the CPU checker (threaded form, same arithmetic as the scalar form)
+computes the expected bytes; every comparison is bit-exact."""
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+THREADS = 16
+NPDT = {"f32": np.float32, "i32": np.int32, "bf16": np.uint16, "f16": np.uint16}
+
+
+def _stream(torch):
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev_random(torch, dtype, count, seed, kind="normal", sigma=1.0, lo=0.5, hi=2.0):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    if dtype == "i32":
+        return torch.randint(-(1 << 20), (1 << 20) + 1, (count,), dtype=torch.int32, device="cuda", generator=g)
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+    out = torch.empty(count, dtype=tdt, device="cuda")
+    step = 1 << 26
+    for a in range(0, count, step):
+        b = min(count, a + step)
+        if kind == "normal":
+            out[a:b] = (torch.randn(b - a, device="cuda", generator=g) * sigma).to(tdt)
+        else:
+            out[a:b] = (torch.rand(b - a, device="cuda", generator=g) * (hi - lo) + lo).to(tdt)
+    return out
+
+
+def _host(t, dtype):
+    """Device tensor -> numpy array in the checker's storage type."""
+    a = t.cpu()
+    if dtype in ("bf16", "f16"):
+        return a.view(__import__("torch").int16).numpy().view(np.uint16)
+    return a.numpy()
+
+
+def _expect(oracle, dtype, compute, host_ins):
+    out = np.empty_like(host_ins[0])
+    oracle.reduce_copy(dtype, compute, host_ins, [out], nthreads=THREADS)
+    return out
+
+
+def test_config2_ring_rank_share_full_size(hip, oracle):
+    """bf16 ring all-reduce, one rank's share at world 8: 256 MiB gradient = 8 x 32 MiB chunks, 7
+    reduce-copy steps (peer chunk + local chunk -> output chunk + send buffer) and 7 copy steps."""
+    import torch
+    W, ce = 8, 1 << 24
+    grad = _dev_random(torch, "bf16", W * ce, 1, sigma=1e-2)
+    peers = [_dev_random(torch, "bf16", ce, 100 + s, sigma=1e-2) for s in range(W - 1)]
+    result = torch.zeros(W * ce, dtype=torch.bfloat16, device="cuda")
+    send = torch.zeros(ce, dtype=torch.bfloat16, device="cuda")
+    h_grad, h_peers = _host(grad, "bf16"), [_host(p, "bf16") for p in peers]
+    h_result = np.zeros(W * ce, dtype=np.uint16)
+    for s in range(W - 1):
+        c = (W - 1 - s) % W
+        sl = slice(c * ce, (c + 1) * ce)
+        hip.reduce_copy("bf16", "sum", [peers[s], grad[sl]], [result[sl], send], ce, _stream(torch))
+        torch.cuda.synchronize()
+        want = _expect(oracle, "bf16", "sum", [h_peers[s], h_grad[sl]])
+        h_result[sl] = want
+        H.assert_bits_equal(_host(send, "bf16"), want, "send buffer after reduce step %d" % s)
+    for s in range(W - 1):
+        c = (W - s) % W
+        sl = slice(c * ce, (c + 1) * ce)
+        hip.reduce_copy("bf16", "sum", [peers[s]], [result[sl]], ce, _stream(torch))
+        h_result[sl] = h_peers[s]
+    torch.cuda.synchronize()
+    H.assert_bits_equal(_host(result, "bf16"), h_result, "assembled 256 MiB result")
+
+
+@pytest.mark.parametrize("dtype, n_out, count", [("bf16", 1, 1 << 26), ("f16", 2, 1 << 26), ("bf16", 1, 1 << 27)])
+def test_config3_eight_input_reduce_full_size(hip, oracle, dtype, n_out, count):
+    """8 inputs -> 1 (or 2) outputs, 128 MiB and 256 MiB per buffer, fixed input order."""
+    import torch
+    ins = [_dev_random(torch, dtype, count, 2000 + k) for k in range(8)]
+    outs = [torch.zeros(count, dtype=ins[0].dtype, device="cuda") for _ in range(n_out)]
+    hip.reduce_copy(dtype, "sum", ins, outs, count, _stream(torch))
+    torch.cuda.synchronize()
+    want = _expect(oracle, dtype, "sum", [_host(t, dtype) for t in ins])
+    for j, o in enumerate(outs):
+        H.assert_bits_equal(_host(o, dtype), want, "%s 8->%d output %d" % (dtype, n_out, j))
+    # the same fold in torch (fp32 accumulate, input order, one rounding) as a second opinion
+    acc = ins[0][:1 << 22].float()
+    for k in range(1, 8):
+        acc = acc + ins[k][:1 << 22].float()
+    assert torch.equal(acc.to(ins[0].dtype), outs[0][:1 << 22])
+
+
+# forced members of the count list plus a log-uniform draw from [1, 2^28] (seed 3)
+FORCED = [1, 2, 3, 5, 7, 31, 127, 8191, 131071, 524287, (1 << 20) + 7, (1 << 24) - 3, (1 << 28) - 57, 1 << 28]
+
+
+def _config4_counts(oracle):
+    extra = []
+    for i in range(6):
+        u = (oracle.rng_u64(3, 99, i) >> 11) / float(1 << 53)
+        extra.append(max(1, int(2.0 ** (28.0 * u))))
+    return FORCED + extra
+
+
+@pytest.mark.parametrize("dtype, compute", [("i32", "sum"), ("i32", "max"), ("f32", "min"), ("f32", "prod")])
+def test_config4_unaligned_mixed_ops(hip, oracle, dtype, compute):
+    """4 inputs -> 1 output; every buffer sits 4..60 bytes past a 64-byte boundary, independently;
+    counts include 1, primes and 2^28."""
+    import torch
+    counts = _config4_counts(oracle)
+    big = max(counts)
+    kind = "uniform" if dtype == "f32" else "normal"
+    pool = [_dev_random(torch, dtype, big + 64, 3000 + k, kind=kind) for k in range(4)]
+    out_pool = torch.zeros((big + 64) * 4 + 256, dtype=torch.uint8, device="cuda")
+    h_pool = [_host(p, dtype) for p in pool]
+    assert all(p.data_ptr() % 64 == 0 for p in pool) and out_pool.data_ptr() % 64 == 0
+    for ci, count in enumerate(counts):
+        offs = [4 * (1 + (oracle.rng_u64(3, 7, ci * 8 + k) % 15)) for k in range(5)]  # 4..60 bytes
+        assert all(4 <= o <= 60 for o in offs)
+        in_ptrs = [pool[k].data_ptr() + offs[k] for k in range(4)]
+        out_ptr = out_pool.data_ptr() + 64 + offs[4]
+        guard_lo = out_pool[:64 + offs[4]].clone()
+        hip.reduce_copy(dtype, compute, in_ptrs, [out_ptr], count, _stream(torch))
+        torch.cuda.synchronize()
+        h_ins = [h_pool[k][offs[k] // 4: offs[k] // 4 + count] for k in range(4)]
+        want = _expect(oracle, dtype, compute, [np.ascontiguousarray(a) for a in h_ins])
+        lo = 64 + offs[4]
+        got = out_pool[lo:lo + 4 * count].cpu().numpy().view(NPDT[dtype])
+        H.assert_bits_equal(got, want, "%s %s count=%d offsets=%s" % (dtype, compute, count, offs))
+        assert torch.equal(out_pool[:lo], guard_lo), "bytes before the output were touched"
+        assert int(out_pool[lo + 4 * count: lo + 4 * count + 64].max()) == 0, "bytes after the output were touched"
+        out_pool[lo:lo + 4 * count].zero_()
+
+
+def test_config5_small_message_schedule_full_size(hip, oracle):
+    """4096 ops (36 ring all-reduces over 8 virtual ranks + 64 copies), bf16 sum, op sizes log-uniform in
+    [8 KiB, 256 KiB], one persistent launch; compared with the checker replaying the op list."""
+    import torch
+    import schedules as S
+    from pccl_amd import lang
+    ir, per = lang.small_message_allreduce()
+    low = ir.lower()
+    assert len(low) == 4096
+    sizes_b = [o["count"] * 2 for o in low]
+    assert min(sizes_b) >= 8 << 10 and max(sizes_b) <= 256 << 10
+    d_in = [_dev_random(torch, "bf16", per, 4000 + r) for r in range(8)]
+    d_out = [torch.zeros(per, dtype=torch.bfloat16, device="cuda") for _ in range(8)]
+    dev = {"in": d_in, "out": d_out}
+    g = hip.Graph(lang.bind(low, lambda b, r, e: dev[b][r].data_ptr() + 2 * e))
+    h = {"in": [_host(t, "bf16") for t in d_in], "out": [np.zeros(per, dtype=np.uint16) for _ in range(8)]}
+    order = oracle.topo_sort(len(low), [(d, i) for i, o in enumerate(low) for d in o["deps"]])
+    host_ops = [dict(o, ins=[h[b][r][e:e + o["count"]] for (b, r, e) in o["ins"]],
+                     outs=[h[b][r][e:e + o["count"]] for (b, r, e) in o["outs"]]) for o in low]
+    oracle.run_ops(host_ops, order)
+    for it in range(3):
+        g.run(_stream(torch))
+        assert g.status(_stream(torch)) == (4096, 4096)
+        for r in range(8):
+            H.assert_bits_equal(_host(d_out[r], "bf16"), h["out"][r], "run %d rank %d" % (it, r))
+        for t in d_out:
+            t.zero_()
+    g.destroy()

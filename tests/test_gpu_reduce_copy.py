@@ -91,6 +91,30 @@ def test_in_place_ring_step(hip, oracle):
     assert d_b.guards_intact() and d_send.guards_intact()
 
 
+def test_fold_order_is_input_order(hip, oracle):
+    """f32 inputs with a wide exponent spread: folding the same buffers in reversed order gives
+    different bits, and the kernel matches the checker for both orders (sum and prod)."""
+    import torch
+    count = 50021
+    for n_in in (3, 8):
+        ins = []
+        for k in range(n_in):
+            mag = np.exp2(oracle.fill_uniform_f32(count, 300, 10 + k, -20.0, 20.0)).astype(np.float32)
+            ins.append(oracle.fill_uniform_f32(count, 300, k, -1.0, 1.0) * mag)
+        fwd, rev = oracle.reduce("f32", "sum", ins), oracle.reduce("f32", "sum", ins[::-1])
+        assert not np.array_equal(fwd.view(np.uint32), rev.view(np.uint32)), "input not order-sensitive: weak test"
+        (got,) = H.hip_reduce(torch, hip, "f32", "sum", ins)
+        H.assert_bits_equal(got, fwd, "forward order n_in=%d" % n_in)
+        (got,) = H.hip_reduce(torch, hip, "f32", "sum", ins[::-1])
+        H.assert_bits_equal(got, rev, "reversed order n_in=%d" % n_in)
+    # (1e8 + 1) - 1e8 = 0 from the left, 1 when the big terms cancel first
+    a, b, c = (np.full(1000, v, dtype=np.float32) for v in (1e8, 1.0, -1e8))
+    (got,) = H.hip_reduce(torch, hip, "f32", "sum", [a, b, c])
+    assert np.all(got == 0.0)
+    (got,) = H.hip_reduce(torch, hip, "f32", "sum", [a, c, b])
+    assert np.all(got == 1.0)
+
+
 def test_special_values(hip, oracle):
     """inf, NaN, signed zero, subnormals and rounding ties through the bf16 / f16 / f32 paths."""
     import torch
