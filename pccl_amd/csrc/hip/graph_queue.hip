@@ -14,6 +14,12 @@
 //   * the workgroup finishing the last part of an op decrements
 //     pre_dependencies_ of each successor (32-bit atomic on the word at offset
 //     12) and publishes the successors that reach zero;
+//   * data moves between workgroups (possibly on different XCDs, whose L2s are not
+//     coherent with each other) through device-coherent accesses: parts load and
+//     store with sc1, wait for their stores, and only then touch the counters with
+//     relaxed device-scope atomics.  An L2-wide write-back + invalidate per part
+//     (what agent-scope release / acquire fences compile to) was measured to cost
+//     about 100 us per part under load;
 //   * per-op mutable state is restored by the op's last part and the run's
 //     last workgroup rewinds the queue and re-publishes the initial entries,
 //     so a finished graph is armed for its next run;
@@ -76,11 +82,14 @@ __device__ __forceinline__ void run_part_body(const RcOperands &a, long head, lo
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < a.n_out) body.out[j] = a.out[j] + head * D::kElemBytes;
-    constexpr int kUnroll = NIN >= 4 ? 1 : NIN >= 2 ? 2 : 4;
-    body_packs<D, Op, NIN, kUnroll, ALIGNED, false, false>(body, n_packs, 0, 1);
+    // Every access of a part is device-coherent: its inputs may have been written
+    // by a workgroup on another XCD moments ago, and its outputs may be read by one.
+    constexpr int kUnroll = NIN >= 3 ? 1 : 2;
+    body_packs<D, Op, NIN, kUnroll, ALIGNED, kMemCoherent, kMemCoherent>(body, n_packs, 0, 1);
   }
   if (threadIdx.x >= kBlock - kWave)
-    edge_elems<D, Op, NIN>(a, head, head + n_packs * kEpp, count, (int)threadIdx.x - (kBlock - kWave));
+    edge_elems<D, Op, NIN, kMemCoherent>(a, head, head + n_packs * kEpp, count, (int)threadIdx.x - (kBlock - kWave));
+  settle_stores();
 }
 
 template <class D, class Op, int NIN>
@@ -149,9 +158,11 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(GraphControl *g) {
   int parts = 0;
   for (;;) {
     if (threadIdx.x == 0) {
-      if (h) {  // the part executed in the previous iteration is complete (barrier below)
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        const int old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_ACQ_REL, AGENT);
+      if (h) {  // the part executed in the previous iteration is complete (barrier below):
+        // every wavefront waited for its write-through stores before that barrier, so
+        // the data is at the point of coherence and relaxed device-scope atomics are
+        // enough to hand it over; no L2 write-back / invalidate is involved
+        const int old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
         if (old == 1) {  // it was the op's last part
           __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
           __hip_atomic_store(word12(h), pl->initial_word12_, __ATOMIC_RELAXED, AGENT);
@@ -159,13 +170,13 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(GraphControl *g) {
           const int *next = h->next_op_uids_head_;
           for (int s = 0; s < n_next; ++s) {
             pccl_operation_layout_header *hs = &g->headers[next[s]];
-            const unsigned int w = __hip_atomic_fetch_sub(word12(hs), 1u, __ATOMIC_ACQ_REL, AGENT);
+            const unsigned int w = __hip_atomic_fetch_sub(word12(hs), 1u, __ATOMIC_RELAXED, AGENT);
             if ((w & 0xffu) == 1u) {  // last dependency gone: publish all its parts
               const int r = hs->required_executors_;
               const int pos = __hip_atomic_fetch_add(&q->tail_, r, __ATOMIC_RELAXED, AGENT);
               for (int p = 0; p < r; ++p) {
                 const unsigned long long e = (unsigned long long)(unsigned int)next[s] | ((unsigned long long)p << 32);
-                __hip_atomic_store(&slots[pos + p], e, __ATOMIC_RELEASE, AGENT);
+                __hip_atomic_store(&slots[pos + p], e, __ATOMIC_RELAXED, AGENT);
               }
             }
           }
@@ -191,7 +202,6 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(GraphControl *g) {
           }
         }
         if (t < total_tiles) {
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
           __hip_atomic_store(&slots[t], kEmptySlot, __ATOMIC_RELAXED, AGENT);  // slot ready for the next run
           s_entry = e;
         }
@@ -219,7 +229,8 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(GraphControl *g) {
 
   // leave: the last workgroup out re-arms the graph for the next run
   if (threadIdx.x == 0) {
-    const unsigned int e = __hip_atomic_fetch_add(&g->exit_count, 1u, __ATOMIC_ACQ_REL, AGENT);
+    settle_stores();  // this workgroup's counter updates land before it counts as gone
+    const unsigned int e = __hip_atomic_fetch_add(&g->exit_count, 1u, __ATOMIC_RELAXED, AGENT);
     s_last = (e == gridDim.x - 1);
   }
   __syncthreads();

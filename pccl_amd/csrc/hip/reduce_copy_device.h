@@ -138,28 +138,75 @@ template <> struct Dtype<PCCL_F16> {
 // ---- pack load / store -------------------------------------------------------
 // ALIGNED: every stream is 16-byte aligned.  Otherwise only output 0 is (the
 // host peels a head so that it is) and the others are element-aligned.
-template <class D, bool ALIGNED, bool NT>
+//
+// Memory policy of an access:
+//   kMemCached    ordinary cached access;
+//   kMemStream    non-temporal hint (operands larger than the Infinity Cache);
+//   kMemCoherent  device-coherent access (sc1): loads read past, and stores write
+//                 through, this XCD's L2, which is not coherent with the L2s of the
+//                 other seven XCDs.  Used where workgroups on different XCDs hand
+//                 data to each other inside one kernel, so that no L2-wide
+//                 write-back / invalidate is needed at every hand-over.  Written
+//                 as inline assembly because the compiler offers sc1 only on
+//                 atomics of at most 8 bytes; the loads are invisible to its
+//                 wait-count tracking, so settle_loads() must precede their use.
+constexpr int kMemCached = 0, kMemStream = 1, kMemCoherent = 2;
+
+template <class D, bool ALIGNED, int MEM>
 __device__ __forceinline__ u32x4 load_pack(const char *p) {
-  if constexpr (ALIGNED) {
-    if constexpr (NT) return __builtin_nontemporal_load((const u32x4 *)p);
+  if constexpr (MEM == kMemCoherent) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+  } else if constexpr (ALIGNED) {
+    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const u32x4 *)p);
     else return *(const u32x4 *)p;
   } else {
     typedef typename D::pack_unaligned P;
-    if constexpr (NT) return __builtin_nontemporal_load((const P *)p);
+    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const P *)p);
     else return *(const P *)p;
   }
 }
 
-template <class D, bool ALIGNED, bool NT>
+template <class D, bool ALIGNED, int MEM>
 __device__ __forceinline__ void store_pack(char *p, u32x4 v) {
-  if constexpr (ALIGNED) {
-    if constexpr (NT) __builtin_nontemporal_store(v, (u32x4 *)p);
+  if constexpr (MEM == kMemCoherent) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+  } else if constexpr (ALIGNED) {
+    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (u32x4 *)p);
     else *(u32x4 *)p = v;
   } else {
     typedef typename D::pack_unaligned P;
-    if constexpr (NT) __builtin_nontemporal_store(v, (P *)p);
+    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (P *)p);
     else *(P *)p = v;
   }
+}
+
+// Makes the values of coherent loads usable: waits for all outstanding vector
+// memory operations and ties every loaded register to the wait, so that the
+// compiler cannot schedule a use above it.  Nothing to do for the other policies.
+template <int MEM, int N>
+__device__ __forceinline__ void settle_loads(u32x4 (&v)[N]) {
+  if constexpr (MEM == kMemCoherent) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[k]) : : "memory");
+  }
+}
+
+// Waits until every coherent store issued by this wavefront has reached the
+// point of coherence (needed before another workgroup is told the data exists).
+__device__ __forceinline__ void settle_stores() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
+
+template <class E, int MEM>
+__device__ __forceinline__ E load_elem(const E *p) {
+  if constexpr (MEM == kMemCoherent) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *p;
+}
+
+template <class E, int MEM>
+__device__ __forceinline__ void store_elem(E *p, E v) {
+  if constexpr (MEM == kMemCoherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
 }
 
 template <class D, class Op, int NIN>
@@ -191,10 +238,10 @@ struct RcOperands {
 // kBlock*UNROLL packs; inside a chunk lane t takes packs t, t+kBlock, ... so
 // every load and store instruction of a wavefront covers 1 KiB contiguously.
 //
-// NTL / NTS mark loads / stores non-temporal (streaming).  Measured on MI355X with
-// buffers far larger than the 256 MB Infinity Cache: reductions want both, a plain
-// copy wants only the stores; cache-resident sizes want neither.
-template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, bool NTL, bool NTS>
+// LD / ST are the memory policies of loads / stores.  Measured on MI355X with
+// buffers far larger than the 256 MB Infinity Cache: reductions want both
+// streaming, a plain copy wants only the stores; cache-resident sizes want neither.
+template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, int LD, int ST>
 __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, long wg, long n_wg) {
   constexpr long kChunk = (long)kBlock * UNROLL;
   for (long base = wg * kChunk; base < n_packs; base += n_wg * kChunk) {
@@ -205,15 +252,17 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
       for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
         for (int k = 0; k < NIN; ++k)
-          v[u][k] = load_pack<D, ALIGNED, NTL>(a.in[k] + (p0 + (long)u * kBlock) * 16);
+          v[u][k] = load_pack<D, ALIGNED, LD>(a.in[k] + (p0 + (long)u * kBlock) * 16);
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) settle_loads<LD>(v[u]);
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const u32x4 r = fold_pack<D, Op, NIN>(v[u]);
         const long off = (p0 + (long)u * kBlock) * 16;
-        store_pack<D, true, NTS>(a.out[0] + off, r);
+        store_pack<D, true, ST>(a.out[0] + off, r);
 #pragma unroll
         for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-          if (j < a.n_out) store_pack<D, ALIGNED, NTS>(a.out[j] + off, r);
+          if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + off, r);
       }
     } else {  // last, partial chunk: same shape, every pack guarded
 #pragma unroll
@@ -222,12 +271,13 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
         if (p < n_packs) {
           u32x4 v[NIN];
 #pragma unroll
-          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, NTL>(a.in[k] + p * 16);
+          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, LD>(a.in[k] + p * 16);
+          settle_loads<LD>(v);
           const u32x4 r = fold_pack<D, Op, NIN>(v);
-          store_pack<D, true, NTS>(a.out[0] + p * 16, r);
+          store_pack<D, true, ST>(a.out[0] + p * 16, r);
 #pragma unroll
           for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-            if (j < a.n_out) store_pack<D, ALIGNED, NTS>(a.out[j] + p * 16, r);
+            if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + p * 16, r);
         }
       }
     }
@@ -236,7 +286,7 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
 
 // Edge elements, one per lane of a single wavefront: elements [0, head) and
 // [tail_begin, count) of the ORIGINAL (un-advanced) streams.
-template <class D, class Op, int NIN>
+template <class D, class Op, int NIN, int MEM = kMemCached>
 __device__ __forceinline__ void edge_elems(const RcOperands &a, long head, long tail_begin,
                                            long count, int lane) {
   typedef typename D::elem_t E;
@@ -245,13 +295,13 @@ __device__ __forceinline__ void edge_elems(const RcOperands &a, long head, long 
     const long i = e < head ? e : tail_begin + (e - head);
     E x[NIN];
 #pragma unroll
-    for (int k = 0; k < NIN; ++k) x[k] = ((const E *)a.in[k])[i];
+    for (int k = 0; k < NIN; ++k) x[k] = load_elem<E, MEM>((const E *)a.in[k] + i);
     E r;
     if constexpr (NIN == 1) r = x[0];
     else r = D::template elem<Op, NIN>(x);
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
-      if (j < a.n_out) ((E *)a.out[j])[i] = r;
+      if (j < a.n_out) store_elem<E, MEM>((E *)a.out[j] + i, r);
   }
 }
 

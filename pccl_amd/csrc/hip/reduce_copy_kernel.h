@@ -36,7 +36,8 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.ops.n_out) body.out[j] = p.ops.out[j] + p.head * D::kElemBytes;
-    body_packs<D, Op, NIN, UNROLL, ALIGNED, (NT && NIN > 1), NT>(body, p.n_packs, blockIdx.x, gridDim.x);
+    body_packs<D, Op, NIN, UNROLL, ALIGNED, (NT && NIN > 1) ? kMemStream : kMemCached, NT ? kMemStream : kMemCached>(
+        body, p.n_packs, blockIdx.x, gridDim.x);
   }
   // head and tail elements: the last wavefront of the last workgroup
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x >= kBlock - kWave) {
