@@ -91,6 +91,11 @@ int pccl_hip_reduce_copy(int dtype, int compute, const void *const *ins, int n_i
  * (0 = built-in choice) and non-temporal access hint (0/1, -1 = built-in). */
 int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);
 
+/* Occupancy override for tuning runs: bytes of (unused) dynamic LDS requested per
+ * workgroup, which caps the workgroups resident on a compute unit at
+ * floor(160 KiB / lds_bytes); -1 = built-in choice, 0 = no cap. */
+int pccl_hip_set_occupancy_lds(int lds_bytes);
+
 /* ---- the op-batching path: a DAG of ops drained by one persistent kernel -- */
 
 /* One IR operation as the host hands it over: the C++ payload level of

@@ -40,7 +40,7 @@ int compute_units() {
 }
 
 static std::mutex g_tuning_mutex;
-static Tuning g_tuning = {0, -1};
+static Tuning g_tuning = {0, -1, -1};
 static bool g_tuning_env_read = false;
 
 Tuning tuning() {
@@ -49,6 +49,7 @@ Tuning tuning() {
     g_tuning_env_read = true;
     if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tuning.workgroups_per_cu = atoi(s);
     if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.nontemporal = atoi(s) ? 1 : 0;
+    if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tuning.lds_bytes = atoi(s);
   }
   return g_tuning;
 }
@@ -134,6 +135,15 @@ int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal) {
   std::lock_guard<std::mutex> lock(g_tuning_mutex);
   g_tuning.workgroups_per_cu = workgroups_per_cu;
   g_tuning.nontemporal = nontemporal < 0 ? -1 : (nontemporal ? 1 : 0);
+  return PCCL_OK;
+}
+
+int pccl_hip_set_occupancy_lds(int lds_bytes) {
+  clear_error();
+  if (lds_bytes > 160 * 1024) return fail(PCCL_ERR_INVALID_ARG, "lds_bytes %d exceeds the 160 KiB of a compute unit", lds_bytes);
+  (void)tuning();
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  g_tuning.lds_bytes = lds_bytes < 0 ? -1 : lds_bytes;
   return PCCL_OK;
 }
 

@@ -22,6 +22,7 @@ int compute_units();
 struct Tuning {
   int workgroups_per_cu;  // 0 = built-in choice
   int nontemporal;        // -1 = built-in choice, else 0/1
+  int lds_bytes;          // -1 = built-in choice, else dynamic LDS requested per workgroup
 };
 Tuning tuning();
 

@@ -7,11 +7,11 @@
 
 namespace pccl_dev {
 
-int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream,
-                const RcLaunch &p) {
+int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
+                hipStream_t stream, const RcLaunch &p) {
   // the dtype only selects the alignment the unaligned pack type may assume
-  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, nt, grid, stream, p);
-  return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, stream, p);
+  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
+  return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
 }
 
 }  // namespace pccl_dev
@@ -77,20 +77,39 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   const long total_bytes = (long)(n_in + n_out) * count * es;
   const bool big = total_bytes > (192l << 20);
   const bool nt = t.nontemporal < 0 ? big : t.nontemporal != 0;
-  const int unroll = big ? 1 : small_unroll_for(n_in);
-  const long chunk = (long)kBlock * unroll;
+  int unroll = big ? 1 : small_unroll_for(n_in);
+  // lean kernel: nothing to peel, at most two outputs, and no gain expected from
+  // several packs per lane
+  const int epp = 16 / es;
+  if (aligned && p.head == 0 && p.n_packs * epp == count && n_out <= 2 && unroll == 1 && t.workgroups_per_cu == 0)
+    unroll = 0;
+  const long chunk = (long)kBlock * (unroll ? unroll : 1);
   long chunks = (p.n_packs + chunk - 1) / chunk;
   if (chunks < 1) chunks = 1;
   // default: one workgroup per chunk; a tuning run may cap it to a persistent grid
   long grid = chunks;
   if (t.workgroups_per_cu > 0) grid = std::min<long>(chunks, (long)pccl_host::compute_units() * t.workgroups_per_cu);
   if (grid > 0x7fffffffl) grid = 0x7fffffffl;  // the kernel's chunk loop covers the rest
+  // Occupancy cap for operands beyond the Infinity Cache.  Measured on MI355X: DRAM
+  // efficiency is best with about 20 (workgroups x streams) resident per compute
+  // unit, i.e. 2 workgroups for 8 -> 1 (+8 %), 5 for 2 -> 2 (+10 %), no cap for a
+  // copy; more concurrent streams per memory channel cost row-buffer locality.  The
+  // cap is imposed by requesting dynamic LDS the kernel never touches.
+  unsigned lds = 0;
+  if (t.lds_bytes >= 0) {
+    lds = (unsigned)t.lds_bytes;
+  } else if (big) {
+    const int streams = n_in + n_out;
+    int wgs = (20 + streams / 2) / streams;
+    wgs = std::max(2, std::min(8, wgs));
+    if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
+  }
   hipStream_t s = (hipStream_t)stream;
-  if (n_in == 1) return launch_copy(es, unroll, aligned, nt, (unsigned)grid, s, p);
+  if (n_in == 1) return launch_copy(es, unroll, aligned, nt, (unsigned)grid, lds, s, p);
   switch (dtype) {
-    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
-    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
-    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
-    default: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, s, p);
+    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    default: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
   }
 }

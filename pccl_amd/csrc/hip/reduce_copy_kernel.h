@@ -46,14 +46,67 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
   }
 }
 
+// ---- lean kernel for the common case -------------------------------------------
+// Every stream 16-byte aligned, count a whole number of packs, at most two
+// outputs: one pack per lane, one workgroup per 4 KiB of every stream, no loop,
+// no edge code.  A workgroup lives for only a few microseconds, so what it does
+// before its first load matters: the arguments hold nothing but the pointers it
+// needs, the per-workgroup offset is added on the scalar unit and the per-lane
+// offset is a 32-bit value (scalar-base addressing, no 64-bit vector adds).
+template <int NIN, int NOUT>
+struct RcLean {
+  const char *in[NIN];
+  char *out[NOUT];
+  long n_packs;
+};
+
+template <int DT, class Op, int NIN, int NOUT, bool NT>
+__global__ void __launch_bounds__(kBlock) reduce_copy_lean_kernel(const RcLean<NIN, NOUT> a) {
+  typedef Dtype<DT> D;
+  constexpr int kLd = (NT && NIN > 1) ? kMemStream : kMemCached;
+  constexpr int kSt = NT ? kMemStream : kMemCached;
+  const unsigned lane_off = threadIdx.x * 16u;
+  const size_t wg_off = (size_t)blockIdx.x * (kBlock * 16);
+  if ((long)blockIdx.x * kBlock + threadIdx.x < a.n_packs) {
+    u32x4 v[NIN];
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, true, kLd>(a.in[k] + wg_off + lane_off);
+    const u32x4 r = fold_pack<D, Op, NIN>(v);
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) store_pack<D, true, kSt>(a.out[j] + wg_off + lane_off, r);
+  }
+}
+
+template <int DT, class Op, int NIN, int NOUT>
+int launch_lean_nout(bool nt, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  RcLean<NIN, NOUT> a;
+  for (int k = 0; k < NIN; ++k) a.in[k] = p.ops.in[k];
+  for (int j = 0; j < NOUT; ++j) a.out[j] = p.ops.out[j];
+  a.n_packs = p.n_packs;
+  const unsigned grid = (unsigned)((p.n_packs + kBlock - 1) / kBlock);
+  if (nt) hipLaunchKernelGGL((reduce_copy_lean_kernel<DT, Op, NIN, NOUT, true>), dim3(grid), dim3(kBlock), lds, stream, a);
+  else hipLaunchKernelGGL((reduce_copy_lean_kernel<DT, Op, NIN, NOUT, false>), dim3(grid), dim3(kBlock), lds, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return pccl_host::fail(PCCL_ERR_HIP, "reduce_copy launch failed: %s", hipGetErrorString(e));
+  return PCCL_OK;
+}
+
+// requires: p.head == 0, p.n_packs * pack == p.count, all streams aligned, n_out <= 2
+template <int DT, class Op, int NIN>
+int launch_lean(bool nt, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  if (p.ops.n_out == 1) return launch_lean_nout<DT, Op, NIN, 1>(nt, lds, stream, p);
+  return launch_lean_nout<DT, Op, NIN, 2>(nt, lds, stream, p);
+}
+
 template <int DT, class Op, int NIN, int UNROLL>
-int launch_shape(bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+int launch_shape(bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
   if (aligned) {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, true>), dim3(grid), dim3(kBlock), 0, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, true>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, false>), dim3(grid), dim3(kBlock), lds, stream, p);
   } else {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, true>), dim3(grid), dim3(kBlock), 0, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, true>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, false>), dim3(grid), dim3(kBlock), lds, stream, p);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
@@ -61,47 +114,49 @@ int launch_shape(bool aligned, bool nt, unsigned grid, hipStream_t stream, const
   return PCCL_OK;
 }
 
-// unroll is 1 or small_unroll_for(NIN); the two coincide for n_in >= 3
+// unroll is 0 (lean kernel), 1 or small_unroll_for(NIN); the last two coincide for n_in >= 3
 template <int DT, class Op, int NIN>
-int launch_nin(int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+int launch_nin(int unroll, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  if (unroll == 0) return launch_lean<DT, Op, NIN>(nt, lds, stream, p);
   if constexpr (small_unroll_for(NIN) != 1) {
-    if (unroll != 1) return launch_shape<DT, Op, NIN, small_unroll_for(NIN)>(aligned, nt, grid, stream, p);
+    if (unroll != 1) return launch_shape<DT, Op, NIN, small_unroll_for(NIN)>(aligned, nt, grid, lds, stream, p);
   }
-  return launch_shape<DT, Op, NIN, 1>(aligned, nt, grid, stream, p);
+  return launch_shape<DT, Op, NIN, 1>(aligned, nt, grid, lds, stream, p);
 }
 
 template <int DT, class Op>
-int launch_op(int n_in, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream, const RcLaunch &p) {
+int launch_op(int n_in, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream,
+              const RcLaunch &p) {
   switch (n_in) {
-    case 2: return launch_nin<DT, Op, 2>(unroll, aligned, nt, grid, stream, p);
-    case 3: return launch_nin<DT, Op, 3>(unroll, aligned, nt, grid, stream, p);
-    case 4: return launch_nin<DT, Op, 4>(unroll, aligned, nt, grid, stream, p);
-    case 5: return launch_nin<DT, Op, 5>(unroll, aligned, nt, grid, stream, p);
-    case 6: return launch_nin<DT, Op, 6>(unroll, aligned, nt, grid, stream, p);
-    case 7: return launch_nin<DT, Op, 7>(unroll, aligned, nt, grid, stream, p);
-    case 8: return launch_nin<DT, Op, 8>(unroll, aligned, nt, grid, stream, p);
+    case 2: return launch_nin<DT, Op, 2>(unroll, aligned, nt, grid, lds, stream, p);
+    case 3: return launch_nin<DT, Op, 3>(unroll, aligned, nt, grid, lds, stream, p);
+    case 4: return launch_nin<DT, Op, 4>(unroll, aligned, nt, grid, lds, stream, p);
+    case 5: return launch_nin<DT, Op, 5>(unroll, aligned, nt, grid, lds, stream, p);
+    case 6: return launch_nin<DT, Op, 6>(unroll, aligned, nt, grid, lds, stream, p);
+    case 7: return launch_nin<DT, Op, 7>(unroll, aligned, nt, grid, lds, stream, p);
+    case 8: return launch_nin<DT, Op, 8>(unroll, aligned, nt, grid, lds, stream, p);
     default: return pccl_host::fail(PCCL_ERR_INVALID_ARG, "n_in %d outside [1, 8]", n_in);
   }
 }
 
 // n_in >= 2.  Defined once per dtype (reduce_copy_inst_*.hip).
 template <int DT>
-int launch_typed(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid,
+int launch_typed(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
                  hipStream_t stream, const RcLaunch &p);
 
 // n_in == 1: bytes move unchanged, so only the element size matters.
-int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, hipStream_t stream,
-                const RcLaunch &p);
+int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
+                hipStream_t stream, const RcLaunch &p);
 
 #define PCCL_DEFINE_LAUNCH_TYPED(DT)                                                            \
   template <>                                                                                   \
   int launch_typed<DT>(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid, \
-                       hipStream_t stream, const RcLaunch &p) {                                 \
+                       unsigned lds, hipStream_t stream, const RcLaunch &p) {                   \
     switch (compute) {                                                                          \
-      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, unroll, aligned, nt, grid, stream, p);           \
-      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, unroll, aligned, nt, grid, stream, p);         \
-      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, unroll, aligned, nt, grid, stream, p);           \
-      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, unroll, aligned, nt, grid, stream, p);           \
+      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
+      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, unroll, aligned, nt, grid, lds, stream, p);         \
+      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
+      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
       default: return pccl_host::fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute); \
     }                                                                                           \
   }
