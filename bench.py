@@ -19,7 +19,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size (figures and commands in
 # profiles/reduce_copy_bf16_8in_256MiB.md).
-MEASURED_TRAFFIC_BYTES = 2414675968
+MEASURED_TRAFFIC_BYTES = 2415523430
 
 
 def parse():
@@ -134,7 +134,7 @@ def main():
     achieved = step_bytes / mean_us / 1e3
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                 "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                "kernel": "reduce_copy_kernel<bf16, sum, n_in=8>", "algorithmic_bytes_per_launch": step_bytes,
+                "kernel": "reduce_copy_lean_kernel<bf16, sum, n_in=8, n_out=1>", "algorithmic_bytes_per_launch": step_bytes,
                 "launch_us": stats(ts)}
 
     # quick self-check of the timed buffers against torch's fp32 accumulate (same fold order)
