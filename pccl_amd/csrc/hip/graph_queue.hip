@@ -5,24 +5,36 @@
 // Protocol (the reference declares the structs, operator.h:7-38, but no code
 // reads or writes them, so the protocol is defined here):
 //   * an op is split into required_executors_ parts of about tile_bytes of
-//     output; a ready-queue entry names (op_uid, part);
-//   * workgroups claim entries by taking tickets from RingBuffer::head_; ticket
-//     t waits until slot t has been published (RingBuffer::tail_ hands out slot
-//     numbers to producers).  A slot is only ever published by a workgroup that
-//     holds a smaller ticket, and tickets are only held by running workgroups,
-//     so the drain cannot deadlock whatever the number of resident workgroups;
+//     output; a queue entry names (op_uid, part);
+//   * the entries of all ops are laid out once, at graph creation, in a
+//     topological order (dependency level, then op id, then part) and dealt
+//     round-robin onto kQueues ready queues (GraphBufferLayout::ready_queues /
+//     num_queues; RingBuffer::tail_ = number of entries).  Workgroup w serves
+//     queue w % kQueues first -- workgroups are dispatched round-robin over the 8
+//     XCDs, so the ticket counter of a queue is hammered from one XCD only -- and
+//     moves on to the other queues when its own is exhausted;
+//   * a workgroup claims an entry by taking a ticket from RingBuffer::head_,
+//     reads the entry, and waits until the op's pre_dependencies_ is 0.  Every
+//     dependency of a claimed entry lies earlier in the global order; each queue
+//     keeps at least one workgroup until it is exhausted; hence the unfinished
+//     claimed entry that comes first in the global order can always run, and the
+//     drain cannot deadlock whatever the number of resident workgroups;
 //   * the workgroup finishing the last part of an op decrements
 //     pre_dependencies_ of each successor (32-bit atomic on the word at offset
-//     12) and publishes the successors that reach zero;
+//     12; the count is the low byte and never borrows);
 //   * data moves between workgroups (possibly on different XCDs, whose L2s are not
 //     coherent with each other) through device-coherent accesses: parts load and
 //     store with sc1, wait for their stores, and only then touch the counters with
 //     relaxed device-scope atomics.  An L2-wide write-back + invalidate per part
 //     (what agent-scope release / acquire fences compile to) was measured to cost
 //     about 100 us per part under load;
+//   * hot-spot atomics are the throughput limit (about 30-60 ns each on one
+//     address): an earlier form with one queue, a tail_ reservation and a slot
+//     store/poll per entry spent 2 contended atomics per entry on two addresses;
+//     this form spends one, spread over kQueues addresses;
 //   * per-op mutable state is restored by the op's last part and the run's
-//     last workgroup rewinds the queue and re-publishes the initial entries,
-//     so a finished graph is armed for its next run;
+//     last workgroup rewinds the ticket counters, so a finished graph is armed
+//     for its next run;
 //   * every wait is bounded: when a wait exceeds spin_limit polls the kernel
 //     raises the abort flag, all workgroups leave, and the host reports
 //     PCCL_ERR_GRAPH instead of hanging.
@@ -39,26 +51,57 @@ using pccl_host::fail;
 
 namespace {
 
-constexpr unsigned long long kEmptySlot = ~0ull;
+constexpr int kQueues = 8;  // one per XCD of an MI355X
 constexpr long kDefaultTileBytes = 32 << 10;
 constexpr unsigned int kDefaultSpinLimit = 1u << 21;  // a few seconds of polling
 
-// Device-resident control block.  The reference's GraphBufferLayout is its
-// first member, so the arena's base address is a GraphBufferLayout*.
+// Words that many workgroups update or poll, each alone on its 256-byte line.
+// Device-scope atomics and sc1 loads are served at the memory side; an ordinary
+// cached load of the same line parks a copy in an XCD's L2 that every later
+// atomic must first probe out again.  Measured: with immutable fields (queue
+// length, entry pointer, part count) sharing lines with ticket counters and
+// dependency counts, a claim took 25 us and a part 13 us under 768 workgroups,
+// against 1.7 us and 1.9 us with 64.  So: lines that are written during a run
+// are touched by atomics / sc1 only, and everything a workgroup reads with
+// ordinary loads lives on lines that no one writes during a run.
+struct alignas(256) HotWord {
+  unsigned int value;
+};
+
+// Device-resident control block; read-only during a run.  The reference's
+// GraphBufferLayout is its first member, so the arena's base address is a
+// GraphBufferLayout*.
 struct GraphControl {
   pccl_graph_buffer_layout layout;
   pccl_operation_layout_header *headers;  // contiguous; layout.operators[i] == &headers[i]
-  unsigned long long *slots;              // ready-queue storage, one pccl_queue_entry each
-  const unsigned long long *initial;      // entries of the ops without dependencies
-  unsigned int completed;                 // *layout.completed_operator
-  unsigned int total;                     // *layout.total_operator
-  unsigned int done_count;                // ops finished in the current run
-  unsigned int exit_count;                // workgroups that have left the current run
-  unsigned int abort;                     // set when a bounded wait gave up
+  char *slots;                            // PayloadSlot of op i at slots + i * kPayloadStride
+  const int *succ;                        // all successor uid lists, back to back
+  HotWord *hot;                           // kHot* words, see below
+  int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
+  const unsigned long long *queue_entries[kQueues];
+  int queue_count[kQueues];
   unsigned int spin_limit;
-  int n_initial;
   int total_tiles;
 };
+
+// indices into GraphControl::hot
+constexpr int kHotCompleted = 0;  // *layout.completed_operator
+constexpr int kHotTotal = 1;      // *layout.total_operator (never written during a run)
+constexpr int kHotAbort = 2;      // set when a bounded wait gave up
+constexpr int kHotExit = 3;       // workgroups that have left the current run
+constexpr int kHotDone = 4;       // kQueues counters of finished ops, summed at the end
+constexpr int kHotWords = kHotDone + kQueues;
+
+// What a workgroup needs to run a part, on lines nothing writes during a run: the
+// op's payload plus the two header facts (part count, successor list) it would
+// otherwise have to read from the header, whose line is under atomic fire.
+constexpr size_t kPayloadStride = 256;
+struct PayloadSlot {
+  pccl_op_payload payload;  // 248 bytes; what OperationLayoutHeader::op_buffer_ points to
+  int parts;                // == required_executors_
+  int succ_start;           // successors at GraphControl::succ + succ_start
+};
+static_assert(sizeof(PayloadSlot) == kPayloadStride, "payload slot stride");
 
 __device__ __forceinline__ unsigned int *word12(pccl_operation_layout_header *h) {
   return (unsigned int *)((char *)h + 12);
@@ -138,125 +181,122 @@ __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, lon
 #define AGENT __HIP_MEMORY_SCOPE_AGENT
 
 template <int DT, class Op>
-__global__ void __launch_bounds__(kBlock) drain_graph_kernel(GraphControl *g) {
-  __shared__ int s_ticket;
+__global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
   __shared__ unsigned long long s_entry;
+  __shared__ int s_go;
   __shared__ int s_last;
-  pccl_ring_buffer *q = g->layout.ready_queues[0];
-  unsigned long long *slots = g->slots;
-  const int total_tiles = g->total_tiles;
-  const unsigned int spin_limit = g->spin_limit;
+  HotWord *hot = g.hot;
+  unsigned int *abort_flag = &hot[kHotAbort].value;
+  const unsigned int spin_limit = g.spin_limit;
+  const int home = blockIdx.x % kQueues;
 
   // Loop shape matters: thread 0's bookkeeping for the part just finished and its
-  // claim of the next ticket sit in ONE conditional block per iteration, and the
+  // claim of the next entry sit in ONE conditional block per iteration, and the
   // loop exit is a scalar branch (readfirstlane).  With two thread-0 blocks (one
   // before the back edge, one after it) the compiler threads the jump between
   // them, the back edge becomes divergent, and the other lanes of thread 0's
   // wavefront run ahead into the next barrier while thread 0 is parked.
   pccl_operation_layout_header *h = nullptr;
-  const pccl_op_payload *pl = nullptr;
-  int parts = 0;
+  const PayloadSlot *slot = nullptr;
+  unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   for (;;) {
     if (threadIdx.x == 0) {
-      if (h) {  // the part executed in the previous iteration is complete (barrier below):
+      if (h) {
+        // The part executed in the previous iteration is complete (barrier below):
         // every wavefront waited for its write-through stores before that barrier, so
         // the data is at the point of coherence and relaxed device-scope atomics are
-        // enough to hand it over; no L2 write-back / invalidate is involved
-        const int old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
+        // enough to hand it over; no L2 write-back / invalidate is involved.
+        const int parts = slot->parts;
+        int old = 1;
+        if (parts > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
         if (old == 1) {  // it was the op's last part
-          __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
-          __hip_atomic_store(word12(h), pl->initial_word12_, __ATOMIC_RELAXED, AGENT);
-          const int n_next = h->num_next_ops_;
-          const int *next = h->next_op_uids_head_;
-          for (int s = 0; s < n_next; ++s) {
-            pccl_operation_layout_header *hs = &g->headers[next[s]];
-            const unsigned int w = __hip_atomic_fetch_sub(word12(hs), 1u, __ATOMIC_RELAXED, AGENT);
-            if ((w & 0xffu) == 1u) {  // last dependency gone: publish all its parts
-              const int r = hs->required_executors_;
-              const int pos = __hip_atomic_fetch_add(&q->tail_, r, __ATOMIC_RELAXED, AGENT);
-              for (int p = 0; p < r; ++p) {
-                const unsigned long long e = (unsigned long long)(unsigned int)next[s] | ((unsigned long long)p << 32);
-                __hip_atomic_store(&slots[pos + p], e, __ATOMIC_RELAXED, AGENT);
-              }
-            }
-          }
-          __hip_atomic_fetch_add(&g->done_count, 1u, __ATOMIC_RELAXED, AGENT);
+          if (parts > 1) __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
+          const unsigned int w12 = slot->payload.initial_word12_;
+          if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);  // re-arm its own count
+          const int n_next = (int)(w12 >> 24);
+          const int *next = g.succ + slot->succ_start;
+          for (int s = 0; s < n_next; ++s)
+            __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
+          __hip_atomic_fetch_add(&hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
         }
       }
-      int t = total_tiles;  // "leave"
-      if (__hip_atomic_load(&g->abort, __ATOMIC_RELAXED, AGENT) == 0)
-        t = __hip_atomic_fetch_add(&q->head_, 1, __ATOMIC_RELAXED, AGENT);
-      if (t < total_tiles) {
-        if (t == 0) __hip_atomic_store(&g->completed, 0u, __ATOMIC_RELAXED, AGENT);
-        unsigned long long e;
+      int go = 0;
+      unsigned long long e = 0;
+      if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) == 0) {
+        for (int i = 0; i < kQueues && !go; ++i) {
+          const int q = (home + i) % kQueues;
+          if (exhausted & (1u << q)) continue;
+          const int n = g.queue_count[q];
+          const int t = n > 0 ? __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT) : n;
+          if (t < n) {
+            e = g.queue_entries[q][t];
+            go = 1;
+            if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
+          } else {
+            exhausted |= 1u << q;
+          }
+        }
+      }
+      if (go) {  // wait for the op's dependencies
+        unsigned int *dep = word12(&g.headers[(int)(e & 0xffffffffu)]);
         unsigned int spins = 0;
-        for (;;) {
-          e = __hip_atomic_load(&slots[t], __ATOMIC_RELAXED, AGENT);
-          if (e != kEmptySlot) break;
-          __builtin_amdgcn_s_sleep(2);
+        while ((__hip_atomic_load(dep, __ATOMIC_RELAXED, AGENT) & 0xffu) != 0) {
+          __builtin_amdgcn_s_sleep(1);
           if ((++spins & 63u) == 0 &&
-              (spins >= spin_limit || __hip_atomic_load(&g->abort, __ATOMIC_RELAXED, AGENT) != 0)) {
-            __hip_atomic_store(&g->abort, 1u, __ATOMIC_RELAXED, AGENT);
-            t = total_tiles;
+              (spins >= spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0)) {
+            __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
+            go = 0;
             break;
           }
         }
-        if (t < total_tiles) {
-          __hip_atomic_store(&slots[t], kEmptySlot, __ATOMIC_RELAXED, AGENT);  // slot ready for the next run
-          s_entry = e;
-        }
       }
-      s_ticket = t;
+      s_entry = e;
+      s_go = go;
     }
     __syncthreads();
-    if (__builtin_amdgcn_readfirstlane(s_ticket) >= total_tiles) break;
+    if (!__builtin_amdgcn_readfirstlane(s_go)) break;
     const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
     const int part = __builtin_amdgcn_readfirstlane((int)(s_entry >> 32));
-    h = &g->headers[uid];
-    pl = (const pccl_op_payload *)h->op_buffer_;
-    parts = h->required_executors_;
+    h = &g.headers[uid];
+    slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
+    const pccl_op_payload *pl = &slot->payload;
     const long count = pl->chunks_[0].num_elems_;
-    const long per = part_elems(count, parts);
+    const long per = part_elems(count, slot->parts);
     const long lo = (long)part * per;
     long n = count - lo;
     if (n > per) n = per;
     if (n > 0) run_part<DT, Op>(pl, lo, n);
-    // every store of this part is issued and complete at workgroup scope before
-    // thread 0 releases it at the top of the next iteration; also keeps s_entry /
-    // s_ticket from being rewritten while other wavefronts still read them
+    // every store of this part has reached the point of coherence (run_part waits)
+    // before thread 0 hands the part over at the top of the next iteration; the
+    // barrier also keeps s_entry / s_go from being rewritten while still being read
     __syncthreads();
   }
 
   // leave: the last workgroup out re-arms the graph for the next run
   if (threadIdx.x == 0) {
     settle_stores();  // this workgroup's counter updates land before it counts as gone
-    const unsigned int e = __hip_atomic_fetch_add(&g->exit_count, 1u, __ATOMIC_RELAXED, AGENT);
+    const unsigned int e = __hip_atomic_fetch_add(&hot[kHotExit].value, 1u, __ATOMIC_RELAXED, AGENT);
     s_last = (e == gridDim.x - 1);
   }
   __syncthreads();
   if (!__builtin_amdgcn_readfirstlane(s_last)) return;
-  if (__hip_atomic_load(&g->abort, __ATOMIC_RELAXED, AGENT) != 0) {
-    if (threadIdx.x == 0) {
-      __hip_atomic_store(&g->completed, __hip_atomic_load(&g->done_count, __ATOMIC_RELAXED, AGENT),
-                         __ATOMIC_RELAXED, AGENT);
-      __hip_atomic_store(&g->exit_count, 0u, __ATOMIC_RELAXED, AGENT);
-    }
-    return;  // state is inconsistent; the host re-uploads it before the next run
-  }
-  const int n_initial = g->n_initial;
-  for (int i = threadIdx.x; i < n_initial; i += kBlock)
-    __hip_atomic_store(&slots[i], g->initial[i], __ATOMIC_RELAXED, AGENT);
   if (threadIdx.x == 0) {
-    __hip_atomic_store(&g->completed, __hip_atomic_load(&g->done_count, __ATOMIC_RELAXED, AGENT),
-                       __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&g->done_count, 0u, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&g->exit_count, 0u, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&q->head_, 0, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&q->tail_, n_initial, __ATOMIC_RELAXED, AGENT);
+    const bool aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0;
+    unsigned int done = 0;
+    for (int q = 0; q < kQueues; ++q) {
+      done += __hip_atomic_load(&hot[kHotDone + q].value, __ATOMIC_RELAXED, AGENT);
+      // after an abort the per-op state is inconsistent: leave it for the host to restore
+      if (!aborted) {
+        __hip_atomic_store(&hot[kHotDone + q].value, 0u, __ATOMIC_RELAXED, AGENT);
+        __hip_atomic_store(g.queue_head[q], 0, __ATOMIC_RELAXED, AGENT);
+      }
+    }
+    __hip_atomic_store(&hot[kHotCompleted].value, done, __ATOMIC_RELAXED, AGENT);
+    __hip_atomic_store(&hot[kHotExit].value, 0u, __ATOMIC_RELAXED, AGENT);
   }
 }
 
-typedef void (*DrainKernel)(GraphControl *);
+typedef void (*DrainKernel)(const GraphControl);
 
 template <int DT>
 DrainKernel drain_for_compute(int compute) {
@@ -290,8 +330,6 @@ struct Graph {
   DrainKernel kernel = nullptr;
   std::mutex mu;
 };
-
-constexpr size_t kPayloadStride = 256;  // sizeof(pccl_op_payload) == 248, padded
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -371,6 +409,8 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
       const int u = ops[i].deps[d];
       succ[succ_start[u] + fill[u]++] = i;
     }
+  // level[i] = length of the longest dependency chain ending in op i
+  std::vector<int> level(n_ops, 0);
   {
     std::vector<int> indeg(n_pred), stack;
     for (int i = 0; i < n_ops; ++i) if (!indeg[i]) stack.push_back(i);
@@ -379,11 +419,18 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
       const int u = stack.back();
       stack.pop_back();
       ++seen;
-      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e)
-        if (--indeg[succ[e]] == 0) stack.push_back(succ[e]);
+      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) {
+        const int v = succ[e];
+        level[v] = std::max(level[v], level[u] + 1);
+        if (--indeg[v] == 0) stack.push_back(v);
+      }
     }
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
   }
+  // global order of the entries: by level, then op id, then part
+  std::vector<int> by_level(n_ops);
+  for (int i = 0; i < n_ops; ++i) by_level[i] = i;
+  std::stable_sort(by_level.begin(), by_level.end(), [&](int a, int b) { return level[a] < level[b]; });
 
   // ---- arena layout ----------------------------------------------------------
   size_t off = align_up(sizeof(GraphControl), 256);
@@ -391,10 +438,10 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   const size_t off_hdr = off;     off = align_up(off + sizeof(pccl_operation_layout_header) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_payload = off; off = align_up(off + kPayloadStride * (size_t)std::max(n_ops, 1), 256);
   const size_t off_succ = off;    off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
-  const size_t off_ring = off;    off = align_up(off + sizeof(pccl_ring_buffer), 256);
-  const size_t off_qptr = off;    off = align_up(off + sizeof(void *), 256);
-  const size_t off_slots = off;   off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1), 256);
-  const size_t off_init = off;    off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1), 256);
+  const size_t off_hot = off;     off = align_up(off + sizeof(HotWord) * kHotWords, 256);
+  const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
+  const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
+  const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
   const size_t arena_bytes = off;
 
   Graph *G = new Graph();
@@ -414,34 +461,53 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   char *dev = G->dev;
 
   GraphControl *C = (GraphControl *)img;
-  C->layout.completed_operator = (unsigned int *)(dev + offsetof(GraphControl, completed));
-  C->layout.total_operator = (unsigned int *)(dev + offsetof(GraphControl, total));
+  HotWord *hot = (HotWord *)(img + off_hot);
+  C->hot = (HotWord *)(dev + off_hot);
+  C->layout.completed_operator = &((HotWord *)(dev + off_hot))[kHotCompleted].value;
+  C->layout.total_operator = &((HotWord *)(dev + off_hot))[kHotTotal].value;
   C->layout.operators = (pccl_operation_layout_header **)(dev + off_opptr);
   C->layout.num_operators = (unsigned int)n_ops;
   C->layout.ready_queues = (pccl_ring_buffer **)(dev + off_qptr);
-  C->layout.num_queues = 1;
+  C->layout.num_queues = kQueues;
   C->headers = (pccl_operation_layout_header *)(dev + off_hdr);
-  C->slots = (unsigned long long *)(dev + off_slots);
-  C->initial = (const unsigned long long *)(dev + off_init);
-  C->completed = 0;
-  C->total = (unsigned int)n_ops;
+  C->slots = dev + off_payload;
+  C->succ = (const int *)(dev + off_succ);
   C->spin_limit = kDefaultSpinLimit;
   C->total_tiles = (int)tiles;
+  hot[kHotCompleted].value = 0;
+  hot[kHotTotal].value = (unsigned int)n_ops;
 
-  *(pccl_ring_buffer **)(img + off_qptr) = (pccl_ring_buffer *)(dev + off_ring);
-  pccl_ring_buffer *R = (pccl_ring_buffer *)(img + off_ring);
-  R->producer_ = 0;  // executor ids are the host layer's; one executor produces and consumes
-  R->consumer_ = 0;
-  R->elem_size_ = (int)sizeof(pccl_queue_entry);
-  R->max_num_elems_ = (int)std::max<long long>(tiles, 1);
-  R->max_flush_time_ = 0;  // producer and consumer share one address space: nothing to flush
-  R->producer_buffer_ = dev + off_slots;
-  R->consumer_buffer_ = dev + off_slots;
-
-  unsigned long long *slots = (unsigned long long *)(img + off_slots);
-  unsigned long long *initial = (unsigned long long *)(img + off_init);
-  for (long long t = 0; t < std::max<long long>(tiles, 1); ++t) slots[t] = kEmptySlot;
-  int n_initial = 0;
+  // deal the entries round-robin onto the queues, in global order
+  std::vector<std::vector<unsigned long long>> qe(kQueues);
+  {
+    long long t = 0;
+    for (int idx = 0; idx < n_ops; ++idx) {
+      const int i = by_level[idx];
+      for (int p = 0; p < parts[i]; ++p, ++t)
+        qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32));
+    }
+  }
+  {
+    size_t pos = off_entries;
+    for (int q = 0; q < kQueues; ++q) {
+      ((pccl_ring_buffer **)(img + off_qptr))[q] = (pccl_ring_buffer *)(dev + off_ring + 256 * (size_t)q);
+      pccl_ring_buffer *R = (pccl_ring_buffer *)(img + off_ring + 256 * (size_t)q);
+      C->queue_head[q] = &((pccl_ring_buffer *)(dev + off_ring + 256 * (size_t)q))->head_;
+      C->queue_entries[q] = (const unsigned long long *)(dev + pos);
+      C->queue_count[q] = (int)qe[q].size();
+      R->producer_ = 0;  // executor ids are the host layer's; one executor fills and drains
+      R->consumer_ = 0;
+      R->elem_size_ = (int)sizeof(pccl_queue_entry);
+      R->max_num_elems_ = (int)qe[q].size();
+      R->max_flush_time_ = 0;  // producer and consumer share one address space: nothing to flush
+      R->tail_ = (int)qe[q].size();
+      R->head_ = 0;
+      R->producer_buffer_ = dev + pos;
+      R->consumer_buffer_ = dev + pos;
+      if (!qe[q].empty()) memcpy(img + pos, qe[q].data(), 8 * qe[q].size());
+      pos += 8 * qe[q].size();
+    }
+  }
 
   for (int i = 0; i < n_ops; ++i) {
     const pccl_op_desc &o = ops[i];
@@ -457,7 +523,10 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     h->num_next_ops_ = (unsigned char)n_succ[i];
     h->op_buffer_ = dev + off_payload + kPayloadStride * (size_t)i;
     h->next_op_uids_head_ = (int *)(dev + off_succ) + succ_start[i];
-    pccl_op_payload *pl = (pccl_op_payload *)(img + off_payload + kPayloadStride * (size_t)i);
+    PayloadSlot *slot = (PayloadSlot *)(img + off_payload + kPayloadStride * (size_t)i);
+    slot->parts = parts[i];
+    slot->succ_start = succ_start[i];
+    pccl_op_payload *pl = &slot->payload;
     pl->primitive_ = o.primitive;
     pl->compute_ = o.compute;
     pl->n_in_ = o.n_in;
@@ -465,16 +534,8 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     memcpy(&pl->initial_word12_, (char *)h + 12, 4);
     for (int k = 0; k < o.n_in; ++k) pl->chunks_[k] = pccl_chunk_meta{o.dtype, (void *)o.ins[k], o.count};
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
-    if (n_pred[i] == 0)
-      for (int p = 0; p < parts[i]; ++p)
-        initial[n_initial++] = (unsigned long long)(unsigned int)i | ((unsigned long long)p << 32);
   }
   if (n_edges) memcpy(img + off_succ, succ.data(), sizeof(int) * n_edges);
-  for (int t = 0; t < n_initial; ++t) slots[t] = initial[t];
-  R->head_ = 0;
-  R->tail_ = n_initial;
-  C->n_initial = n_initial;
-
   // launch width: enough workgroups to fill the chip, never more than entries
   int occ = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)G->kernel, kBlock, 0) != hipSuccess || occ < 1) {
@@ -500,7 +561,12 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_run: graph is null");
   if (G->total_tiles == 0) return PCCL_OK;
-  hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, (GraphControl *)G->dev);
+  GraphControl control;
+  {
+    std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
+    memcpy(&control, G->image.data(), sizeof(control));
+  }
+  hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run launch failed: %s", hipGetErrorString(e));
   return PCCL_OK;
@@ -511,16 +577,18 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed, un
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_status: graph is null");
   PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
-  GraphControl c;
-  PCCL_HIP_CHECK(hipMemcpy(&c, G->dev, sizeof(c), hipMemcpyDeviceToHost));
-  if (completed) *completed = c.completed;
-  if (total) *total = c.total;
-  if (c.abort) {
+  const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
+  HotWord hot[kHotWords];
+  PCCL_HIP_CHECK(hipMemcpy(hot, G->dev + off_hot, sizeof(hot), hipMemcpyDeviceToHost));
+  if (completed) *completed = hot[kHotCompleted].value;
+  if (total) *total = hot[kHotTotal].value;
+  if (hot[kHotAbort].value) {
     // put the pristine state back so that the graph can be used again
     std::lock_guard<std::mutex> lock(G->mu);
     PCCL_HIP_CHECK(hipMemcpy(G->dev, G->image.data(), G->image.size(), hipMemcpyHostToDevice));
-    return fail(PCCL_ERR_GRAPH, "drain gave up: a queue slot was not published within the spin limit "
-                                "(%u of %u ops had completed); graph state was reset", c.completed, c.total);
+    return fail(PCCL_ERR_GRAPH, "drain gave up: an op's dependencies were not satisfied within the spin limit "
+                                "(%u of %u ops had completed); graph state was reset",
+                hot[kHotCompleted].value, hot[kHotTotal].value);
   }
   return PCCL_OK;
 }
