@@ -194,6 +194,16 @@ def main():
         assert torch.equal(o, a + b)
         extras["f32_2in_1out_4MiB"] = stats(t)
 
+        # ---- unaligned operands: i32 4 -> 1, 2^28-57 elements, every buffer 4..60 bytes off 64 ----
+        cu = (1 << 28) - 57
+        pool = [torch.randint(-(1 << 20), 1 << 20, (cu + 64,), dtype=torch.int32, device="cuda") for _ in range(4)]
+        ou = torch.empty(cu + 64, dtype=torch.int32, device="cuda")
+        offs = [4, 12, 20, 60, 8]
+        ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
+        t = event_times_us(torch, lambda: hip.reduce_copy("i32", "sum", ptr_in, [ou.data_ptr() + offs[4]], cu, stream), 10, 2)
+        extras["unaligned_i32_4in_1out_1GiB"] = dict(stats(t), GBps_median=gbps(5 * 4 * cu, t[len(t) // 2]), byte_offsets=offs)
+        del pool, ou
+
         # ---- small ops: 64 KiB direct launch and through the queue --------------------------
         n64 = 32768
         x, y = randn(torch, n64, "bf16"), randn(torch, n64, "bf16")

@@ -70,6 +70,7 @@ int pccl_device_ipc_available(const char *device_name, int *yes);
 /* ---- launch options: include/common/environ.h:11-37, python_api.cc:24-27 ------------- */
 int pccl_env_list_opt(char *buf, int buf_len);                   /* '\n'-separated */
 int pccl_env_get(const char *name, char *buf, int buf_len);
+int pccl_env_register_opt(const char *name);                     /* registerOpt */
 
 /* ---- schedule generators (native side of pccl/lang) ---------------------------------- */
 /* Each writes a schedule file that pccl_engine_reg_op loads. */

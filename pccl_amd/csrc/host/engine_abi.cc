@@ -232,6 +232,11 @@ int pccl_env_get(const char *name, char *buf, int buf_len) {
   return guarded([&] { copy_out(utils::LaunchEnvironments::getEnv(name), buf, buf_len); });
 }
 
+int pccl_env_register_opt(const char *name) {
+  if (!name) return bad_arg("name is null");
+  return guarded([&] { utils::LaunchEnvironments::registerOpt(name); });
+}
+
 int pccl_schedule_write_ring_allreduce(const char *path, const char *dtype, const char *compute, int devices,
                                        long chunk_elems) {
   if (!path || !dtype || !compute) return bad_arg("null argument");

@@ -55,6 +55,7 @@ def lib():
             "pccl_device_ipc_available": [cs, P(ci)],
             "pccl_env_list_opt": [cs, ci],
             "pccl_env_get": [cs, cs, ci],
+            "pccl_env_register_opt": [cs],
             "pccl_schedule_write_ring_allreduce": [cs, cs, cs, ci, cl],
             "pccl_schedule_write_direct_allreduce": [cs, cs, cs, ci, cl],
             "pccl_schedule_write_small_message": [cs, cs, ci, ci, ci, ctypes.c_ulong, cl, cl],
@@ -218,6 +219,10 @@ class LaunchEnvironments:
         buf = ctypes.create_string_buffer(4096)
         _check(lib().pccl_env_list_opt(buf, 4096))
         return [x for x in buf.value.decode().split("\n") if x]
+
+    @staticmethod
+    def registerOpt(name):
+        _check(lib().pccl_env_register_opt(_b(name)))
 
     @staticmethod
     def getEnv(name):

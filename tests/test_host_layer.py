@@ -107,6 +107,11 @@ def test_cpu_plugin_allocator(E):
 
 def test_launch_options_listed(E):
     assert {"PCCL_HIP_WG_PER_CU", "PCCL_HIP_NT", "PCCL_HIP_TILE_BYTES"} <= set(E.LaunchEnvironments.listOpt())
+    E.LaunchEnvironments.registerOpt("PCCL_TEST_OPTION")
+    E.LaunchEnvironments.registerOpt("PCCL_TEST_OPTION")
+    assert E.LaunchEnvironments.listOpt().count("PCCL_TEST_OPTION") == 1
+    from pccl_amd import engine_c  # module layout of csrc/python_api.cc
+    assert engine_c.Engine is E.Engine and engine_c.utils.LaunchEnvironments.listOpt() == E.LaunchEnvironments.listOpt()
     assert E.LaunchEnvironments.getEnv("PCCL_SURELY_UNSET_VARIABLE") == ""
     assert E.LaunchEnvironments.getEnv("PATH") == os.environ["PATH"]
 
