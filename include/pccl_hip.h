@@ -99,10 +99,18 @@ int pccl_hip_set_occupancy_lds(int lds_bytes);
 /* ---- the op-batching path: a DAG of ops drained by one persistent kernel -- */
 
 /* One IR operation as the host hands it over: the C++ payload level of
- * PrimitiveOp (pccl/lang/chunk.py:46-55): op kind, operands, dependencies. */
+ * PrimitiveOp (pccl/lang/chunk.py:46-55): op kind, operands, dependencies.
+ * Signal ops (chunk.py:9-10; signal words like the int slots of csrc/engine.cc:16-18):
+ *   NOTIFY        n_in 0, n_out 1: outs[0] = address of a 32-bit signal word, count =
+ *                 value (0..65535); once its dependencies are complete it stores
+ *                 signal_base + value to the word (system scope);
+ *   GET_NOTIFIED  n_in 1, n_out 0: ins[0] = signal word, count = value; it completes
+ *                 when (int)(word - (signal_base + value)) >= 0 (bounded wait).
+ * signal_base = run number << 16 (pccl_hip_graph_next_signal_base), so a word left over
+ * from an earlier run never satisfies a wait of a later one. */
 typedef struct pccl_op_desc {
   int op_uid;                          /* dense 0..n_ops-1, chunk.py:82-83           */
-  unsigned char primitive;             /* enum pccl_primitive (COPY or REDUCE)        */
+  unsigned char primitive;             /* enum pccl_primitive                         */
   unsigned char dtype;                 /* enum pccl_dtype                             */
   unsigned char compute;               /* enum pccl_compute                           */
   unsigned char n_in;                  /* 1..8                                        */
@@ -140,6 +148,10 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
 
 /* Device address of the GraphBufferLayout and launch facts, for inspection. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
+
+/* signal_base the NEXT pccl_hip_graph_run of this graph will use: a party outside the
+ * graph that wants to satisfy a GET_NOTIFIED(value) stores *base + value to the word. */
+int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
 
 /* Bounds every wait inside the drain kernel to `polls` polls of a queue slot
  * (default about 2 million, a few seconds).  When a wait gives up the kernel

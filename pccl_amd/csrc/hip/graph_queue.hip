@@ -82,6 +82,7 @@ struct GraphControl {
   int queue_count[kQueues];
   unsigned int spin_limit;
   int total_tiles;
+  unsigned int signal_base;               // run number << 16: added to the value of NOTIFY / GET_NOTIFIED ops
 };
 
 // indices into GraphControl::hot
@@ -167,7 +168,14 @@ template <int DT, class Op>
 __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, long count) {
   typedef Dtype<DT> D;
   switch (pl->n_in_) {
-    case 1: run_part_nin<D, Op, 1>(pl, lo, count); break;
+    case 1: {
+      // COPY moves bytes, and its element size is its own, not that of the graph's
+      // REDUCE ops: run it as a copy of 2-byte units
+      const int dt = pl->chunks_[0].dtype_;
+      const long units = (dt == PCCL_F32 || dt == PCCL_I32) ? 2 : 1;
+      run_part_nin<Dtype<PCCL_BF16>, OpSum, 1>(pl, lo * units, count * units);
+      break;
+    }
     case 2: run_part_nin<D, Op, 2>(pl, lo, count); break;
     case 3: run_part_nin<D, Op, 3>(pl, lo, count); break;
     case 4: run_part_nin<D, Op, 4>(pl, lo, count); break;
@@ -179,6 +187,40 @@ __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, lon
 }
 
 #define AGENT __HIP_MEMORY_SCOPE_AGENT
+
+// Polls `ready` until it holds.  Gives up (and raises the abort word, so that every
+// workgroup leaves) after spin_limit polls or when another workgroup has given up.
+template <class Ready>
+__device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned int spin_limit, Ready ready) {
+  unsigned int spins = 0;
+  while (!ready()) {
+    __builtin_amdgcn_s_sleep(1);
+    if ((++spins & 63u) == 0 &&
+        (spins >= spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0)) {
+      __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
+      return false;
+    }
+  }
+  return true;
+}
+
+// Thread 0, after a part of op `h` is complete: count it; the op's last part re-arms
+// the op's counters for the next run and releases its successors.
+__device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
+                                            const PayloadSlot *slot, int home) {
+  const int parts = slot->parts;
+  int old = 1;
+  if (parts > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
+  if (old != 1) return;
+  if (parts > 1) __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
+  const unsigned int w12 = slot->payload.initial_word12_;
+  if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);
+  const int n_next = (int)(w12 >> 24);
+  const int *next = g.succ + slot->succ_start;
+  for (int s = 0; s < n_next; ++s)
+    __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
+  __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
+}
 
 template <int DT, class Op>
 __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
@@ -201,28 +243,18 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   for (;;) {
     if (threadIdx.x == 0) {
-      if (h) {
-        // The part executed in the previous iteration is complete (barrier below):
-        // every wavefront waited for its write-through stores before that barrier, so
-        // the data is at the point of coherence and relaxed device-scope atomics are
-        // enough to hand it over; no L2 write-back / invalidate is involved.
-        const int parts = slot->parts;
-        int old = 1;
-        if (parts > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
-        if (old == 1) {  // it was the op's last part
-          if (parts > 1) __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
-          const unsigned int w12 = slot->payload.initial_word12_;
-          if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);  // re-arm its own count
-          const int n_next = (int)(w12 >> 24);
-          const int *next = g.succ + slot->succ_start;
-          for (int s = 0; s < n_next; ++s)
-            __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
-          __hip_atomic_fetch_add(&hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
-        }
-      }
+      // The part executed in the previous iteration is complete (barrier below): every
+      // wavefront waited for its write-through stores before that barrier, so the data is
+      // at the point of coherence and relaxed device-scope atomics are enough to hand it
+      // over; no L2 write-back / invalidate is involved.
+      if (h) finish_part(g, h, slot, home);
       int go = 0;
       unsigned long long e = 0;
-      if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) == 0) {
+      // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
+      // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
+      for (;;) {
+        go = 0;
+        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0) break;
         for (int i = 0; i < kQueues && !go; ++i) {
           const int q = (home + i) % kQueues;
           if (exhausted & (1u << q)) continue;
@@ -236,19 +268,31 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
             exhausted |= 1u << q;
           }
         }
-      }
-      if (go) {  // wait for the op's dependencies
-        unsigned int *dep = word12(&g.headers[(int)(e & 0xffffffffu)]);
-        unsigned int spins = 0;
-        while ((__hip_atomic_load(dep, __ATOMIC_RELAXED, AGENT) & 0xffu) != 0) {
-          __builtin_amdgcn_s_sleep(1);
-          if ((++spins & 63u) == 0 &&
-              (spins >= spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0)) {
-            __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
-            go = 0;
-            break;
-          }
+        if (!go) break;
+        const int uid = (int)(e & 0xffffffffu);
+        pccl_operation_layout_header *hc = &g.headers[uid];
+        // wait for the op's dependencies
+        if (!bounded_wait(abort_flag, spin_limit, [&] {
+              return (__hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT) & 0xffu) == 0;
+            })) {
+          go = 0;
+          break;
         }
+        const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
+        const int prim = sc->payload.primitive_;
+        if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
+        unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
+        const unsigned int want = g.signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
+        if (prim == PCCL_NOTIFY) {
+          // everything this op depends on is already at the point of coherence
+          __hip_atomic_store(sig, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        } else if (!bounded_wait(abort_flag, spin_limit, [&] {
+                     return (int)(__hip_atomic_load(sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
+                   })) {
+          go = 0;
+          break;
+        }
+        finish_part(g, hc, sc, home);
       }
       s_entry = e;
       s_go = go;
@@ -327,6 +371,7 @@ struct Graph {
   int total_tiles = 0;
   int n_wg = 0;
   int device = 0;
+  unsigned int runs = 0;        // launches so far; run r uses signal values (r << 16) + value
   DrainKernel kernel = nullptr;
   std::mutex mu;
 };
@@ -350,35 +395,50 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
 
   // ---- validate; one (dtype, compute) pair for all REDUCE ops --------------
   int g_dtype = -1, g_compute = -1;
-  std::vector<int> n_succ(n_ops, 0), n_pred(n_ops, 0), parts(n_ops, 1);
+  std::vector<int> n_succ(n_ops, 0), n_pred(n_ops, 0), parts(n_ops, 1), signal_ops;
   size_t n_edges = 0;
   long long tiles = 0;
   for (int i = 0; i < n_ops; ++i) {
     const pccl_op_desc &o = ops[i];
     if (o.op_uid != i) return fail(PCCL_ERR_GRAPH, "op %d: op_uid %d is not its index (uids are dense from 0)", i, o.op_uid);
-    if (o.primitive != PCCL_COPY && o.primitive != PCCL_REDUCE)
-      return fail(PCCL_ERR_UNSUPPORTED, "op %d: primitive %d is not COPY or REDUCE", i, o.primitive);
-    if (o.dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown dtype code %d", i, o.dtype);
-    if (o.compute > PCCL_MAX) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown compute code %d", i, o.compute);
-    if (o.n_in < 1 || o.n_in > PCCL_MAX_INPUTS || o.n_out < 1 || o.n_out > PCCL_MAX_OUTPUTS ||
-        o.n_in + o.n_out > PCCL_MAX_OP_CHUNKS)
-      return fail(PCCL_ERR_INVALID_ARG, "op %d: n_in %d / n_out %d (each 1..8, at most 10 operands in all)", i, o.n_in, o.n_out);
-    if (o.primitive == PCCL_COPY && o.n_in != 1)
-      return fail(PCCL_ERR_INVALID_ARG, "op %d: COPY takes exactly one input", i);
-    if (o.count < 0) return fail(PCCL_ERR_INVALID_ARG, "op %d: count %ld < 0", i, o.count);
-    const int es = elem_bytes(o.dtype);
-    for (int k = 0; k < o.n_in; ++k) {
-      if (!o.ins[k] && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: input %d is null", i, k);
-      if ((uintptr_t)o.ins[k] % es) return fail(PCCL_ERR_MISALIGNED, "op %d: input %d not %d-byte aligned", i, k, es);
-    }
-    for (int k = 0; k < o.n_out; ++k) {
-      if (!o.outs[k] && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: output %d is null", i, k);
-      if ((uintptr_t)o.outs[k] % es) return fail(PCCL_ERR_MISALIGNED, "op %d: output %d not %d-byte aligned", i, k, es);
-    }
-    if (o.n_in > 1) {
-      if (g_dtype < 0) { g_dtype = o.dtype; g_compute = o.compute; }
-      else if (g_dtype != o.dtype || g_compute != o.compute)
-        return fail(PCCL_ERR_UNSUPPORTED, "op %d: a graph holds REDUCE ops of one (dtype, compute) pair only", i);
+    if (o.primitive > PCCL_GET_NOTIFIED)
+      return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown primitive code %d", i, o.primitive);
+    const bool is_signal = o.primitive == PCCL_NOTIFY || o.primitive == PCCL_GET_NOTIFIED;
+    int es = 1;
+    if (is_signal) {
+      // NOTIFY: outs[0] is the signal word, GET_NOTIFIED: ins[0]; count is the value
+      const bool notify = o.primitive == PCCL_NOTIFY;
+      if (o.n_in != (notify ? 0 : 1) || o.n_out != (notify ? 1 : 0))
+        return fail(PCCL_ERR_INVALID_ARG, "op %d: NOTIFY takes 0 inputs / 1 output, GET_NOTIFIED 1 input / 0 outputs", i);
+      const void *sig = notify ? (const void *)o.outs[0] : o.ins[0];
+      if (!sig) return fail(PCCL_ERR_INVALID_ARG, "op %d: signal address is null", i);
+      if ((uintptr_t)sig % 4) return fail(PCCL_ERR_MISALIGNED, "op %d: signal address not 4-byte aligned", i);
+      if (o.count < 0 || o.count > 0xffff)
+        return fail(PCCL_ERR_INVALID_ARG, "op %d: signal value %ld outside [0, 65535]", i, o.count);
+      signal_ops.push_back(i);
+    } else {
+      if (o.dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown dtype code %d", i, o.dtype);
+      if (o.compute > PCCL_MAX) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown compute code %d", i, o.compute);
+      if (o.n_in < 1 || o.n_in > PCCL_MAX_INPUTS || o.n_out < 1 || o.n_out > PCCL_MAX_OUTPUTS ||
+          o.n_in + o.n_out > PCCL_MAX_OP_CHUNKS)
+        return fail(PCCL_ERR_INVALID_ARG, "op %d: n_in %d / n_out %d (each 1..8, at most 10 operands in all)", i, o.n_in, o.n_out);
+      if (o.primitive == PCCL_COPY && o.n_in != 1)
+        return fail(PCCL_ERR_INVALID_ARG, "op %d: COPY takes exactly one input", i);
+      if (o.count < 0) return fail(PCCL_ERR_INVALID_ARG, "op %d: count %ld < 0", i, o.count);
+      es = elem_bytes(o.dtype);
+      for (int k = 0; k < o.n_in; ++k) {
+        if (!o.ins[k] && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: input %d is null", i, k);
+        if ((uintptr_t)o.ins[k] % es) return fail(PCCL_ERR_MISALIGNED, "op %d: input %d not %d-byte aligned", i, k, es);
+      }
+      for (int k = 0; k < o.n_out; ++k) {
+        if (!o.outs[k] && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: output %d is null", i, k);
+        if ((uintptr_t)o.outs[k] % es) return fail(PCCL_ERR_MISALIGNED, "op %d: output %d not %d-byte aligned", i, k, es);
+      }
+      if (o.n_in > 1) {
+        if (g_dtype < 0) { g_dtype = o.dtype; g_compute = o.compute; }
+        else if (g_dtype != o.dtype || g_compute != o.compute)
+          return fail(PCCL_ERR_UNSUPPORTED, "op %d: a graph holds REDUCE ops of one (dtype, compute) pair only", i);
+      }
     }
     if (o.n_deps < 0 || (o.n_deps > 0 && !o.deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
     if (o.n_deps > 255) return fail(PCCL_ERR_GRAPH, "op %d: %d dependencies exceed pre_dependencies_ (unsigned char)", i, o.n_deps);
@@ -389,7 +449,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     }
     n_pred[i] = o.n_deps;
     n_edges += (size_t)o.n_deps;
-    const long bytes = o.count * es;
+    const long bytes = is_signal ? 0 : o.count * es;
     long p = (bytes + tile_bytes - 1) / tile_bytes;
     parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
     tiles += parts[i];
@@ -409,21 +469,39 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
       const int u = ops[i].deps[d];
       succ[succ_start[u] + fill[u]++] = i;
     }
+  // A GET_NOTIFIED must not be claimed ahead of the NOTIFY that satisfies it (same signal
+  // word, same value, same graph), or workgroups could fill up with waits nobody can end.
+  // Such pairs are ordering edges: they count for levels and cycles, not for
+  // pre_dependencies_ (the hand-over itself goes through the signal word).
+  std::vector<std::vector<int>> order_succ(n_ops);
+  std::vector<int> order_pred(n_ops, 0);
+  for (int a : signal_ops) {
+    if (ops[a].primitive != PCCL_NOTIFY) continue;
+    for (int b : signal_ops)
+      if (ops[b].primitive == PCCL_GET_NOTIFIED && ops[b].ins[0] == ops[a].outs[0] && ops[b].count == ops[a].count) {
+        order_succ[a].push_back(b);
+        ++order_pred[b];
+      }
+  }
   // level[i] = length of the longest dependency chain ending in op i
   std::vector<int> level(n_ops, 0);
   {
-    std::vector<int> indeg(n_pred), stack;
-    for (int i = 0; i < n_ops; ++i) if (!indeg[i]) stack.push_back(i);
+    std::vector<int> indeg(n_ops), stack;
+    for (int i = 0; i < n_ops; ++i) {
+      indeg[i] = n_pred[i] + order_pred[i];
+      if (!indeg[i]) stack.push_back(i);
+    }
     int seen = 0;
+    auto relax = [&](int u, int v) {
+      level[v] = std::max(level[v], level[u] + 1);
+      if (--indeg[v] == 0) stack.push_back(v);
+    };
     while (!stack.empty()) {
       const int u = stack.back();
       stack.pop_back();
       ++seen;
-      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) {
-        const int v = succ[e];
-        level[v] = std::max(level[v], level[u] + 1);
-        if (--indeg[v] == 0) stack.push_back(v);
-      }
+      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) relax(u, succ[e]);
+      for (int v : order_succ[u]) relax(u, v);
     }
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
   }
@@ -532,6 +610,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     pl->n_in_ = o.n_in;
     pl->n_out_ = o.n_out;
     memcpy(&pl->initial_word12_, (char *)h + 12, 4);
+    // signal ops: the only operand is the signal word, num_elems_ carries the value
     for (int k = 0; k < o.n_in; ++k) pl->chunks_[k] = pccl_chunk_meta{o.dtype, (void *)o.ins[k], o.count};
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
   }
@@ -565,6 +644,8 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   {
     std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
     memcpy(&control, G->image.data(), sizeof(control));
+    control.signal_base = (G->runs + 1u) << 16;
+    ++G->runs;
   }
   hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
   hipError_t e = hipGetLastError();
@@ -626,6 +707,15 @@ int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_
   if (device_layout) *device_layout = G->dev;
   if (n_tiles) *n_tiles = G->total_tiles;
   if (n_workgroups) *n_workgroups = G->n_wg;
+  return PCCL_OK;
+}
+
+int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base) {
+  pccl_host::clear_error();
+  Graph *G = (Graph *)graph;
+  if (!G || !base) return fail(PCCL_ERR_INVALID_ARG, "graph_next_signal_base: null argument");
+  std::lock_guard<std::mutex> lock(G->mu);
+  *base = (G->runs + 1u) << 16;
   return PCCL_OK;
 }
 

@@ -75,6 +75,8 @@ def lib():
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.pccl_hip_graph_next_signal_base.argtypes = [vp, ctypes.POINTER(ctypes.c_uint)]
+        L.pccl_hip_graph_set_spin_limit.argtypes = [vp, ctypes.c_uint]
         L.pccl_hip_graph_destroy.argtypes = [vp]
         for name in ("pccl_hip_last_error", "pccl_hip_version"):
             getattr(L, name).restype = ctypes.c_char_p
@@ -153,16 +155,24 @@ class Graph:
         for i, o in enumerate(ops):
             d = arr[i]
             d.op_uid = i
-            n_in, n_out = len(o["ins"]), len(o["outs"])
-            d.primitive = o.get("primitive", COPY if n_in == 1 else REDUCE)
-            d.dtype = _code(DTYPES, o["dtype"])
-            d.compute = _code(COMPUTES, o.get("compute", "sum"))
-            d.n_in, d.n_out = n_in, n_out
-            for k in range(min(n_in, MAX_INPUTS)):
-                d.ins[k] = _addr(o["ins"][k])
-            for k in range(min(n_out, MAX_OUTPUTS)):
-                d.outs[k] = _addr(o["outs"][k])
-            d.count = o["count"]
+            prim = o.get("primitive")
+            if prim in (NOTIFY, GET_NOTIFIED):
+                # signal op: "signal" = address of the 32-bit word, "value" = 0..65535
+                d.primitive = prim
+                d.n_in, d.n_out = (0, 1) if prim == NOTIFY else (1, 0)
+                (d.outs if prim == NOTIFY else d.ins)[0] = _addr(o["signal"])
+                d.count = o["value"]
+            else:
+                n_in, n_out = len(o["ins"]), len(o["outs"])
+                d.primitive = prim if prim is not None else (COPY if n_in == 1 else REDUCE)
+                d.dtype = _code(DTYPES, o["dtype"])
+                d.compute = _code(COMPUTES, o.get("compute", "sum"))
+                d.n_in, d.n_out = n_in, n_out
+                for k in range(min(n_in, MAX_INPUTS)):
+                    d.ins[k] = _addr(o["ins"][k])
+                for k in range(min(n_out, MAX_OUTPUTS)):
+                    d.outs[k] = _addr(o["outs"][k])
+                d.count = o["count"]
             deps = list(o.get("deps", ()))
             d.n_deps = len(deps)
             buf = (ctypes.c_int * max(len(deps), 1))(*deps)
@@ -182,6 +192,14 @@ class Graph:
     def rebind(self, old_base, new_base, nbytes, stream=None):
         _check(lib().pccl_hip_graph_rebind(self._h, ctypes.c_void_p(_addr(old_base)), ctypes.c_void_p(_addr(new_base)),
                                            nbytes, ctypes.c_void_p(_addr(stream))))
+
+    def next_signal_base(self):
+        b = ctypes.c_uint(0)
+        _check(lib().pccl_hip_graph_next_signal_base(self._h, ctypes.byref(b)))
+        return b.value
+
+    def set_spin_limit(self, polls):
+        _check(lib().pccl_hip_graph_set_spin_limit(self._h, polls))
 
     def info(self):
         lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)

@@ -170,8 +170,8 @@ def test_graph_errors(hip):
     with pytest.raises(hip.PcclError) as e:  # two (dtype, compute) pairs
         hip.Graph([op, dict(op, compute="max")])
     assert e.value.code == hip.ERR_UNSUPPORTED
-    with pytest.raises(hip.PcclError) as e:  # NOTIFY is not executable here
-        hip.Graph([dict(op, primitive=hip.NOTIFY)])
+    with pytest.raises(hip.PcclError) as e:  # unknown primitive code
+        hip.Graph([dict(op, primitive=9)])
     assert e.value.code == hip.ERR_UNSUPPORTED
     with pytest.raises(hip.PcclError) as e:
         hip.Graph([dict(op, ins=[t.data_ptr() + 1, t])])
@@ -194,9 +194,7 @@ def test_bounded_wait_aborts_cleanly(hip, oracle):
     ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
            dict(dtype="f32", compute="sum", ins=[dt.ptr, db.ptr], outs=[du.ptr], count=count, deps=[0])]
     g = hip.Graph(ops)
-    L = hip.lib()
-    L.pccl_hip_graph_set_spin_limit.argtypes = [ctypes.c_void_p, ctypes.c_uint]
-    assert L.pccl_hip_graph_set_spin_limit(g._h, 256) == 0
+    g.set_spin_limit(256)
     # GraphBufferLayout.operators (offset 16) -> headers; op 1's byte 12 is pre_dependencies_
     lay = g.info()["device_layout"]
     host = torch.empty(48, dtype=torch.uint8)
@@ -215,7 +213,164 @@ def test_bounded_wait_aborts_cleanly(hip, oracle):
         g.status(_stream(torch))
     assert e.value.code == hip.ERR_GRAPH
     # status restored the pristine graph: it runs correctly now
-    assert L.pccl_hip_graph_set_spin_limit(g._h, 1 << 21) == 0
+    g.set_spin_limit(1 << 21)
     _run_and_check(torch, hip, g, 2)
     H.assert_bits_equal(du.download(), oracle.reduce("f32", "sum", [oracle.reduce("f32", "sum", [a, b]), b]), "after reset")
     g.destroy()
+
+
+# ---- signal ops: NOTIFY / GET_NOTIFIED ---------------------------------------------------------
+
+def _signal_ring_ops(world, size, signals_ptr, dev_in, dev_out, es=2, dtype="bf16"):
+    """Ring all-reduce written the way ranks on different GPUs would have to write it: DAG edges
+    only inside a rank; the hand-over between ranks goes NOTIFY (producer rank) -> signal word ->
+    GET_NOTIFIED (consumer rank).  Signal word of link p -> r: slot r; value: the step number.
+    Returns (ops, data_ops) where data_ops maps op index -> symbolic op for the CPU replay."""
+    ops, sym = [], {}
+    last_of_rank = {}           # rank -> its latest op (program order inside a rank)
+    notify_of = {}              # (rank, step) -> index of the NOTIFY that publishes that step's output
+
+    def add(op):
+        ops.append(op)
+        return len(ops) - 1
+
+    for step in range(1, 2 * world - 1):
+        reduce_phase = step < world
+        for r in range(world):
+            p = (r - 1) % world
+            c = (r - step) % world if reduce_phase else (r - (step - (world - 1)) + 1) % world
+            deps = [last_of_rank[r]] if r in last_of_rank else []
+            if step > 1:  # wait for the neighbour's previous step through the signal word of link p -> r
+                w = add(dict(primitive=3, signal=signals_ptr + 4 * r, value=step - 1, deps=deps))
+                deps = [w]
+            off = c * size
+            if reduce_phase:
+                src = ("in" if step == 1 else "out", p, off)
+                o = dict(dtype=dtype, compute="sum", ins=[src, ("in", r, off)], outs=[("out", r, off)], count=size, deps=deps)
+            else:
+                o = dict(dtype=dtype, compute="sum", ins=[("out", p, off)], outs=[("out", r, off)], count=size, deps=deps)
+            bound = dict(o)
+            bound["ins"] = [(dev_in if b == "in" else dev_out)[rk].ptr + e * es for (b, rk, e) in o["ins"]]
+            bound["outs"] = [(dev_in if b == "in" else dev_out)[rk].ptr + e * es for (b, rk, e) in o["outs"]]
+            i = add(bound)
+            sym[i] = o
+            # tell the next rank that this step's output is there: link r -> r+1 is slot r+1
+            n = add(dict(primitive=2, signal=signals_ptr + 4 * ((r + 1) % world), value=step, deps=[i]))
+            notify_of[(r, step)] = n
+            last_of_rank[r] = n
+    return ops, sym
+
+
+def test_ring_allreduce_over_signal_words(hip, oracle):
+    import torch
+    world, size = 8, 3001
+    per = world * size
+    host_in = [H.gen("bf16", per, 81 + it, 0) for it in range(2)]  # two runs, different inputs
+    d_in = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    d_out = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    signals = torch.zeros(64, dtype=torch.int32, device="cuda")
+    ops, sym = _signal_ring_ops(world, size, signals.data_ptr(), d_in, d_out)
+    assert sum(1 for o in ops if o.get("primitive") == 2) == world * (2 * world - 2)
+    g = hip.Graph(ops)
+    # CPU replay of the data ops: program order of creation is a valid order
+    for it in range(2):
+        ins = [H.gen("bf16", per, 90 + 10 * it, r) for r in range(world)]
+        outs = [np.zeros(per, dtype=np.uint16) for _ in range(world)]
+        bufs = {"in": ins, "out": outs}
+        for i in sorted(sym):
+            o = sym[i]
+            oracle.reduce_copy("bf16", "sum", [bufs[b][r][e:e + size] for (b, r, e) in o["ins"]],
+                               [bufs[b][r][e:e + size] for (b, r, e) in o["outs"]])
+        for r in range(world):
+            d_in[r].upload(ins[r])
+            d_out[r].view().fill_(0xFF)
+        base = g.next_signal_base()
+        g.run(_stream(torch))
+        assert g.status(_stream(torch)) == (len(ops), len(ops))
+        for r in range(world):
+            H.assert_bits_equal(d_out[r].download(), outs[r], "run %d rank %d" % (it, r))
+        # every link's word ends at the last step of this run
+        assert signals[:world].cpu().tolist() == [base + 2 * world - 2] * world
+    g.destroy()
+
+
+def test_get_notified_from_outside_and_never(hip, oracle):
+    """A wait satisfied by a word the host set before the launch passes; a wait nobody satisfies
+    ends in PCCL_ERR_GRAPH through the bounded wait (no hang), and the graph works afterwards."""
+    import torch
+    count = 2048
+    a = H.gen("f32", count, 85, 0)
+    da, do = H.DevBuf(torch, "f32", count, 0, src=a), H.DevBuf(torch, "f32", count, 0)
+    sig = torch.zeros(4, dtype=torch.int32, device="cuda")
+    ops = [dict(primitive=3, signal=sig.data_ptr(), value=7, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[da.ptr], outs=[do.ptr], count=count, deps=[0])]
+    g = hip.Graph(ops)
+    g.set_spin_limit(512)
+    base = g.next_signal_base()
+    sig[0] = base + 7 - (1 << 32) if base + 7 >= (1 << 31) else base + 7
+    torch.cuda.synchronize()
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (2, 2)
+    H.assert_bits_equal(do.download(), a, "copy released by an outside notify")
+    # next run: the word still holds the previous run's value, which must NOT satisfy the wait
+    do.view().fill_(0)
+    g.run(_stream(torch))
+    with pytest.raises(hip.PcclError) as e:
+        g.status(_stream(torch))
+    assert e.value.code == hip.ERR_GRAPH
+    assert int(do.view().max()) == 0, "the dependent copy must not have run"
+    # the aborted run still consumed a run number; set the word for the coming one and run again
+    sig[0] = g.next_signal_base() + 7
+    torch.cuda.synchronize()
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (2, 2)
+    H.assert_bits_equal(do.download(), a, "after the aborted run")
+    g.destroy()
+
+
+def test_signal_op_argument_errors(hip):
+    import torch
+    sig = torch.zeros(4, dtype=torch.int32, device="cuda")
+    with pytest.raises(hip.PcclError) as e:
+        hip.Graph([dict(primitive=2, signal=sig.data_ptr() + 2, value=1)])
+    assert e.value.code == hip.ERR_MISALIGNED
+    with pytest.raises(hip.PcclError) as e:
+        hip.Graph([dict(primitive=2, signal=sig.data_ptr(), value=70000)])
+    assert e.value.code == hip.ERR_INVALID_ARG
+    with pytest.raises(hip.PcclError) as e:
+        hip.Graph([dict(primitive=3, signal=0, value=1)])
+    assert e.value.code == hip.ERR_INVALID_ARG
+    # a wait that depends on the very notify that would satisfy it, in reverse: cycle through the signal
+    with pytest.raises(hip.PcclError) as e:
+        hip.Graph([dict(primitive=3, signal=sig.data_ptr(), value=1, deps=[]),
+                   dict(primitive=2, signal=sig.data_ptr(), value=1, deps=[0])])
+    assert e.value.code == hip.ERR_GRAPH
+
+
+def test_copy_ops_keep_their_own_element_size(hip, oracle):
+    """COPY ops of 4-byte and 2-byte elements inside graphs whose REDUCE ops use the other size
+    (and in copy-only graphs): byte counts come from the op's dtype, not from the graph's kernel."""
+    import torch
+    n = 70001
+    f = H.gen("f32", n, 95, 0)
+    b = H.gen("bf16", n, 95, 1)
+    df, dfo = H.DevBuf(torch, "f32", n, 4, src=f), H.DevBuf(torch, "f32", n, 12)
+    db, dbo = H.DevBuf(torch, "bf16", n, 2, src=b), H.DevBuf(torch, "bf16", n, 6)
+    dsum = H.DevBuf(torch, "bf16", n, 0)
+    cases = {
+        "copy-only": [dict(dtype="f32", compute="sum", ins=[df.ptr], outs=[dfo.ptr], count=n),
+                      dict(dtype="bf16", compute="sum", ins=[db.ptr], outs=[dbo.ptr], count=n)],
+        "bf16 reduce + f32 copy": [dict(dtype="bf16", compute="sum", ins=[db.ptr, db.ptr], outs=[dsum.ptr], count=n),
+                                   dict(dtype="f32", compute="sum", ins=[df.ptr], outs=[dfo.ptr], count=n),
+                                   dict(dtype="bf16", compute="sum", ins=[dsum.ptr], outs=[dbo.ptr], count=n, deps=[0])],
+    }
+    for name, ops in cases.items():
+        for buf in (dfo, dbo, dsum):
+            buf.view().fill_(0xFF)
+        g = hip.Graph(ops, tile_bytes=8192)
+        _run_and_check(torch, hip, g, len(ops))
+        H.assert_bits_equal(dfo.download(), f, name + ": f32 copy")
+        want_b = b if name == "copy-only" else oracle.reduce("bf16", "sum", [b, b])
+        H.assert_bits_equal(dbo.download(), want_b, name + ": bf16 copy")
+        assert dfo.guards_intact() and dbo.guards_intact()
+        g.destroy()
