@@ -96,10 +96,23 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
       const char *base = x.buffer == "in" ? static_cast<const char *>(input) : static_cast<char *>(output);
       return const_cast<char *>(base) + ((long)x.device * s.elems_per_device + x.offset) * es;
     };
+    const PrimitiveType notify = TypeRegistry::getTypeId("notify"), get_notified = TypeRegistry::getTypeId("get_notified");
+    int *signals = nullptr;
+    if (buffers_->hasDevBuffer(rocm)) signals = static_cast<int *>(std::get<1>(buffers_->getDevBuffer(rocm)));
     std::vector<BoundOp> bound(s.ops.size());
     for (size_t i = 0; i < s.ops.size(); ++i) {
       const ScheduleOp &o = s.ops[i];
       BoundOp &b = bound[i];
+      if (o.isSignal()) {  // the operand is one of the workspace's signal slots, the count its value
+        if (!signals || o.slot >= SLOT)
+          throw std::runtime_error("Engine::exeOp(): signal slot " + std::to_string(o.slot) + " is not available");
+        b.primitive = o.kind == ScheduleOp::NOTIFY ? notify : get_notified;
+        b.compute = compute;
+        b.deps = o.deps;
+        const ChunkMeta word{dt, signals + o.slot, o.count};
+        (o.kind == ScheduleOp::NOTIFY ? b.outs : b.ins).push_back(word);
+        continue;
+      }
       b.primitive = o.reduce ? reduce : copy;
       b.compute = compute;
       b.deps = o.deps;

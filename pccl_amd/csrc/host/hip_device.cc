@@ -39,7 +39,7 @@ struct HipPluginRegistration {
     const int prim_codes[] = {PCCL_COPY, PCCL_REDUCE, PCCL_NOTIFY, PCCL_GET_NOTIFIED};
     for (int i = 0; i < 4; ++i) {
       t.primitive[TypeRegistry::registerPrimitive(prims[i])] = prim_codes[i];
-      if (i < 2) TypeRegistry::registerCompatibility("hip", prims[i]);  // notify / get_notified need a peer
+      TypeRegistry::registerCompatibility("hip", prims[i]);
     }
     const char *dtypes[] = {"f32", "i32", "bf16", "f16"};
     const int dtype_codes[] = {PCCL_F32, PCCL_I32, PCCL_BF16, PCCL_F16};
@@ -154,15 +154,18 @@ void *HipExecutor::createGraph(const std::vector<BoundOp> &ops) {
     const BoundOp &o = ops[i];
     pccl_op_desc &d = descs[i];
     d = pccl_op_desc{};
-    if (o.ins.empty() || o.outs.empty() || o.ins.size() > PCCL_MAX_INPUTS || o.outs.size() > PCCL_MAX_OUTPUTS)
-      throw std::runtime_error("HipExecutor::createGraph(): op " + std::to_string(i) + " has a bad operand count");
     d.op_uid = (int)i;
     d.primitive = (unsigned char)hipPrimitiveCode(o.primitive);
-    d.dtype = (unsigned char)hipDtypeCode(o.ins[0].dtype_);
+    const bool is_signal = d.primitive == PCCL_NOTIFY || d.primitive == PCCL_GET_NOTIFIED;
+    if (o.ins.size() > PCCL_MAX_INPUTS || o.outs.size() > PCCL_MAX_OUTPUTS || o.ins.size() + o.outs.size() == 0 ||
+        (!is_signal && (o.ins.empty() || o.outs.empty())))
+      throw std::runtime_error("HipExecutor::createGraph(): op " + std::to_string(i) + " has a bad operand count");
+    const ChunkMeta &first = o.ins.empty() ? o.outs[0] : o.ins[0];
+    d.dtype = (unsigned char)hipDtypeCode(first.dtype_);
     d.compute = (unsigned char)hipComputeCode(o.compute);
     d.n_in = (unsigned char)o.ins.size();
     d.n_out = (unsigned char)o.outs.size();
-    d.count = o.ins[0].num_elems_;
+    d.count = first.num_elems_;  // signal ops: the value
     for (size_t k = 0; k < o.ins.size(); ++k) d.ins[k] = o.ins[k].addr_;
     for (size_t k = 0; k < o.outs.size(); ++k) d.outs[k] = o.outs[k].addr_;
     d.n_deps = (int)o.deps.size();

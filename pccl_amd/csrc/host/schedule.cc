@@ -30,6 +30,16 @@ void Schedule::validate() const {
     const ScheduleOp &o = ops[i];
     const std::string at = "op " + std::to_string(i) + ": ";
     if (o.count < 0) bad(at + "negative count");
+    if (o.isSignal()) {
+      if (o.slot < 0 || o.slot >= 256) bad(at + "signal slot outside [0, 256)");
+      if (o.count > 0xffff) bad(at + "signal value outside [0, 65535]");
+      if (!o.srcs.empty() || !o.dsts.empty()) bad(at + "a signal op has no data operands");
+      if (o.deps.size() > 255) bad(at + "more than 255 dependencies");
+      for (int d : o.deps)
+        if (d < 0 || d >= n || d == i) bad(at + "dependency " + std::to_string(d) + " is not another op");
+      continue;
+    }
+    if ((o.kind == ScheduleOp::REDUCE) != o.reduce) bad(at + "kind and reduce flag disagree");
     if (o.srcs.empty() || o.srcs.size() > 8) bad(at + "needs 1..8 sources");
     if (o.dsts.empty() || o.dsts.size() > 8) bad(at + "needs 1..8 destinations");
     if (o.srcs.size() + o.dsts.size() > 10) bad(at + "more than 10 operands in all");
@@ -96,8 +106,13 @@ std::string Schedule::serialize() const {
   os << "ops " << ops.size() << "\n";
   for (size_t i = 0; i < ops.size(); ++i) {
     const ScheduleOp &o = ops[i];
-    os << "op " << i << ' ' << (o.reduce ? "REDUCE" : "COPY") << ' ' << o.count << " deps " << o.deps.size();
+    static const char *kinds[] = {"COPY", "REDUCE", "NOTIFY", "GET_NOTIFIED"};
+    os << "op " << i << ' ' << kinds[o.kind] << ' ' << o.count << " deps " << o.deps.size();
     for (int d : o.deps) os << ' ' << d;
+    if (o.isSignal()) {
+      os << " slot " << o.slot << "\n";
+      continue;
+    }
     os << " src " << o.srcs.size();
     for (const auto &x : o.srcs) os << ' ' << x.buffer << ' ' << x.device << ' ' << x.offset;
     os << " dst " << o.dsts.size();
@@ -162,15 +177,22 @@ Schedule Schedule::parse(const std::string &text) {
     if (integer("op id") != i) bad("op ids must be 0, 1, 2, ... in file order");
     ScheduleOp &o = s.ops[(size_t)i];
     const std::string kind = word("op kind");
-    if (kind == "REDUCE") o.reduce = true;
-    else if (kind == "COPY") o.reduce = false;
-    else if (kind == "NOTIFY" || kind == "GET_NOTIFIED") bad("op " + std::to_string(i) + ": " + kind + " signals between GPUs and cannot run on one device");
+    if (kind == "REDUCE") o.kind = ScheduleOp::REDUCE;
+    else if (kind == "COPY") o.kind = ScheduleOp::COPY;
+    else if (kind == "NOTIFY") o.kind = ScheduleOp::NOTIFY;
+    else if (kind == "GET_NOTIFIED") o.kind = ScheduleOp::GET_NOTIFIED;
     else bad("op " + std::to_string(i) + ": unknown kind '" + kind + "'");
+    o.reduce = o.kind == ScheduleOp::REDUCE;
     o.count = integer("count");
     expect("deps");
     const long nd = integer("dependency count");
     if (nd < 0 || nd > 255) bad("op " + std::to_string(i) + ": dependency count out of range");
     for (long d = 0; d < nd; ++d) o.deps.push_back((int)integer("dependency"));
+    if (o.isSignal()) {
+      expect("slot");
+      o.slot = (int)integer("slot");
+      continue;
+    }
     for (int side = 0; side < 2; ++side) {
       expect(side == 0 ? "src" : "dst");
       const long k = integer("operand count");
@@ -214,6 +236,7 @@ long appendRingAllReduce(Schedule &s, long chunk_elems, long base) {
       const int c = mod(r - step), p = mod(r - 1);
       const long off = base + (long)c * chunk_elems;
       ScheduleOp o;
+      o.kind = ScheduleOp::REDUCE;
       o.reduce = true;
       o.count = chunk_elems;
       o.srcs.push_back({step == 1 ? "in" : "out", p, off});  // partial sum arriving from rank r-1
@@ -252,6 +275,7 @@ long appendDirectAllReduce(Schedule &s, long slice_elems, long base) {
     const long off = base + (long)d * slice_elems;
     ScheduleOp red;
     red.reduce = W > 1;
+    red.kind = W > 1 ? ScheduleOp::REDUCE : ScheduleOp::COPY;
     red.count = slice_elems;
     for (int r = 0; r < W; ++r) red.srcs.push_back({"in", r, off});  // fixed order: rank 0 first
     red.dsts.push_back({"out", d, off});

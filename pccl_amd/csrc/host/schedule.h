@@ -18,6 +18,11 @@
 //   ops <n>
 //   op <id> <COPY|REDUCE> <count> deps <k> <id>*k  src <s> (<buffer> <device> <offset>)*s
 //                                                  dst <d> (<buffer> <device> <offset>)*d
+//   op <id> <NOTIFY|GET_NOTIFIED> <value> deps <k> <id>*k slot <index>
+// A signal op names one of the device workspace's int signal slots (csrc/engine.cc:16-18:
+// 256 slots behind the 256 MiB workspace) and a value in [0, 65535]; NOTIFY publishes the
+// value once its dependencies are complete, GET_NOTIFIED completes when the slot has
+// reached it (pccl/lang/chunk.py:9-10).
 // Buffers: "in" and "out" are the tensors given to exeOp, laid out as W consecutive
 // per-device regions of elems_per_device elements; "ws" is the device workspace.
 #pragma once
@@ -34,7 +39,11 @@ struct ScheduleOperand {
 };
 
 struct ScheduleOp {
-  bool reduce = false;  // false: COPY
+  enum Kind { COPY, REDUCE, NOTIFY, GET_NOTIFIED };
+  Kind kind = COPY;
+  bool reduce = false;  // kind == REDUCE (kept in step with kind by the parser and generators)
+  bool isSignal() const { return kind == NOTIFY || kind == GET_NOTIFIED; }
+  int slot = 0;         // signal ops: index of the signal slot; count is the value
   long count = 0;
   std::vector<int> deps;
   std::vector<ScheduleOperand> srcs;

@@ -59,6 +59,46 @@ def ring_allreduce(world, chunk_elems, dtype="bf16", compute="sum", name="ring_a
     return ir, base + W * chunk_elems
 
 
+def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", name="ring_allreduce_signalled",
+                             first_slot=0):
+    """The same ring all-reduce written the way ranks on different GPUs have to write it:
+    dependency edges only between ops of one rank; the hand-over between neighbours goes
+    NOTIFY (producer) -> signal slot -> GET_NOTIFIED (consumer).  Link (r-1) -> r uses slot
+    first_slot + r, and the value is the step number, so every slot sees its values rise.
+    Returns (ir, elements_per_rank_used)."""
+    W = world
+    ir = _ring_ir(name, W, dtype, compute)
+    last = {}  # rank -> its latest op
+    for step in range(1, 2 * W - 1):
+        reduce_phase = step < W
+        for r in range(W):
+            p = (r - 1) % W
+            c = (r - step) % W if reduce_phase else (r - (step - (W - 1)) + 1) % W
+            off = c * chunk_elems
+            deps = [last[r]] if r in last else []
+            if step > 1:
+                whole = Chunk(set(), p, chunk_elems, off)
+                deps = [ir.create_operation(PrimitiveOpType.GET_NOTIFIED, src_chunk=whole, tgt_chunk=whole, src_device=p,
+                                            tgt_device=r, dependencies=deps,
+                                            metadata={"slot": first_slot + r, "value": step - 1})]
+            if reduce_phase:
+                ranks = {(c + i) % W for i in range(step + 1)}
+                op = ir.create_operation(
+                    PrimitiveOpType.REDUCE, src_chunk=Chunk(ranks - {r}, p, chunk_elems, off),
+                    tgt_chunk=Chunk(ranks, r, chunk_elems, off), src_device=p, tgt_device=r, dependencies=deps,
+                    metadata={"srcs": [("in" if step == 1 else "out", p, off), ("in", r, off)], "tgt_buffer": "out"})
+            else:
+                full = set(range(W))
+                op = ir.create_operation(
+                    PrimitiveOpType.COPY, src_chunk=Chunk(full, p, chunk_elems, off), tgt_chunk=Chunk(full, r, chunk_elems, off),
+                    src_device=p, tgt_device=r, dependencies=deps, metadata={"src_buffer": "out", "tgt_buffer": "out"})
+            done = Chunk(set(), r, chunk_elems, off)
+            last[r] = ir.create_operation(PrimitiveOpType.NOTIFY, src_chunk=done, tgt_chunk=done, src_device=r,
+                                          tgt_device=(r + 1) % W, dependencies=[op],
+                                          metadata={"slot": first_slot + (r + 1) % W, "value": step})
+    return ir, W * chunk_elems
+
+
 def log_uniform_sizes(n, seed, lo_bytes, hi_bytes, elem_bytes):
     """n sizes in elements, log-uniform in [lo_bytes, hi_bytes] (splitmix64 stream of `seed`)."""
     def mix(z):
@@ -98,11 +138,18 @@ def small_message_allreduce(world=8, n_slices=36, n_extra=64, seed=4, lo_bytes=8
     return ir, base
 
 
-def bind(lowered, resolve):
-    """Replaces symbolic operands: resolve(buffer, device, element_offset) -> address."""
+def bind(lowered, resolve, signals=None):
+    """Replaces symbolic operands: resolve(buffer, device, element_offset) -> address.
+    Signal ops get "signal" = signals + 4 * slot (signals: address of the int slot array)."""
     out = []
     for o in lowered:
         d = dict(o)
+        if o.get("primitive", 0) >= 2:
+            if signals is None:
+                raise ValueError("schedule has signal ops: pass the address of the signal slots")
+            d["signal"] = int(signals) + 4 * o["slot"]
+            out.append(d)
+            continue
         d["ins"] = [resolve(*x) for x in o["ins"]]
         d["outs"] = [resolve(*x) for x in o["outs"]]
         out.append(d)

@@ -149,9 +149,13 @@ class CollectiveIR:
         lines = ["pccl-schedule 1", "name %s" % (self.name.replace(" ", "_") or "unnamed"), "dtype %s" % self.dtype,
                  "compute %s" % self.compute, "devices %d" % max(len(self.devices), 1),
                  "elems_per_device %d" % elems_per_device, "ops %d" % len(low)]
+        kinds = ("COPY", "REDUCE", "NOTIFY", "GET_NOTIFIED")
         for i, o in enumerate(low):
-            parts = ["op %d %s %d deps %d" % (i, "REDUCE" if o["primitive"] == 1 else "COPY", o["count"], len(o["deps"]))]
+            parts = ["op %d %s %d deps %d" % (i, kinds[o["primitive"]], o["count"], len(o["deps"]))]
             parts += [str(d) for d in o["deps"]]
+            if o["primitive"] >= 2:
+                lines.append(" ".join(parts + ["slot %d" % o["slot"]]))
+                continue
             for key, ops in (("src", o["ins"]), ("dst", o["outs"])):
                 parts.append("%s %d" % (key, len(ops)))
                 parts += ["%s %d %d" % (b, dev, off) for (b, dev, off) in ops]
@@ -167,6 +171,7 @@ class CollectiveIR:
         """Returns a list of dicts (dtype, compute, primitive, ins, outs, count, deps) whose
         operands are symbolic ``(buffer, device, element_offset)`` triples, op ids preserved.
 
+        NOTIFY / GET_NOTIFIED lower to signal ops (``primitive`` 2 / 3, ``slot``, ``value``).
         A COPY reads ``src_chunk`` and writes ``tgt_chunk``.  A REDUCE folds its sources in
         order and writes every destination; without ``metadata["srcs"]`` it is the reference's
         two-operand form "reduce src into tgt": fold(src, tgt) -> tgt."""
@@ -175,8 +180,13 @@ class CollectiveIR:
             op = self.ops[op_id]
             md = op.metadata
             if op.op_type in (PrimitiveOpType.NOTIFY, PrimitiveOpType.GET_NOTIFIED):
-                raise NotImplementedError("NOTIFY / GET_NOTIFIED are signalling ops between GPUs; "
-                                          "they have no single-GPU lowering")
+                # signal ops name a workspace signal slot and a value (metadata "slot", "value")
+                if "slot" not in md or "value" not in md:
+                    raise ValueError("op %d: NOTIFY / GET_NOTIFIED need metadata 'slot' and 'value'" % op_id)
+                prim = 2 if op.op_type is PrimitiveOpType.NOTIFY else 3
+                out.append(dict(primitive=prim, slot=int(md["slot"]), value=int(md["value"]), ins=[], outs=[],
+                                count=int(md["value"]), deps=list(op.dependencies)))
+                continue
             src = (md.get("src_buffer", "out"), op.src_device, op.src_chunk.offset)
             tgt = (md.get("tgt_buffer", "out"), op.tgt_device, op.tgt_chunk.offset)
             if op.op_type is PrimitiveOpType.COPY:

@@ -96,6 +96,10 @@ def parse_schedule_text(text):
         kind, count = nxt(), int(nxt())
         assert nxt() == "deps"
         deps = [int(nxt()) for _ in range(int(nxt()))]
+        if kind in ("NOTIFY", "GET_NOTIFIED"):
+            assert nxt() == "slot"
+            ops.append(dict(signal=kind, slot=int(nxt()), value=count, ins=[], outs=[], count=0, deps=deps))
+            continue
         sides = []
         for key in ("src", "dst"):
             assert nxt() == key
@@ -103,3 +107,20 @@ def parse_schedule_text(text):
         assert kind in ("COPY", "REDUCE")
         ops.append(dict(dtype=hdr["dtype"], compute=hdr["compute"], ins=sides[0], outs=sides[1], count=count, deps=deps))
     return hdr, ops
+
+
+def replay_with_signals(oracle, ops, order, resolve):
+    """CPU replay of a schedule that may hold signal ops: data ops go to the checker, NOTIFY
+    records its value, GET_NOTIFIED asserts that the value it waits for has been published."""
+    slots = {}
+    for i in order:
+        o = ops[i]
+        if o.get("signal") == "NOTIFY":
+            assert slots.get(o["slot"], -1) < o["value"], "slot %d must rise" % o["slot"]
+            slots[o["slot"]] = o["value"]
+        elif o.get("signal") == "GET_NOTIFIED":
+            assert slots.get(o["slot"], -1) >= o["value"], "op %d waits for a value nobody published before it" % i
+        else:
+            oracle.reduce_copy(o["dtype"], o["compute"], [resolve(*x, o["count"]) for x in o["ins"]],
+                               [resolve(*x, o["count"]) for x in o["outs"]])
+    return slots

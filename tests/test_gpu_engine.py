@@ -110,6 +110,34 @@ def test_direct_allreduce_8_inputs(E, eng, oracle, tmp_path):
     H.assert_bits_equal(got[:per], oracle.reduce("f16", "sum", wide), "equals one 8-input fold in rank order")
 
 
+def test_signalled_ring_schedule(E, eng, oracle, tmp_path):
+    """A schedule whose cross-rank hand-over goes through NOTIFY / GET_NOTIFIED on the workspace's
+    signal slots (no dependency edge between ranks), registered from a file and run twice."""
+    import torch
+    from pccl_amd import lang
+    ir, per = lang.ring_allreduce_signalled(8, 2500, dtype="bf16", first_slot=16)
+    p = str(tmp_path / "sig.sched")
+    ir.save(p, per)
+    text = open(p).read()
+    assert "NOTIFY" in text and "GET_NOTIFIED" in text
+    eng.regOp("sig", p)
+    hdr, ops = S.parse_schedule_text(text)
+    n = 8 * per
+    for it in range(2):
+        host_in = H.gen("bf16", n, 76 + it, 0)
+        want = np.zeros(n, dtype=np.uint16)
+        bufs = {"in": host_in, "out": want}
+        # file order is a valid order (each rank's program order, steps ascending)
+        slots = S.replay_with_signals(oracle, ops, range(len(ops)), lambda b, r, e, c: bufs[b][r * per + e:r * per + e + c])
+        assert slots == {16 + r: 14 for r in range(8)}
+        d_in, d_out = _to_dev(torch, host_in), torch.zeros(n * 2, dtype=torch.uint8, device="cuda")
+        eng.exeOp("sig", d_in, d_out)
+        eng.waitOp("sig")
+        H.assert_bits_equal(d_out.cpu().numpy().view(np.uint16), want, "signalled ring, run %d" % it)
+        for r in range(1, 8):
+            H.assert_bits_equal(want[r * per:(r + 1) * per], want[:per], "rank %d equals rank 0" % r)
+
+
 def test_exe_op_argument_errors(E, eng, tmp_path):
     import torch
     p = str(tmp_path / "r.sched")

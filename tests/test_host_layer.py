@@ -67,7 +67,7 @@ def test_registry_plugins_registered_at_load(E):
     assert len(set(ids)) == len(ids), "all kinds share one id space"
     for n in ("copy", "reduce", "f32", "i32", "bf16", "f16", "sum", "prod", "min", "max"):
         assert E.is_compatible("hip", n)
-    assert not E.is_compatible("hip", "notify") and not E.is_compatible("hip", "get_notified")
+    assert E.is_compatible("hip", "notify") and E.is_compatible("hip", "get_notified")
 
 
 def test_registry_register_and_errors(E):
@@ -161,7 +161,11 @@ def test_direct_allreduce_schedule_shape(E, tmp_path):
     ("pccl-schedule 1\nname x\ndtype f64\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "dtype"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute xor\ndevices 1\nelems_per_device 4\nops 0\n", "compute"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
-     "op 0 NOTIFY 4 deps 0 src 1 in 0 0 dst 1 out 0 0\n", "NOTIFY"),
+     "op 0 NOTIFY 4 deps 0 slot 256\n", "signal slot"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 GET_NOTIFIED 70000 deps 0 slot 3\n", "signal value"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 NOTIFY 4 deps 0 src 1 in 0 0 dst 1 out 0 0\n", "expected 'slot'"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
      "op 0 COPY 8 deps 0 src 1 in 0 0 dst 1 out 0 0\n", "past elems_per_device"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
@@ -268,8 +272,14 @@ def test_collective_ir_container():
     low = ir.lower()
     assert low[1]["ins"] == [("out", 1, 0), ("out", 2, 0)] and low[1]["outs"] == [("out", 2, 0)]  # reduce src into tgt
     ir.create_operation(PrimitiveOpType.NOTIFY, c, c, 0, 1)
-    with pytest.raises(NotImplementedError):
-        ir.lower()
+    with pytest.raises(ValueError):
+        ir.lower()  # a signal op needs a slot and a value
+    ir.ops[2].metadata.update(slot=5, value=9)
+    w = ir.create_operation(PrimitiveOpType.GET_NOTIFIED, c, c, 0, 1, dependencies=[b], metadata=dict(slot=5, value=9))
+    low = ir.lower()
+    assert low[2]["primitive"] == 2 and low[w]["primitive"] == 3 and low[w]["slot"] == 5 and low[w]["deps"] == [b]
+    text = ir.serialize()
+    assert "op 2 NOTIFY 9 deps 0 slot 5" in text and "op 3 GET_NOTIFIED 9 deps 1 1 slot 5" in text
     bad = CollectiveIR("cyc")
     x = bad.create_operation(PrimitiveOpType.COPY, c, c, 0, 0)
     bad.op_dag.add_edge(x, x)
