@@ -96,6 +96,10 @@ int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);
  * floor(160 KiB / lds_bytes); -1 = built-in choice, 0 = no cap. */
 int pccl_hip_set_occupancy_lds(int lds_bytes);
 
+/* Kernel-shape override for tuning runs: -1 = built-in choice, 0 = the lean one-pack-per-lane
+ * kernel wherever it applies, 1 or 4 = packs per lane of the general kernel. */
+int pccl_hip_set_unroll(int unroll);
+
 /* ---- the op-batching path: a DAG of ops drained by one persistent kernel -- */
 
 /* One IR operation as the host hands it over: the C++ payload level of

@@ -40,7 +40,7 @@ int compute_units() {
 }
 
 static std::mutex g_tuning_mutex;
-static Tuning g_tuning = {0, -1, -1};
+static Tuning g_tuning = {0, -1, -1, -1};
 static bool g_tuning_env_read = false;
 
 Tuning tuning() {
@@ -50,6 +50,7 @@ Tuning tuning() {
     if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tuning.workgroups_per_cu = atoi(s);
     if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.nontemporal = atoi(s) ? 1 : 0;
     if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tuning.lds_bytes = atoi(s);
+    if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tuning.unroll = atoi(s);
   }
   return g_tuning;
 }
@@ -135,6 +136,16 @@ int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal) {
   std::lock_guard<std::mutex> lock(g_tuning_mutex);
   g_tuning.workgroups_per_cu = workgroups_per_cu;
   g_tuning.nontemporal = nontemporal < 0 ? -1 : (nontemporal ? 1 : 0);
+  return PCCL_OK;
+}
+
+int pccl_hip_set_unroll(int unroll) {
+  clear_error();
+  if (unroll != -1 && unroll != 0 && unroll != 1 && unroll != 4)
+    return fail(PCCL_ERR_INVALID_ARG, "unroll %d is not -1, 0, 1 or 4", unroll);
+  (void)tuning();
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  g_tuning.unroll = unroll;
   return PCCL_OK;
 }
 

@@ -23,6 +23,7 @@ struct Tuning {
   int workgroups_per_cu;  // 0 = built-in choice
   int nontemporal;        // -1 = built-in choice, else 0/1
   int lds_bytes;          // -1 = built-in choice, else dynamic LDS requested per workgroup
+  int unroll;             // -1 = built-in choice, 0 = lean kernel where it applies, else packs per lane (1 or 4)
 };
 Tuning tuning();
 

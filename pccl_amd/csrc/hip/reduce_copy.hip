@@ -81,11 +81,12 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   const bool big = total_bytes > (192l << 20);
   const bool nt = t.nontemporal < 0 ? total_bytes >= (48l << 20) : t.nontemporal != 0;
   int unroll = big ? 1 : small_unroll_for(n_in);
+  if (t.unroll == 1 || t.unroll == 4) unroll = t.unroll == 4 ? small_unroll_for(n_in) : 1;
   // lean kernel: nothing to peel, at most two outputs, and no gain expected from
   // several packs per lane
   const int epp = 16 / es;
-  if (aligned && p.head == 0 && p.n_packs * epp == count && n_out <= 2 && unroll == 1 && t.workgroups_per_cu == 0)
-    unroll = 0;
+  const bool lean_ok = aligned && p.head == 0 && p.n_packs * epp == count && n_out <= 2 && t.workgroups_per_cu == 0;
+  if (lean_ok && (t.unroll == 0 || (t.unroll < 0 && unroll == 1))) unroll = 0;
   const long chunk = (long)kBlock * (unroll ? unroll : 1);
   long chunks = (p.n_packs + chunk - 1) / chunk;
   if (chunks < 1) chunks = 1;

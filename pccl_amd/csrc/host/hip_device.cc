@@ -56,6 +56,8 @@ struct HipPluginRegistration {
     regExecutor(t.executor, std::make_shared<HipExecutor>());
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_WG_PER_CU");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_NT");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_LDS_BYTES");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_UNROLL");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_TILE_BYTES");
   }
 };

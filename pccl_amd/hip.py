@@ -70,6 +70,7 @@ def lib():
         L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_set_tuning.argtypes = [ci, ci]
         L.pccl_hip_set_occupancy_lds.argtypes = [ci]
+        L.pccl_hip_set_unroll.argtypes = [ci]
         L.pccl_hip_graph_create.argtypes = [ctypes.POINTER(OpDesc), ci, cl, ctypes.POINTER(vp)]
         L.pccl_hip_graph_run.argtypes = [vp, vp]
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
@@ -133,6 +134,10 @@ def set_tuning(workgroups_per_cu=0, nontemporal=-1):
 
 def set_occupancy_lds(lds_bytes=-1):
     _check(lib().pccl_hip_set_occupancy_lds(lds_bytes))
+
+
+def set_unroll(unroll=-1):
+    _check(lib().pccl_hip_set_unroll(unroll))
 
 
 def reduce_copy(dtype, compute, ins, outs, count, stream=None):
