@@ -159,6 +159,13 @@ def main():
         assert torch.equal(o16[0], o16[1])
         del ins16, o16
 
+        # ---- fold one 128 MiB input into 7 destinations (the multimem.red role) -------------
+        src = randn(torch, c3, "bf16")
+        dsts = [randn(torch, c3, "bf16") for _ in range(7)]
+        t = event_times_us(torch, lambda: hip.accumulate("bf16", "sum", src, dsts, c3, stream), 20, 3)
+        extras["accumulate_bf16_1in_7dst_128MiB"] = dict(stats(t), GBps_median=gbps(15 * c3 * 2, t[len(t) // 2]))
+        del src, dsts
+
         # ---- ring all-reduce, one rank's share at world 8: 7 reduce-copy + 7 copy steps ----
         W, ce = 8, 1 << 24  # 32 MiB chunks of a 256 MiB gradient
         grad = randn(torch, W * ce, "bf16", 1e-2)

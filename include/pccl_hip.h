@@ -87,6 +87,14 @@ int pccl_hip_free(void *p);
 int pccl_hip_reduce_copy(int dtype, int compute, const void *const *ins, int n_in,
                          void *const *outs, int n_out, long count, void *stream);
 
+/* Folds ONE input into each of n_out destinations, reading the input once:
+ *   outs[j][i] = cvt(op(up(outs[j][i]), up(in[i])))      (destination first, then the value).
+ * The destinations must be distinct buffers that nothing else writes during the launch.
+ * Role: multimemStoreReduce, include/plugins/cuda_executor/utils/multimem.h:104-127
+ * (multimem.red.add of one pack into every peer's copy). */
+int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *outs, int n_out, long count,
+                        void *stream);
+
 /* Launch-shape overrides for tuning runs: workgroups per compute unit
  * (0 = built-in choice) and non-temporal access hint (0/1, -1 = built-in). */
 int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);

@@ -1,0 +1,125 @@
+// accumulate.hip -- pccl_hip_accumulate: fold ONE input into each of K destinations,
+//   outs[j][i] = cvt(op(up(outs[j][i]), up(in[i]))),
+// reading the input once.  Fills the role of multimemStoreReduce (reference
+// include/plugins/cuda_executor/utils/multimem.h:104-127: multimem.red.add of one
+// register pack into every peer's copy; only .add and only f32 / f16x2 there).
+// The destination is the accumulator (input 0 of the fold), the value is input 1;
+// each destination element is read and written by the same lane, so no atomics
+// are needed as long as nobody else writes the destinations during the launch.
+#include <algorithm>
+#include <cstring>
+
+#include "plugin_common.h"
+#include "reduce_copy_device.h"
+
+using namespace pccl_dev;
+using pccl_host::fail;
+
+namespace {
+
+struct AccLaunch {
+  const char *in;
+  char *out[PCCL_MAX_OUTPUTS];
+  int n_out;
+  long head;     // elements before the first 16-byte pack of output 0
+  long n_packs;  // 16-byte packs in the body
+  long count;
+};
+
+// ALIGNED: input and every output 16-byte aligned after the head peel.
+template <int DT, class Op, bool ALIGNED>
+__global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
+  typedef Dtype<DT> D;
+  typedef typename D::elem_t E;
+  constexpr int kEpp = 16 / D::kElemBytes;
+  const long pack = (long)blockIdx.x * kBlock + threadIdx.x;
+  if (pack < p.n_packs) {
+    const long off = p.head * D::kElemBytes + pack * 16;
+    u32x4 v[2];
+    v[1] = load_pack<D, ALIGNED, kMemCached>(p.in + off);
+#pragma unroll
+    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
+      if (j < p.n_out) {
+        // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
+        v[0] = j == 0 ? load_pack<D, true, kMemCached>(p.out[0] + off) : load_pack<D, ALIGNED, kMemCached>(p.out[j] + off);
+        const u32x4 r = fold_pack<D, Op, 2>(v);
+        if (j == 0) store_pack<D, true, kMemCached>(p.out[0] + off, r);
+        else store_pack<D, ALIGNED, kMemCached>(p.out[j] + off, r);
+      }
+  }
+  // head and tail elements: the last wavefront of the last workgroup
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x >= kBlock - kWave) {
+    const long tail_begin = p.head + p.n_packs * kEpp;
+    const long n_edge = p.head + (p.count - tail_begin);
+    for (long e = (long)threadIdx.x - (kBlock - kWave); e < n_edge; e += kWave) {
+      const long i = e < p.head ? e : tail_begin + (e - p.head);
+      E x[2];
+      x[1] = ((const E *)p.in)[i];
+#pragma unroll
+      for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
+        if (j < p.n_out) {
+          x[0] = ((const E *)p.out[j])[i];
+          ((E *)p.out[j])[i] = D::template elem<Op, 2>(x);
+        }
+    }
+  }
+}
+
+template <int DT, class Op>
+int launch_acc(bool aligned, unsigned grid, hipStream_t stream, const AccLaunch &p) {
+  if (aligned) hipLaunchKernelGGL((accumulate_kernel<DT, Op, true>), dim3(grid), dim3(kBlock), 0, stream, p);
+  else hipLaunchKernelGGL((accumulate_kernel<DT, Op, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(PCCL_ERR_HIP, "accumulate launch failed: %s", hipGetErrorString(e));
+  return PCCL_OK;
+}
+
+template <int DT>
+int launch_acc_op(int compute, bool aligned, unsigned grid, hipStream_t stream, const AccLaunch &p) {
+  switch (compute) {
+    case PCCL_SUM: return launch_acc<DT, OpSum>(aligned, grid, stream, p);
+    case PCCL_PROD: return launch_acc<DT, OpProd>(aligned, grid, stream, p);
+    case PCCL_MIN: return launch_acc<DT, OpMin>(aligned, grid, stream, p);
+    default: return launch_acc<DT, OpMax>(aligned, grid, stream, p);
+  }
+}
+
+}  // namespace
+
+extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *outs, int n_out,
+                                   long count, void *stream) {
+  pccl_host::clear_error();
+  if (dtype < PCCL_F32 || dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+  if (compute < PCCL_SUM || compute > PCCL_MAX) return fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute);
+  if (n_out < 1 || n_out > PCCL_MAX_OUTPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_out %d outside [1, 8]", n_out);
+  if (count < 0) return fail(PCCL_ERR_INVALID_ARG, "count %ld < 0", count);
+  if (!outs) return fail(PCCL_ERR_INVALID_ARG, "output array is null");
+  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  if (!in && count) return fail(PCCL_ERR_INVALID_ARG, "input is null");
+  if ((uintptr_t)in % es) return fail(PCCL_ERR_MISALIGNED, "input (%p) not %d-byte aligned", in, es);
+  AccLaunch p;
+  memset(&p, 0, sizeof(p));
+  p.in = (const char *)in;
+  for (int j = 0; j < n_out; ++j) {
+    if (!outs[j] && count) return fail(PCCL_ERR_INVALID_ARG, "output %d is null", j);
+    if ((uintptr_t)outs[j] % es) return fail(PCCL_ERR_MISALIGNED, "output %d (%p) not %d-byte aligned", j, outs[j], es);
+    for (int k = 0; k < j; ++k)
+      if (outs[k] == outs[j]) return fail(PCCL_ERR_INVALID_ARG, "outputs %d and %d are the same buffer", k, j);
+    p.out[j] = (char *)outs[j];
+  }
+  if (count == 0) return PCCL_OK;
+  p.n_out = n_out;
+  p.count = count;
+  p.head = std::min<long>(count, (long)((16 - ((uintptr_t)outs[0] & 15)) & 15) / es);
+  p.n_packs = (count - p.head) / (16 / es);
+  bool aligned = (((uintptr_t)in + (uintptr_t)p.head * es) & 15) == 0;
+  for (int j = 0; j < n_out; ++j) aligned = aligned && (((uintptr_t)outs[j] + (uintptr_t)p.head * es) & 15) == 0;
+  const unsigned grid = (unsigned)std::max<long>(1, (p.n_packs + kBlock - 1) / kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, grid, s, p);
+    case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, grid, s, p);
+    case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, grid, s, p);
+    default: return launch_acc_op<PCCL_F16>(compute, aligned, grid, s, p);
+  }
+}

@@ -68,6 +68,7 @@ def lib():
         L.pccl_hip_alloc.argtypes = [ctypes.POINTER(vp), cl]
         L.pccl_hip_free.argtypes = [vp]
         L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
+        L.pccl_hip_accumulate.argtypes = [ci, ci, vp, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_set_tuning.argtypes = [ci, ci]
         L.pccl_hip_set_occupancy_lds.argtypes = [ci]
         L.pccl_hip_set_unroll.argtypes = [ci]
@@ -147,6 +148,13 @@ def reduce_copy(dtype, compute, ins, outs, count, stream=None):
     a_out = (ctypes.c_void_p * max(n_out, 1))(*[_addr(x) for x in outs])
     _check(lib().pccl_hip_reduce_copy(_code(DTYPES, dtype), _code(COMPUTES, compute), a_in, n_in,
                                       a_out, n_out, count, ctypes.c_void_p(_addr(stream))))
+
+
+def accumulate(dtype, compute, src, outs, count, stream=None):
+    """outs[j][:count] = compute(outs[j][:count], src[:count]) for every j, reading src once."""
+    a_out = (ctypes.c_void_p * max(len(outs), 1))(*[_addr(x) for x in outs])
+    _check(lib().pccl_hip_accumulate(_code(DTYPES, dtype), _code(COMPUTES, compute), ctypes.c_void_p(_addr(src)), a_out,
+                                     len(outs), count, ctypes.c_void_p(_addr(stream))))
 
 
 class Graph:
