@@ -27,8 +27,10 @@ struct AccLaunch {
 };
 
 // ALIGNED: input and every output 16-byte aligned after the head peel.
-template <int DT, class Op, bool ALIGNED>
+// NT: streaming hints, for operands beyond the Infinity Cache.
+template <int DT, class Op, bool ALIGNED, bool NT>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
+  constexpr int kMem = NT ? kMemStream : kMemCached;
   typedef Dtype<DT> D;
   typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
@@ -36,15 +38,15 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   if (pack < p.n_packs) {
     const long off = p.head * D::kElemBytes + pack * 16;
     u32x4 v[2];
-    v[1] = load_pack<D, ALIGNED, kMemCached>(p.in + off);
+    v[1] = load_pack<D, ALIGNED, kMem>(p.in + off);
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.n_out) {
         // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
-        v[0] = j == 0 ? load_pack<D, true, kMemCached>(p.out[0] + off) : load_pack<D, ALIGNED, kMemCached>(p.out[j] + off);
+        v[0] = j == 0 ? load_pack<D, true, kMem>(p.out[0] + off) : load_pack<D, ALIGNED, kMem>(p.out[j] + off);
         const u32x4 r = fold_pack<D, Op, 2>(v);
-        if (j == 0) store_pack<D, true, kMemCached>(p.out[0] + off, r);
-        else store_pack<D, ALIGNED, kMemCached>(p.out[j] + off, r);
+        if (j == 0) store_pack<D, true, kMem>(p.out[0] + off, r);
+        else store_pack<D, ALIGNED, kMem>(p.out[j] + off, r);
       }
   }
   // head and tail elements: the last wavefront of the last workgroup
@@ -66,21 +68,27 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
 }
 
 template <int DT, class Op>
-int launch_acc(bool aligned, unsigned grid, hipStream_t stream, const AccLaunch &p) {
-  if (aligned) hipLaunchKernelGGL((accumulate_kernel<DT, Op, true>), dim3(grid), dim3(kBlock), 0, stream, p);
-  else hipLaunchKernelGGL((accumulate_kernel<DT, Op, false>), dim3(grid), dim3(kBlock), 0, stream, p);
+int launch_acc(bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const AccLaunch &p) {
+  if (aligned) {
+    if (nt) hipLaunchKernelGGL((accumulate_kernel<DT, Op, true, true>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((accumulate_kernel<DT, Op, true, false>), dim3(grid), dim3(kBlock), lds, stream, p);
+  } else {
+    if (nt) hipLaunchKernelGGL((accumulate_kernel<DT, Op, false, true>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((accumulate_kernel<DT, Op, false, false>), dim3(grid), dim3(kBlock), lds, stream, p);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "accumulate launch failed: %s", hipGetErrorString(e));
   return PCCL_OK;
 }
 
 template <int DT>
-int launch_acc_op(int compute, bool aligned, unsigned grid, hipStream_t stream, const AccLaunch &p) {
+int launch_acc_op(int compute, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream,
+                  const AccLaunch &p) {
   switch (compute) {
-    case PCCL_SUM: return launch_acc<DT, OpSum>(aligned, grid, stream, p);
-    case PCCL_PROD: return launch_acc<DT, OpProd>(aligned, grid, stream, p);
-    case PCCL_MIN: return launch_acc<DT, OpMin>(aligned, grid, stream, p);
-    default: return launch_acc<DT, OpMax>(aligned, grid, stream, p);
+    case PCCL_SUM: return launch_acc<DT, OpSum>(aligned, nt, grid, lds, stream, p);
+    case PCCL_PROD: return launch_acc<DT, OpProd>(aligned, nt, grid, lds, stream, p);
+    case PCCL_MIN: return launch_acc<DT, OpMin>(aligned, nt, grid, lds, stream, p);
+    default: return launch_acc<DT, OpMax>(aligned, nt, grid, lds, stream, p);
   }
 }
 
@@ -115,11 +123,24 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
   bool aligned = (((uintptr_t)in + (uintptr_t)p.head * es) & 15) == 0;
   for (int j = 0; j < n_out; ++j) aligned = aligned && (((uintptr_t)outs[j] + (uintptr_t)p.head * es) & 15) == 0;
   const unsigned grid = (unsigned)std::max<long>(1, (p.n_packs + kBlock - 1) / kBlock);
+  // Launch policy, measured on MI355X with 128 MiB operands.  A lane handles its
+  // destinations one after the other (a store to one may alias a load of the next), so
+  // only two loads are in flight per lane and the kernel wants more resident workgroups
+  // than reduce_copy does: streaming hints pay from two destinations on (6.3 vs 5.8 TB/s;
+  // with one destination the read-modify-write prefers cached accesses, 7.0 vs 6.2), and a
+  // cap of 5 workgroups per compute unit pays from three destinations on (1 -> 7: 6.4 vs
+  // 5.5 TB/s uncapped, 4.6 with 2 workgroups).
+  const pccl_host::Tuning t = pccl_host::tuning();
+  const long total_bytes = (long)(1 + 2 * n_out) * count * es;
+  const bool nt = t.nontemporal < 0 ? (n_out >= 2 && total_bytes >= (48l << 20)) : t.nontemporal != 0;
+  unsigned lds = 0;
+  if (t.lds_bytes >= 0) lds = (unsigned)t.lds_bytes;
+  else if (n_out >= 3 && total_bytes > (192l << 20)) lds = 160 * 1024 / 5 - 256;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, grid, s, p);
-    case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, grid, s, p);
-    case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, grid, s, p);
-    default: return launch_acc_op<PCCL_F16>(compute, aligned, grid, s, p);
+    case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, nt, grid, lds, s, p);
+    case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, nt, grid, lds, s, p);
+    case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, nt, grid, lds, s, p);
+    default: return launch_acc_op<PCCL_F16>(compute, aligned, nt, grid, lds, s, p);
   }
 }
