@@ -37,8 +37,15 @@ enum pccl_dtype {   /* element types with 16-byte packs in                      
   PCCL_F32 = 0,     /* include/plugins/cuda_executor/utils/vector_datatype.h:66    */
   PCCL_I32 = 1,     /* :64                                                         */
   PCCL_BF16 = 2,    /* :71 (bf16x8)                                                */
-  PCCL_F16 = 3      /* :70 (f16x8)                                                 */
+  PCCL_F16 = 3,     /* :70 (f16x8)                                                 */
+  PCCL_F8E4M3 = 4,  /* :75-77 (fp8_e4m3 packs): OCP E4M3FN, 16 per 16-byte pack     */
+  PCCL_F8E5M2 = 5   /* :78-80 (fp8_e5m2 packs): OCP E5M2                            */
 };
+#define PCCL_NUM_DTYPES 6
+
+/* Element size in bytes of a dtype code (the scalar types of vector_datatype.h:55-80),
+ * 0 for an unknown code. */
+int pccl_hip_dtype_bytes(int dtype);
 enum pccl_compute { /* multimem.h:12-59 only has .add; min/max/prod complete the   */
   PCCL_SUM = 0,     /* set of ComputeType names the registry is meant to hold      */
   PCCL_PROD = 1,
@@ -76,8 +83,8 @@ int pccl_hip_free(void *p);
 
 /* out[j][i] = cvt(fold_op(up(in[0][i]) ... up(in[n_in-1][i]))) for j < n_out,
  * i < count.  Strict left fold in input order; float accumulator for
- * f32/bf16/f16 with one round-to-nearest-even at the end; uint32 wraparound
- * for i32; n_in == 1 copies bytes.  Any element-aligned addresses; an output
+ * f32/bf16/f16/f8 with one round-to-nearest-even at the end (f8: saturating to the
+ * largest finite value); uint32 wraparound for i32; n_in == 1 copies bytes.  Any element-aligned addresses; an output
  * may be the same buffer as an input (in place), other overlaps are undefined.
  * One kernel launch on `stream` (a hipStream_t; NULL = the default stream);
  * returns without waiting.

@@ -73,6 +73,80 @@ uint16_t pccl_oracle_f32_to_f16(float x) {
   return (uint16_t)(sign | q); /* q == 0x400 is the smallest normal: correct */
 }
 
+/* ------------------------------------------------------------------------ */
+/* 8-bit floats.  One routine for both layouts: MAN mantissa bits, BIAS, and  */
+/* whether the top exponent code is reserved for inf/NaN (e5m2) or only       */
+/* S.1111.111 is NaN (e4m3).                                                  */
+/* ------------------------------------------------------------------------ */
+static float f8_to_f32(uint8_t h, int man_bits, int bias, int ieee_specials) {
+  const int exp_bits = 7 - man_bits;
+  const uint32_t sign = ((uint32_t)h & 0x80u) << 24;
+  const uint32_t exp = ((uint32_t)h >> man_bits) & ((1u << exp_bits) - 1u);
+  const uint32_t man = (uint32_t)h & ((1u << man_bits) - 1u);
+  const uint32_t exp_max = (1u << exp_bits) - 1u;
+  if (ieee_specials && exp == exp_max)
+    return u2f(sign | 0x7f800000u | (man ? 0x00400000u | (man << (23 - man_bits)) : 0u));
+  if (!ieee_specials && exp == exp_max && man == (1u << man_bits) - 1u) return u2f(sign | 0x7fc00000u);
+  if (exp != 0) return u2f(sign | ((exp + 127u - (uint32_t)bias) << 23) | (man << (23 - man_bits)));
+  /* subnormal: man * 2^(1 - bias - man_bits); small integers and powers of two are exact */
+  float v = (float)man * u2f((uint32_t)(127 + 1 - bias - man_bits) << 23);
+  return sign ? -v : v;
+}
+
+static uint8_t f32_to_f8(float x, int man_bits, int bias, int ieee_specials) {
+  const int exp_bits = 7 - man_bits;
+  const uint32_t u = f2u(x);
+  const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  const uint32_t a = u & 0x7fffffffu;
+  const uint8_t nan_code = 0x7fu; /* S.1111.111 and S.11111.11 */
+  /* largest finite code: e4m3 S.1111.110, e5m2 S.11110.11 */
+  const uint8_t max_code = ieee_specials ? (uint8_t)(((((1u << exp_bits) - 2u)) << man_bits) | ((1u << man_bits) - 1u))
+                                         : (uint8_t)0x7eu;
+  if (a > 0x7f800000u) return (uint8_t)(sign | nan_code);
+  /* a true infinity stays infinite where the format has one and is NaN where it has none */
+  if (a == 0x7f800000u) return (uint8_t)(sign | (ieee_specials ? 0x7cu : nan_code));
+  const int e = (int)(a >> 23) - 127;         /* unbiased exponent of |x| (normal binary32) */
+  const int min_normal = 1 - bias;            /* unbiased exponent of the smallest normal */
+  uint32_t q;                                  /* result without the sign */
+  if ((a >> 23) == 0) {
+    q = 0;                                     /* binary32 subnormals are far below half the smallest step */
+  } else if (e >= min_normal) {
+    /* normal result: keep man_bits of mantissa, round to nearest even on the rest */
+    const int drop = 23 - man_bits;
+    uint32_t v = a - ((uint32_t)(127 - bias) << 23);   /* rebias the exponent field */
+    v += ((1u << (drop - 1)) - 1u) + ((v >> drop) & 1u);
+    q = v >> drop;                             /* a mantissa carry walks into the exponent */
+  } else {
+    /* subnormal result: integer count of steps of 2^(min_normal - man_bits) */
+    const uint32_t man = (a & 0x7fffffu) | 0x800000u;  /* value = man * 2^(e - 23) */
+    const int shift = (min_normal - man_bits) - (e - 23);
+    if (shift > 31) {
+      q = 0;
+    } else {
+      q = man >> shift;
+      const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+      if (rem > half || (rem == half && (q & 1u))) ++q;  /* q == 2^man_bits is the smallest normal */
+    }
+  }
+  if (q > max_code) q = max_code;              /* saturate: finite overflow and rounding past the top */
+  return (uint8_t)(sign | q);
+}
+
+uint8_t pccl_oracle_f32_to_e4m3(float x) { return f32_to_f8(x, 3, 7, 0); }
+float pccl_oracle_e4m3_to_f32(uint8_t h) { return f8_to_f32(h, 3, 7, 0); }
+uint8_t pccl_oracle_f32_to_e5m2(float x) { return f32_to_f8(x, 2, 15, 1); }
+float pccl_oracle_e5m2_to_f32(uint8_t h) { return f8_to_f32(h, 2, 15, 1); }
+
+void pccl_oracle_narrow_array8(int dtype, const float *src, uint8_t *dst, long n) {
+  for (long i = 0; i < n; ++i)
+    dst[i] = dtype == PCCL_ORACLE_F8E4M3 ? pccl_oracle_f32_to_e4m3(src[i]) : pccl_oracle_f32_to_e5m2(src[i]);
+}
+
+void pccl_oracle_widen_array8(int dtype, const uint8_t *src, float *dst, long n) {
+  for (long i = 0; i < n; ++i)
+    dst[i] = dtype == PCCL_ORACLE_F8E4M3 ? pccl_oracle_e4m3_to_f32(src[i]) : pccl_oracle_e5m2_to_f32(src[i]);
+}
+
 void pccl_oracle_narrow_array(int dtype, const float *src, uint16_t *dst, long n) {
   for (long i = 0; i < n; ++i)
     dst[i] = dtype == PCCL_ORACLE_BF16 ? pccl_oracle_f32_to_bf16(src[i])
@@ -102,6 +176,7 @@ static size_t dtype_size(int dtype) {
   switch (dtype) {
     case PCCL_ORACLE_F32: case PCCL_ORACLE_I32: return 4;
     case PCCL_ORACLE_BF16: case PCCL_ORACLE_F16: return 2;
+    case PCCL_ORACLE_F8E4M3: case PCCL_ORACLE_F8E5M2: return 1;
     default: return 0;
   }
 }
@@ -145,6 +220,12 @@ static int reduce_range(int dtype, int op, const void *const *ins, int n_in,
       break;
     case PCCL_ORACLE_F16:
       BY_OP(uint16_t, float, pccl_oracle_f16_to_f32, pccl_oracle_f32_to_f16, f);
+      break;
+    case PCCL_ORACLE_F8E4M3:
+      BY_OP(uint8_t, float, pccl_oracle_e4m3_to_f32, pccl_oracle_f32_to_e4m3, f);
+      break;
+    case PCCL_ORACLE_F8E5M2:
+      BY_OP(uint8_t, float, pccl_oracle_e5m2_to_f32, pccl_oracle_f32_to_e5m2, f);
       break;
     default: return -1;
   }
@@ -313,6 +394,8 @@ void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64
       case PCCL_ORACLE_F32: ((float *)dst)[i] = z; break;
       case PCCL_ORACLE_BF16: ((uint16_t *)dst)[i] = pccl_oracle_f32_to_bf16(z); break;
       case PCCL_ORACLE_F16: ((uint16_t *)dst)[i] = pccl_oracle_f32_to_f16(z); break;
+      case PCCL_ORACLE_F8E4M3: ((uint8_t *)dst)[i] = pccl_oracle_f32_to_e4m3(z); break;
+      case PCCL_ORACLE_F8E5M2: ((uint8_t *)dst)[i] = pccl_oracle_f32_to_e5m2(z); break;
       default: return;
     }
   }

@@ -34,6 +34,11 @@
  *       pinned: exhaustive 2^16 widening and a committed fixture of
  *       round-to-nearest-even cases checked against numpy/torch conversions
  *       (tests/test_oracle_convert.py).
+ *   pccl_oracle_f32_to_e4m3 / e4m3_to_f32 / f32_to_e5m2 / e5m2_to_f32
+ *       pinned: all 256 encodings widened against torch.float8_e4m3fn / float8_e5m2;
+ *       narrowing against torch for every float that does not overflow (torch does
+ *       not saturate) and for infinities, and against the closed form for the
+ *       saturating range (tests/test_oracle_convert.py).
  *   pccl_oracle_reduce_copy
  *       pinned against the mathematics: exact-rational brute force with one
  *       rounding per step, fold-order-sensitive known answers, int32
@@ -54,7 +59,8 @@ extern "C" {
 #endif
 
 /* dtype / compute / primitive codes: same numbering as include/pccl_hip.h. */
-enum { PCCL_ORACLE_F32 = 0, PCCL_ORACLE_I32 = 1, PCCL_ORACLE_BF16 = 2, PCCL_ORACLE_F16 = 3 };
+enum { PCCL_ORACLE_F32 = 0, PCCL_ORACLE_I32 = 1, PCCL_ORACLE_BF16 = 2, PCCL_ORACLE_F16 = 3,
+       PCCL_ORACLE_F8E4M3 = 4, PCCL_ORACLE_F8E5M2 = 5 };
 enum { PCCL_ORACLE_SUM = 0, PCCL_ORACLE_PROD = 1, PCCL_ORACLE_MIN = 2, PCCL_ORACLE_MAX = 3 };
 
 /* ---- conversions -------------------------------------------------------- */
@@ -62,9 +68,24 @@ uint16_t pccl_oracle_f32_to_bf16(float x);
 float pccl_oracle_bf16_to_f32(uint16_t h);
 uint16_t pccl_oracle_f32_to_f16(float x);
 float pccl_oracle_f16_to_f32(uint16_t h);
-/* bulk forms used by the tests: dtype is BF16 or F16 */
+/* 8-bit floats of include/plugins/cuda_executor/utils/vector_datatype.h:11-16,75-80:
+ * e4m3 = OCP E4M3FN (bias 7, no infinity, NaN = S.1111.111, largest finite 448),
+ * e5m2 = OCP E5M2 (bias 15, IEEE-like infinities and NaNs, largest finite 57344).
+ * Narrowing rounds to nearest even; a FINITE value beyond the largest finite one SATURATES
+ * to it (what the __nv_fp8_* types the reference names do when built from float); a true
+ * infinity stays infinite in e5m2 and becomes NaN in e4m3, which has none (no fold of e4m3
+ * operands can produce one); NaN becomes S.1111.111 / S.11111.11 here, and any NaN encoding
+ * of the format counts as equal to it. */
+uint8_t pccl_oracle_f32_to_e4m3(float x);
+float pccl_oracle_e4m3_to_f32(uint8_t h);
+uint8_t pccl_oracle_f32_to_e5m2(float x);
+float pccl_oracle_e5m2_to_f32(uint8_t h);
+/* bulk forms used by the tests: dtype is BF16 or F16 (uint16_t storage) */
 void pccl_oracle_narrow_array(int dtype, const float *src, uint16_t *dst, long n);
 void pccl_oracle_widen_array(int dtype, const uint16_t *src, float *dst, long n);
+/* dtype is F8E4M3 or F8E5M2 (uint8_t storage) */
+void pccl_oracle_narrow_array8(int dtype, const float *src, uint8_t *dst, long n);
+void pccl_oracle_widen_array8(int dtype, const uint8_t *src, float *dst, long n);
 
 /* ---- the reduce-copy itself --------------------------------------------- */
 /* Returns 0 on success, -1 on a bad argument.  Operand element type follows

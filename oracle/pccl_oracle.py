@@ -12,12 +12,12 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpccl_oracle.so")
 
-F32, I32, BF16, F16 = 0, 1, 2, 3
+F32, I32, BF16, F16, F8E4M3, F8E5M2 = 0, 1, 2, 3, 4, 5
 SUM, PROD, MIN, MAX = 0, 1, 2, 3
-DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16}
+DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16, "f8e4m3": F8E4M3, "f8e5m2": F8E5M2}
 COMPUTES = {"sum": SUM, "prod": PROD, "min": MIN, "max": MAX}
 # numpy storage type per dtype code (bf16/f16 travel as raw uint16 bit patterns)
-NP_STORAGE = {F32: np.float32, I32: np.int32, BF16: np.uint16, F16: np.uint16}
+NP_STORAGE = {F32: np.float32, I32: np.int32, BF16: np.uint16, F16: np.uint16, F8E4M3: np.uint8, F8E5M2: np.uint8}
 
 
 class OracleOp(ctypes.Structure):
@@ -53,6 +53,10 @@ def lib():
         L.pccl_oracle_narrow_array.restype = None
         L.pccl_oracle_widen_array.argtypes = [ci, vp, vp, cl]
         L.pccl_oracle_widen_array.restype = None
+        L.pccl_oracle_narrow_array8.argtypes = [ci, vp, vp, cl]
+        L.pccl_oracle_narrow_array8.restype = None
+        L.pccl_oracle_widen_array8.argtypes = [ci, vp, vp, cl]
+        L.pccl_oracle_widen_array8.restype = None
         L.pccl_oracle_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl]
         L.pccl_oracle_reduce_copy_mt.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, ci]
         L.pccl_oracle_run_ops.argtypes = [ctypes.POINTER(OracleOp), ci, ctypes.POINTER(ci)]
@@ -78,17 +82,28 @@ def _ptr(a):
 
 
 def narrow(dtype, x):
-    """float32 array -> uint16 bit patterns of bf16 / f16 (round to nearest even)."""
+    """float32 array -> bit patterns of bf16 / f16 (uint16) or f8e4m3 / f8e5m2 (uint8)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
+    dt = _code(DTYPES, dtype)
+    if dt in (F8E4M3, F8E5M2):
+        out = np.empty(x.shape, dtype=np.uint8)
+        lib().pccl_oracle_narrow_array8(dt, x.ctypes.data, out.ctypes.data, x.size)
+        return out
     out = np.empty(x.shape, dtype=np.uint16)
-    lib().pccl_oracle_narrow_array(_code(DTYPES, dtype), x.ctypes.data, out.ctypes.data, x.size)
+    lib().pccl_oracle_narrow_array(dt, x.ctypes.data, out.ctypes.data, x.size)
     return out
 
 
 def widen(dtype, h):
+    dt = _code(DTYPES, dtype)
+    if dt in (F8E4M3, F8E5M2):
+        h = np.ascontiguousarray(h, dtype=np.uint8)
+        out = np.empty(h.shape, dtype=np.float32)
+        lib().pccl_oracle_widen_array8(dt, h.ctypes.data, out.ctypes.data, h.size)
+        return out
     h = np.ascontiguousarray(h, dtype=np.uint16)
     out = np.empty(h.shape, dtype=np.float32)
-    lib().pccl_oracle_widen_array(_code(DTYPES, dtype), h.ctypes.data, out.ctypes.data, h.size)
+    lib().pccl_oracle_widen_array(dt, h.ctypes.data, out.ctypes.data, h.size)
     return out
 
 

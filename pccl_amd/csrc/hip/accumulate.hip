@@ -32,6 +32,7 @@ template <int DT, class Op, bool ALIGNED, bool NT>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   constexpr int kMem = NT ? kMemStream : kMemCached;
   typedef Dtype<DT> D;
+  D::wave_init();
   typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
   const long pack = (long)blockIdx.x * kBlock + threadIdx.x;
@@ -97,12 +98,12 @@ int launch_acc_op(int compute, bool aligned, bool nt, unsigned grid, unsigned ld
 extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *outs, int n_out,
                                    long count, void *stream) {
   pccl_host::clear_error();
-  if (dtype < PCCL_F32 || dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+  if (dtype < 0 || dtype >= PCCL_NUM_DTYPES) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
   if (compute < PCCL_SUM || compute > PCCL_MAX) return fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute);
   if (n_out < 1 || n_out > PCCL_MAX_OUTPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_out %d outside [1, 8]", n_out);
   if (count < 0) return fail(PCCL_ERR_INVALID_ARG, "count %ld < 0", count);
   if (!outs) return fail(PCCL_ERR_INVALID_ARG, "output array is null");
-  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  const int es = pccl_host::pccl_dtype_bytes(dtype);
   if (!in && count) return fail(PCCL_ERR_INVALID_ARG, "input is null");
   if ((uintptr_t)in % es) return fail(PCCL_ERR_MISALIGNED, "input (%p) not %d-byte aligned", in, es);
   AccLaunch p;
@@ -141,6 +142,8 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
     case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, nt, grid, lds, s, p);
     case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, nt, grid, lds, s, p);
     case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, nt, grid, lds, s, p);
-    default: return launch_acc_op<PCCL_F16>(compute, aligned, nt, grid, lds, s, p);
+    case PCCL_F16: return launch_acc_op<PCCL_F16>(compute, aligned, nt, grid, lds, s, p);
+    case PCCL_F8E4M3: return launch_acc_op<PCCL_F8E4M3>(compute, aligned, nt, grid, lds, s, p);
+    default: return launch_acc_op<PCCL_F8E5M2>(compute, aligned, nt, grid, lds, s, p);
   }
 }

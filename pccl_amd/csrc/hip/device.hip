@@ -160,6 +160,8 @@ int pccl_hip_set_occupancy_lds(int lds_bytes) {
 
 const char *pccl_hip_last_error(void) { return g_error; }
 
+int pccl_hip_dtype_bytes(int dtype) { return pccl_dtype_bytes(dtype); }
+
 const char *pccl_hip_version(void) { return "pccl_hip 0.1 (gfx950)"; }
 
 }  // extern "C"

@@ -170,10 +170,10 @@ __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, lon
   switch (pl->n_in_) {
     case 1: {
       // COPY moves bytes, and its element size is its own, not that of the graph's
-      // REDUCE ops: run it as a copy of 2-byte units
+      // REDUCE ops: run it as a copy of 1-byte units
       const int dt = pl->chunks_[0].dtype_;
-      const long units = (dt == PCCL_F32 || dt == PCCL_I32) ? 2 : 1;
-      run_part_nin<Dtype<PCCL_BF16>, OpSum, 1>(pl, lo * units, count * units);
+      const long units = (dt == PCCL_F32 || dt == PCCL_I32) ? 4 : (dt == PCCL_BF16 || dt == PCCL_F16) ? 2 : 1;
+      run_part_nin<Dtype<PCCL_F8E4M3>, OpSum, 1>(pl, lo * units, count * units);
       break;
     }
     case 2: run_part_nin<D, Op, 2>(pl, lo, count); break;
@@ -227,6 +227,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   __shared__ unsigned long long s_entry;
   __shared__ int s_go;
   __shared__ int s_last;
+  Dtype<DT>::wave_init();
   HotWord *hot = g.hot;
   unsigned int *abort_flag = &hot[kHotAbort].value;
   const unsigned int spin_limit = g.spin_limit;
@@ -357,7 +358,9 @@ DrainKernel drain_for(int dtype, int compute) {
     case PCCL_F32: return drain_for_compute<PCCL_F32>(compute);
     case PCCL_I32: return drain_for_compute<PCCL_I32>(compute);
     case PCCL_BF16: return drain_for_compute<PCCL_BF16>(compute);
-    default: return drain_for_compute<PCCL_F16>(compute);
+    case PCCL_F16: return drain_for_compute<PCCL_F16>(compute);
+    case PCCL_F8E4M3: return drain_for_compute<PCCL_F8E4M3>(compute);
+    default: return drain_for_compute<PCCL_F8E5M2>(compute);
   }
 }
 
@@ -378,7 +381,7 @@ struct Graph {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-int elem_bytes(int dtype) { return (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2; }
+int elem_bytes(int dtype) { return pccl_host::pccl_dtype_bytes(dtype); }
 
 }  // namespace
 
@@ -417,7 +420,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
         return fail(PCCL_ERR_INVALID_ARG, "op %d: signal value %ld outside [0, 65535]", i, o.count);
       signal_ops.push_back(i);
     } else {
-      if (o.dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown dtype code %d", i, o.dtype);
+      if (o.dtype >= PCCL_NUM_DTYPES) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown dtype code %d", i, o.dtype);
       if (o.compute > PCCL_MAX) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown compute code %d", i, o.compute);
       if (o.n_in < 1 || o.n_in > PCCL_MAX_INPUTS || o.n_out < 1 || o.n_out > PCCL_MAX_OUTPUTS ||
           o.n_in + o.n_out > PCCL_MAX_OP_CHUNKS)

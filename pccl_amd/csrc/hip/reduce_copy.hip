@@ -9,9 +9,10 @@ namespace pccl_dev {
 
 int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
                 hipStream_t stream, const RcLaunch &p) {
-  // the dtype only selects the alignment the unaligned pack type may assume
+  // the dtype only selects the element size and the alignment the unaligned pack type may assume
   if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
-  return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
+  if (elem_bytes == 2) return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
+  return launch_nin<PCCL_F8E4M3, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
 }
 
 }  // namespace pccl_dev
@@ -25,14 +26,14 @@ namespace pccl_host {
 // launch record.  Returns PCCL_OK or an error code (text set).
 int plan_reduce_copy(int dtype, int compute, const void *const *ins, int n_in, void *const *outs,
                      int n_out, long count, RcLaunch *out, bool *aligned) {
-  if (dtype < PCCL_F32 || dtype > PCCL_F16) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+  if (dtype < 0 || dtype >= PCCL_NUM_DTYPES) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
   if (compute < PCCL_SUM || compute > PCCL_MAX)
     return fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute);
   if (n_in < 1 || n_in > PCCL_MAX_INPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_in %d outside [1, 8]", n_in);
   if (n_out < 1 || n_out > PCCL_MAX_OUTPUTS) return fail(PCCL_ERR_INVALID_ARG, "n_out %d outside [1, 8]", n_out);
   if (count < 0) return fail(PCCL_ERR_INVALID_ARG, "count %ld < 0", count);
   if (!ins || !outs) return fail(PCCL_ERR_INVALID_ARG, "operand array is null");
-  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  const int es = pccl_host::pccl_dtype_bytes(dtype);
   RcLaunch p;
   memset(&p, 0, sizeof(p));
   for (int k = 0; k < n_in; ++k) {
@@ -71,7 +72,7 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   if (rc != PCCL_OK) return rc;
   if (count == 0) return PCCL_OK;
   const pccl_host::Tuning t = pccl_host::tuning();
-  const int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+  const int es = pccl_host::pccl_dtype_bytes(dtype);
   // Operands that together exceed what the 256 MB Infinity Cache can hold run one
   // pack per lane under an occupancy cap (below).  Streaming hints start earlier,
   // at 48 MiB: a collective step works on data that just arrived and will not be
@@ -114,6 +115,8 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
     case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
     case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
     case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    default: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    case PCCL_F16: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    case PCCL_F8E4M3: return launch_typed<PCCL_F8E4M3>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    default: return launch_typed<PCCL_F8E5M2>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
   }
 }

@@ -23,6 +23,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // global_load_dwordx4 / global_store_dwordx4.
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -63,6 +64,7 @@ template <> struct Dtype<PCCL_F32> {
   static constexpr int kElemBytes = 4;
   typedef unsigned int elem_t;
   typedef u32x4_a4 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
   template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
     float acc = as_f32(w[0]);
 #pragma unroll
@@ -78,6 +80,7 @@ template <> struct Dtype<PCCL_I32> {
   static constexpr int kElemBytes = 4;
   typedef unsigned int elem_t;
   typedef u32x4_a4 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
   template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
     unsigned int acc = w[0];
 #pragma unroll
@@ -93,6 +96,7 @@ template <> struct Dtype<PCCL_BF16> {
   static constexpr int kElemBytes = 2;
   typedef unsigned short elem_t;
   typedef u32x4_a2 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
   // two bf16 per word: widen by shifting into the top half of a binary32,
   // fold both halves in float, round once (v_cvt_pk_bf16_f32: nearest even)
   template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
@@ -117,6 +121,7 @@ template <> struct Dtype<PCCL_F16> {
   static constexpr int kElemBytes = 2;
   typedef unsigned short elem_t;
   typedef u32x4_a2 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
   template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
     f32x2 acc = __builtin_convertvector(__builtin_bit_cast(f16x2, w[0]), f32x2);
 #pragma unroll
@@ -134,6 +139,85 @@ template <> struct Dtype<PCCL_F16> {
     return __builtin_bit_cast(unsigned short, (_Float16)acc);
   }
 };
+
+// 8-bit floats (OCP E4M3FN and E5M2), four per word.  Widening is the hardware's exact
+// v_cvt_f32_fp8 / v_cvt_f32_bf8; narrowing is v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 (round to
+// nearest even) with the wave's FP16_OVFL mode bit set, under which a finite value beyond the
+// largest finite one saturates to it instead of becoming NaN / infinity, NaN stays NaN and a
+// true infinity stays infinite (E5M2) or becomes NaN (E4M3FN, which has no infinity; no fold
+// of E4M3FN operands can produce one).  Checked against clamp-then-convert over all 2^32
+// binary32 patterns.  wave_init() must run once per wave before the first narrowing.
+template <bool E5M2> struct F8Fmt {
+  static __device__ __forceinline__ void wave_init() {
+    // MODE register (hwreg 1), bit 23 = FP16_OVFL; the clobber keeps loads (and so every
+    // conversion of loaded data) behind the mode change
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1" ::: "memory");
+  }
+  static __device__ __forceinline__ float up(unsigned int w, int byte) {
+    if constexpr (E5M2) {
+      switch (byte) {
+        case 0: return __builtin_amdgcn_cvt_f32_bf8(w, 0);
+        case 1: return __builtin_amdgcn_cvt_f32_bf8(w, 1);
+        case 2: return __builtin_amdgcn_cvt_f32_bf8(w, 2);
+        default: return __builtin_amdgcn_cvt_f32_bf8(w, 3);
+      }
+    } else {
+      switch (byte) {
+        case 0: return __builtin_amdgcn_cvt_f32_fp8(w, 0);
+        case 1: return __builtin_amdgcn_cvt_f32_fp8(w, 1);
+        case 2: return __builtin_amdgcn_cvt_f32_fp8(w, 2);
+        default: return __builtin_amdgcn_cvt_f32_fp8(w, 3);
+      }
+    }
+  }
+  // two at a time: bytes 0,1 (hi = false) or 2,3 (hi = true) of w
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  template <bool HI> static __device__ __forceinline__ f32x2 up2(unsigned int w) {
+    if constexpr (E5M2) return __builtin_amdgcn_cvt_pk_f32_bf8((int)w, HI);
+    else return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HI);
+  }
+  static __device__ __forceinline__ unsigned int down4(float a, float b, float c, float d) {
+    int p = 0;
+    if constexpr (E5M2) {
+      p = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, p, false);
+      p = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, p, true);
+    } else {
+      p = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p, false);
+      p = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, p, true);
+    }
+    return (unsigned int)p;
+  }
+};
+
+template <bool E5M2> struct DtypeF8 {
+  typedef F8Fmt<E5M2> F;
+  static constexpr int kElemBytes = 1;
+  typedef unsigned char elem_t;
+  typedef u32x4_a1 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() { F::wave_init(); }
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    typename F::f32x2 lo = F::template up2<false>(w[0]), hi = F::template up2<true>(w[0]);
+    float a = lo.x, b = lo.y, c = hi.x, d = hi.y;
+#pragma unroll
+    for (int k = 1; k < N; ++k) {
+      lo = F::template up2<false>(w[k]);
+      hi = F::template up2<true>(w[k]);
+      a = Op::f(a, lo.x);
+      b = Op::f(b, lo.y);
+      c = Op::f(c, hi.x);
+      d = Op::f(d, hi.y);
+    }
+    return F::down4(a, b, c, d);
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    float acc = F::up((unsigned int)e[0], 0);
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::f(acc, F::up((unsigned int)e[k], 0));
+    return (elem_t)(F::down4(acc, 0.0f, 0.0f, 0.0f) & 0xffu);
+  }
+};
+template <> struct Dtype<PCCL_F8E4M3> : DtypeF8<false> {};
+template <> struct Dtype<PCCL_F8E5M2> : DtypeF8<true> {};
 
 // ---- pack load / store -------------------------------------------------------
 // ALIGNED: every stream is 16-byte aligned.  Otherwise only output 0 is (the

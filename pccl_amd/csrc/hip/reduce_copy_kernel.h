@@ -27,6 +27,7 @@ __host__ __device__ constexpr int small_unroll_for(int n_in) { return n_in <= 2 
 template <int DT, class Op, int NIN, int UNROLL, bool ALIGNED, bool NT>
 __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
   typedef Dtype<DT> D;
+  if constexpr (NIN > 1) D::wave_init();
   constexpr int kEpp = 16 / D::kElemBytes;  // elements per pack
   if (p.n_packs > 0) {
     RcOperands body;
@@ -63,6 +64,7 @@ struct RcLean {
 template <int DT, class Op, int NIN, int NOUT, bool NT>
 __global__ void __launch_bounds__(kBlock) reduce_copy_lean_kernel(const RcLean<NIN, NOUT> a) {
   typedef Dtype<DT> D;
+  if constexpr (NIN > 1) D::wave_init();
   constexpr int kLd = (NT && NIN > 1) ? kMemStream : kMemCached;
   constexpr int kSt = NT ? kMemStream : kMemCached;
   const unsigned lane_off = threadIdx.x * 16u;

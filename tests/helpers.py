@@ -4,8 +4,9 @@ import numpy as np
 
 import pccl_oracle as orc
 
-ELEM_BYTES = {"f32": 4, "i32": 4, "bf16": 2, "f16": 2}
-STORAGE = {"f32": np.float32, "i32": np.int32, "bf16": np.uint16, "f16": np.uint16}
+ELEM_BYTES = {"f32": 4, "i32": 4, "bf16": 2, "f16": 2, "f8e4m3": 1, "f8e5m2": 1}
+STORAGE = {"f32": np.float32, "i32": np.int32, "bf16": np.uint16, "f16": np.uint16,
+           "f8e4m3": np.uint8, "f8e5m2": np.uint8}
 
 
 def gen(dtype, count, seed, stream, kind="normal", **kw):
