@@ -169,7 +169,11 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 
 /* signal_base the NEXT pccl_hip_graph_run of this graph will use: a party outside the
- * graph that wants to satisfy a GET_NOTIFIED(value) stores *base + value to the word. */
+ * graph that wants to satisfy a GET_NOTIFIED(value) stores *base + value to the word.
+ * The run number itself lives on the device and moves on with every execution of the
+ * drain kernel, so a pccl_hip_graph_run recorded into a HIP graph (stream capture) uses a
+ * fresh base on every replay; this call counts pccl_hip_graph_run calls only, and a
+ * caller that replays recorded runs adds 65536 per replay itself. */
 int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
 
 /* Bounds every wait inside the drain kernel to `polls` polls of a queue slot

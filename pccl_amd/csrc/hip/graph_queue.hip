@@ -82,7 +82,6 @@ struct GraphControl {
   int queue_count[kQueues];
   unsigned int spin_limit;
   int total_tiles;
-  unsigned int signal_base;               // run number << 16: added to the value of NOTIFY / GET_NOTIFIED ops
 };
 
 // indices into GraphControl::hot
@@ -91,7 +90,8 @@ constexpr int kHotTotal = 1;      // *layout.total_operator (never written durin
 constexpr int kHotAbort = 2;      // set when a bounded wait gave up
 constexpr int kHotExit = 3;       // workgroups that have left the current run
 constexpr int kHotDone = 4;       // kQueues counters of finished ops, summed at the end
-constexpr int kHotWords = kHotDone + kQueues;
+constexpr int kHotRun = kHotDone + kQueues;  // number of the current run (first run = 1), bumped by the last workgroup out
+constexpr int kHotWords = kHotRun + 1;
 
 // What a workgroup needs to run a part, on lines nothing writes during a run: the
 // op's payload plus the two header facts (part count, successor list) it would
@@ -242,6 +242,12 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   pccl_operation_layout_header *h = nullptr;
   const PayloadSlot *slot = nullptr;
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
+  // Signal values are offset by (run number << 16).  The run number lives on the device (not
+  // in the kernel arguments) so that a launch recorded into a HIP graph uses a fresh one on
+  // every replay; it is read at the first signal op, always before the last workgroup out of
+  // this run bumps it.
+  unsigned int signal_base = 0;
+  bool have_signal_base = false;
   for (;;) {
     if (threadIdx.x == 0) {
       // The part executed in the previous iteration is complete (barrier below): every
@@ -283,7 +289,11 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         const int prim = sc->payload.primitive_;
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
-        const unsigned int want = g.signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
+        if (!have_signal_base) {
+          signal_base = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT) << 16;
+          have_signal_base = true;
+        }
+        const unsigned int want = signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
         if (prim == PCCL_NOTIFY) {
           // everything this op depends on is already at the point of coherence
           __hip_atomic_store(sig, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -338,6 +348,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
     }
     __hip_atomic_store(&hot[kHotCompleted].value, done, __ATOMIC_RELAXED, AGENT);
     __hip_atomic_store(&hot[kHotExit].value, 0u, __ATOMIC_RELAXED, AGENT);
+    __hip_atomic_fetch_add(&hot[kHotRun].value, 1u, __ATOMIC_RELAXED, AGENT);
   }
 }
 
@@ -557,6 +568,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   C->total_tiles = (int)tiles;
   hot[kHotCompleted].value = 0;
   hot[kHotTotal].value = (unsigned int)n_ops;
+  hot[kHotRun].value = 1;
 
   // deal the entries round-robin onto the queues, in global order
   std::vector<std::vector<unsigned long long>> qe(kQueues);
@@ -647,7 +659,6 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   {
     std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
     memcpy(&control, G->image.data(), sizeof(control));
-    control.signal_base = (G->runs + 1u) << 16;
     ++G->runs;
   }
   hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
@@ -670,6 +681,9 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed, un
     // put the pristine state back so that the graph can be used again
     std::lock_guard<std::mutex> lock(G->mu);
     PCCL_HIP_CHECK(hipMemcpy(G->dev, G->image.data(), G->image.size(), hipMemcpyHostToDevice));
+    // ... except the run number, which the aborted run has already moved on
+    PCCL_HIP_CHECK(hipMemcpy(G->dev + off_hot + sizeof(HotWord) * kHotRun, &hot[kHotRun], sizeof(HotWord),
+                             hipMemcpyHostToDevice));
     return fail(PCCL_ERR_GRAPH, "drain gave up: an op's dependencies were not satisfied within the spin limit "
                                 "(%u of %u ops had completed); graph state was reset",
                 hot[kHotCompleted].value, hot[kHotTotal].value);

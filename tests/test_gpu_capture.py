@@ -1,0 +1,91 @@
+"""The asynchronous entry points recorded into a HIP graph by stream capture (torch.cuda.graph)
+and replayed: they allocate nothing, synchronise nothing and enqueue no memset, so a replay is
+just their kernels.  Every replay runs on fresh inputs, with eager work and synchronisation in
+between, and is checked bit for bit against the CPU checker."""
+import numpy as np
+import pytest
+
+import helpers as H
+from test_gpu_graph import _signal_ring_ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _capture(torch, record):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        record(side.cuda_stream)            # warm-up on the capture stream (module load etc.)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        record(torch.cuda.current_stream().cuda_stream)
+    return graph
+
+
+def test_reduce_copy_and_accumulate_replay(hip, oracle):
+    import torch
+    n = 1_000_003
+    d_in = [H.DevBuf(torch, "bf16", n, offset=2 * k) for k in range(3)]
+    d_sum = H.DevBuf(torch, "bf16", n)
+    d_acc = [H.DevBuf(torch, "bf16", n, offset=4), H.DevBuf(torch, "bf16", n)]
+
+    def record(stream):
+        hip.reduce_copy("bf16", "sum", [b.ptr for b in d_in], [d_sum.ptr], n, stream)
+        hip.accumulate("bf16", "sum", d_sum.ptr, [b.ptr for b in d_acc], n, stream)
+
+    graph = _capture(torch, record)
+    for it in range(3):
+        ins = [H.gen("bf16", n, 200 + it, k) for k in range(3)]
+        acc0 = [H.gen("bf16", n, 200 + it, 3 + k) for k in range(2)]
+        for b, a in zip(d_in + d_acc, ins + acc0):
+            b.upload(a)
+        d_sum.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle.reduce("bf16", "sum", ins)
+        H.assert_bits_equal(d_sum.download(), want, "replay %d sum" % it)
+        for k in range(2):
+            H.assert_bits_equal(d_acc[k].download(), oracle.reduce("bf16", "sum", [acc0[k], want]),
+                                "replay %d destination %d" % (it, k))
+            assert d_acc[k].guards_intact()
+
+
+def test_queue_run_with_signal_ops_replay(hip, oracle):
+    """A ring whose virtual ranks are linked only by NOTIFY / GET_NOTIFIED, recorded once: each
+    replay must use a fresh run number, or the waits would be satisfied by the previous replay's
+    signal values before the data is there."""
+    import torch
+    world, size = 8, 3001
+    per = world * size
+    d_in = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    d_out = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    signals = torch.zeros(64, dtype=torch.int32, device="cuda")
+    ops, sym = _signal_ring_ops(world, size, signals.data_ptr(), d_in, d_out)
+    g = hip.Graph(ops)
+    graph = _capture(torch, lambda stream: g.run(stream))   # the warm-up inside is run 1, the recording run 2
+    seen = []
+    for it in range(3):
+        ins = [H.gen("bf16", per, 300 + 10 * it, r) for r in range(world)]
+        outs = [np.zeros(per, dtype=np.uint16) for _ in range(world)]
+        bufs = {"in": ins, "out": outs}
+        for i in sorted(sym):
+            o = sym[i]
+            oracle.reduce_copy("bf16", "sum", [bufs[b][r][e:e + size] for (b, r, e) in o["ins"]],
+                               [bufs[b][r][e:e + size] for (b, r, e) in o["outs"]])
+        for r in range(world):
+            d_in[r].upload(ins[r])
+            d_out[r].view().fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert g.status(torch.cuda.current_stream().cuda_stream) == (len(ops), len(ops))
+        for r in range(world):
+            H.assert_bits_equal(d_out[r].download(), outs[r], "replay %d rank %d" % (it, r))
+        word = signals[:world].cpu().tolist()
+        assert len(set(word)) == 1
+        seen.append(word[0])
+    # consecutive replays used consecutive run numbers
+    assert [b - a for a, b in zip(seen, seen[1:])] == [1 << 16, 1 << 16]
+    g.destroy()
