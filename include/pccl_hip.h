@@ -103,7 +103,8 @@ int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *out
                         void *stream);
 
 /* Launch-shape overrides for tuning runs: workgroups per compute unit
- * (0 = built-in choice) and non-temporal access hint (0/1, -1 = built-in). */
+ * (0 = built-in choice) and cache treatment (-1 = built-in choice, 0 = cacheable,
+ * 1 = non-temporal loads and stores, 2 = non-temporal loads and write-through stores). */
 int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);
 
 /* Occupancy override for tuning runs: bytes of (unused) dynamic LDS requested per

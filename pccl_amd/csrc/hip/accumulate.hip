@@ -10,7 +10,7 @@
 #include <cstring>
 
 #include "plugin_common.h"
-#include "reduce_copy_device.h"
+#include "reduce_copy_kernel.h"
 
 using namespace pccl_dev;
 using pccl_host::fail;
@@ -27,10 +27,11 @@ struct AccLaunch {
 };
 
 // ALIGNED: input and every output 16-byte aligned after the head peel.
-// NT: streaming hints, for operands beyond the Infinity Cache.
-template <int DT, class Op, bool ALIGNED, bool NT>
+// MEM: cache treatment as for reduce_copy (0 cacheable, 1 streaming, 2 streaming loads and
+// write-through stores).
+template <int DT, class Op, bool ALIGNED, int MEM>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
-  constexpr int kMem = NT ? kMemStream : kMemCached;
+  constexpr int kLd = LaunchMem<MEM, 2>::kLd, kSt = LaunchMem<MEM, 2>::kSt;
   typedef Dtype<DT> D;
   D::wave_init();
   typedef typename D::elem_t E;
@@ -39,15 +40,15 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   if (pack < p.n_packs) {
     const long off = p.head * D::kElemBytes + pack * 16;
     u32x4 v[2];
-    v[1] = load_pack<D, ALIGNED, kMem>(p.in + off);
+    v[1] = load_pack<D, ALIGNED, kLd>(p.in + off);
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.n_out) {
         // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
-        v[0] = j == 0 ? load_pack<D, true, kMem>(p.out[0] + off) : load_pack<D, ALIGNED, kMem>(p.out[j] + off);
+        v[0] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + off) : load_pack<D, ALIGNED, kLd>(p.out[j] + off);
         const u32x4 r = fold_pack<D, Op, 2>(v);
-        if (j == 0) store_pack<D, true, kMem>(p.out[0] + off, r);
-        else store_pack<D, ALIGNED, kMem>(p.out[j] + off, r);
+        if (j == 0) store_pack<D, true, kSt>(p.out[0] + off, r);
+        else store_pack<D, ALIGNED, kSt>(p.out[j] + off, r);
       }
   }
   // head and tail elements: the last wavefront of the last workgroup
@@ -69,27 +70,25 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
 }
 
 template <int DT, class Op>
-int launch_acc(bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const AccLaunch &p) {
-  if (aligned) {
-    if (nt) hipLaunchKernelGGL((accumulate_kernel<DT, Op, true, true>), dim3(grid), dim3(kBlock), lds, stream, p);
-    else hipLaunchKernelGGL((accumulate_kernel<DT, Op, true, false>), dim3(grid), dim3(kBlock), lds, stream, p);
-  } else {
-    if (nt) hipLaunchKernelGGL((accumulate_kernel<DT, Op, false, true>), dim3(grid), dim3(kBlock), lds, stream, p);
-    else hipLaunchKernelGGL((accumulate_kernel<DT, Op, false, false>), dim3(grid), dim3(kBlock), lds, stream, p);
-  }
+int launch_acc(bool aligned, int mem, unsigned grid, unsigned lds, hipStream_t stream, const AccLaunch &p) {
+  with_launch_mem(mem, [&](auto m) {
+    constexpr int kMem = decltype(m)::value;
+    if (aligned) hipLaunchKernelGGL((accumulate_kernel<DT, Op, true, kMem>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((accumulate_kernel<DT, Op, false, kMem>), dim3(grid), dim3(kBlock), lds, stream, p);
+  });
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "accumulate launch failed: %s", hipGetErrorString(e));
   return PCCL_OK;
 }
 
 template <int DT>
-int launch_acc_op(int compute, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream,
+int launch_acc_op(int compute, bool aligned, int mem, unsigned grid, unsigned lds, hipStream_t stream,
                   const AccLaunch &p) {
   switch (compute) {
-    case PCCL_SUM: return launch_acc<DT, OpSum>(aligned, nt, grid, lds, stream, p);
-    case PCCL_PROD: return launch_acc<DT, OpProd>(aligned, nt, grid, lds, stream, p);
-    case PCCL_MIN: return launch_acc<DT, OpMin>(aligned, nt, grid, lds, stream, p);
-    default: return launch_acc<DT, OpMax>(aligned, nt, grid, lds, stream, p);
+    case PCCL_SUM: return launch_acc<DT, OpSum>(aligned, mem, grid, lds, stream, p);
+    case PCCL_PROD: return launch_acc<DT, OpProd>(aligned, mem, grid, lds, stream, p);
+    case PCCL_MIN: return launch_acc<DT, OpMin>(aligned, mem, grid, lds, stream, p);
+    default: return launch_acc<DT, OpMax>(aligned, mem, grid, lds, stream, p);
   }
 }
 
@@ -124,26 +123,33 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
   bool aligned = (((uintptr_t)in + (uintptr_t)p.head * es) & 15) == 0;
   for (int j = 0; j < n_out; ++j) aligned = aligned && (((uintptr_t)outs[j] + (uintptr_t)p.head * es) & 15) == 0;
   const unsigned grid = (unsigned)std::max<long>(1, (p.n_packs + kBlock - 1) / kBlock);
-  // Launch policy, measured on MI355X with 128 MiB operands.  A lane handles its
-  // destinations one after the other (a store to one may alias a load of the next), so
-  // only two loads are in flight per lane and the kernel wants more resident workgroups
-  // than reduce_copy does: streaming hints pay from two destinations on (6.3 vs 5.8 TB/s;
-  // with one destination the read-modify-write prefers cached accesses, 7.0 vs 6.2), and a
-  // cap of 5 workgroups per compute unit pays from three destinations on (1 -> 7: 6.4 vs
-  // 5.5 TB/s uncapped, 4.6 with 2 workgroups).
+  // Launch policy, measured on MI355X.  A lane handles its destinations one after the
+  // other (a store to one may alias a load of the next), so only two loads are in flight
+  // per lane and the kernel wants more resident workgroups than reduce_copy does.  One
+  // destination: the read-modify-write prefers cached accesses (7.2 vs 6.5 TB/s at
+  // 128 MiB).  Two: streaming loads with write-through stores beyond the Infinity Cache
+  // (7.1 vs 6.5 with non-temporal stores, 5.8 cached), non-temporal stores below.  Three and more: cached while input and
+  // destinations fit the 256 MB Infinity Cache together (1 -> 7 at 32 MiB: 7.05 vs 6.1),
+  // else non-temporal loads and stores (1 -> 7 at 128 MiB: 6.45 vs 6.2 write-through,
+  // 5.85 cached) under a cap of 5 workgroups per compute unit (6.4 vs 5.5 uncapped).
   const pccl_host::Tuning t = pccl_host::tuning();
   const long total_bytes = (long)(1 + 2 * n_out) * count * es;
-  const bool nt = t.nontemporal < 0 ? (n_out >= 2 && total_bytes >= (48l << 20)) : t.nontemporal != 0;
+  const long working_set = (long)(1 + n_out) * count * es;
+  int mem = kLaunchMemCached;
+  if (n_out == 2 && total_bytes >= (48l << 20))
+    mem = total_bytes > (192l << 20) ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
+  else if (n_out >= 3 && working_set > (256l << 20)) mem = kLaunchMemStream;
+  if (t.nontemporal >= 0) mem = std::min(t.nontemporal, (int)kLaunchMemStreamWriteThrough);
   unsigned lds = 0;
   if (t.lds_bytes >= 0) lds = (unsigned)t.lds_bytes;
   else if (n_out >= 3 && total_bytes > (192l << 20)) lds = 160 * 1024 / 5 - 256;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, nt, grid, lds, s, p);
-    case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, nt, grid, lds, s, p);
-    case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, nt, grid, lds, s, p);
-    case PCCL_F16: return launch_acc_op<PCCL_F16>(compute, aligned, nt, grid, lds, s, p);
-    case PCCL_F8E4M3: return launch_acc_op<PCCL_F8E4M3>(compute, aligned, nt, grid, lds, s, p);
-    default: return launch_acc_op<PCCL_F8E5M2>(compute, aligned, nt, grid, lds, s, p);
+    case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_I32: return launch_acc_op<PCCL_I32>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_F16: return launch_acc_op<PCCL_F16>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_F8E4M3: return launch_acc_op<PCCL_F8E4M3>(compute, aligned, mem, grid, lds, s, p);
+    default: return launch_acc_op<PCCL_F8E5M2>(compute, aligned, mem, grid, lds, s, p);
   }
 }

@@ -3,6 +3,7 @@
 // deallocate (reference csrc/plugins/cuda_executor/device.cc:53-144): sizes are
 // rounded up to 2 MiB (:60,70), nbytes <= 0 gives a null pointer (:61), live
 // allocations are tracked in a pointer-keyed map under a mutex (:50-51,121-144).
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -48,7 +49,7 @@ Tuning tuning() {
   if (!g_tuning_env_read) {  // same knobs the host plugin lists as launch options
     g_tuning_env_read = true;
     if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tuning.workgroups_per_cu = atoi(s);
-    if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.nontemporal = atoi(s) ? 1 : 0;
+    if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.nontemporal = std::max(0, std::min(2, atoi(s)));
     if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tuning.lds_bytes = atoi(s);
     if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tuning.unroll = atoi(s);
   }
@@ -135,7 +136,7 @@ int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal) {
   (void)tuning();  // make sure the environment was read before overriding it
   std::lock_guard<std::mutex> lock(g_tuning_mutex);
   g_tuning.workgroups_per_cu = workgroups_per_cu;
-  g_tuning.nontemporal = nontemporal < 0 ? -1 : (nontemporal ? 1 : 0);
+  g_tuning.nontemporal = nontemporal < 0 ? -1 : std::min(nontemporal, 2);
   return PCCL_OK;
 }
 

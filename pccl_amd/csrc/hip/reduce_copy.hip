@@ -7,12 +7,12 @@
 
 namespace pccl_dev {
 
-int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
+int launch_copy(int elem_bytes, int unroll, bool aligned, int mem, unsigned grid, unsigned lds,
                 hipStream_t stream, const RcLaunch &p) {
   // the dtype only selects the element size and the alignment the unaligned pack type may assume
-  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
-  if (elem_bytes == 2) return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
-  return launch_nin<PCCL_F8E4M3, OpSum, 1>(unroll, aligned, nt, grid, lds, stream, p);
+  if (elem_bytes == 4) return launch_nin<PCCL_F32, OpSum, 1>(unroll, aligned, mem, grid, lds, stream, p);
+  if (elem_bytes == 2) return launch_nin<PCCL_BF16, OpSum, 1>(unroll, aligned, mem, grid, lds, stream, p);
+  return launch_nin<PCCL_F8E4M3, OpSum, 1>(unroll, aligned, mem, grid, lds, stream, p);
 }
 
 }  // namespace pccl_dev
@@ -74,13 +74,26 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   const pccl_host::Tuning t = pccl_host::tuning();
   const int es = pccl_host::pccl_dtype_bytes(dtype);
   // Operands that together exceed what the 256 MB Infinity Cache can hold run one
-  // pack per lane under an occupancy cap (below).  Streaming hints start earlier,
+  // pack per lane under an occupancy cap (below).  Streaming treatment starts earlier,
   // at 48 MiB: a collective step works on data that just arrived and will not be
-  // touched again soon (measured on a walk over 7 x 32 MiB ring steps: copy steps
-  // 5.0 -> 6.05 TB/s, reduce steps 5.5 -> 5.6 TB/s); smaller operands stay cacheable.
+  // touched again soon; smaller operands stay cacheable.  Which streaming treatment
+  // (measured on MI355X in steady state, TB/s with non-temporal vs write-through
+  // stores): reductions beyond the Infinity Cache prefer write-through stores (8 -> 1 at
+  // 256 MiB 6.5 vs 6.6, 8 -> 2 at 128 MiB 6.5 vs 6.8, 4 -> 1 6.3 vs 6.7, 2 -> 1 6.6 vs
+  // 7.2); copies prefer non-temporal stores (1 -> 1 at 256 MiB 7.3 vs 6.1), and so do
+  // reductions over several GiB (i32 4 -> 1 at 1 GiB per operand 6.1 vs 6.0, unaligned
+  // 5.9 vs 5.4).  Between 48 and 192 MiB write-through stores look better on a step
+  // that is repeated in place (2 -> 2 at 32 MiB 6.0 vs 6.9) but leave the caches in a
+  // state the NEXT kernel pays for: a walk over 14 ring steps of 32 MiB takes 239 us
+  // with non-temporal stores throughout and 256 us with write-through reductions.
   const long total_bytes = (long)(n_in + n_out) * count * es;
   const bool big = total_bytes > (192l << 20);
-  const bool nt = t.nontemporal < 0 ? total_bytes >= (48l << 20) : t.nontemporal != 0;
+  int mem = kLaunchMemCached;
+  if (total_bytes >= (48l << 20)) {
+    const bool write_through = n_in > 1 && big && total_bytes <= (4l << 30);
+    mem = write_through ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
+  }
+  if (t.nontemporal >= 0) mem = std::min(t.nontemporal, (int)kLaunchMemStreamWriteThrough);
   int unroll = big ? 1 : small_unroll_for(n_in);
   if (t.unroll == 1 || t.unroll == 4) unroll = t.unroll == 4 ? small_unroll_for(n_in) : 1;
   // lean kernel: nothing to peel, at most two outputs, and no gain expected from
@@ -110,13 +123,13 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
     if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
   }
   hipStream_t s = (hipStream_t)stream;
-  if (n_in == 1) return launch_copy(es, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+  if (n_in == 1) return launch_copy(es, unroll, aligned, mem, (unsigned)grid, lds, s, p);
   switch (dtype) {
-    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    case PCCL_F16: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    case PCCL_F8E4M3: return launch_typed<PCCL_F8E4M3>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
-    default: return launch_typed<PCCL_F8E5M2>(compute, n_in, unroll, aligned, nt, (unsigned)grid, lds, s, p);
+    case PCCL_F32: return launch_typed<PCCL_F32>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
+    case PCCL_I32: return launch_typed<PCCL_I32>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
+    case PCCL_BF16: return launch_typed<PCCL_BF16>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
+    case PCCL_F16: return launch_typed<PCCL_F16>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
+    case PCCL_F8E4M3: return launch_typed<PCCL_F8E4M3>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
+    default: return launch_typed<PCCL_F8E5M2>(compute, n_in, unroll, aligned, mem, (unsigned)grid, lds, s, p);
   }
 }

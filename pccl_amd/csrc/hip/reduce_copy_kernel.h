@@ -3,6 +3,8 @@
 // the dtype x compute x n_in matrix compiles in parallel.
 #pragma once
 
+#include <type_traits>
+
 #include "plugin_common.h"
 #include "reduce_copy_device.h"
 
@@ -22,9 +24,27 @@ struct RcLaunch {
 // 2-input reductions gain (about 5 %) from 4 packs per lane.
 __host__ __device__ constexpr int small_unroll_for(int n_in) { return n_in <= 2 ? 4 : 1; }
 
-// NT: streaming hint.  Reductions apply it to loads and stores, a copy to its
-// stores only.
-template <int DT, class Op, int NIN, int UNROLL, bool ALIGNED, bool NT>
+// MEM: how the launch treats the caches (host-side choice by operand size and shape).
+//   0  everything cacheable;
+//   1  streaming: non-temporal loads and stores (a copy: stores only);
+//   2  streaming loads (a copy: cacheable loads), write-through (sc1) stores.  Measured on
+//      MI355X this beats 1 wherever the stores compete with many load streams for the
+//      L2: bf16 8 -> 1 at 256 MiB 6.62 -> 6.86 TB/s, 2 -> 2 at 32 MiB 5.5 -> 6.4 TB/s.
+constexpr int kLaunchMemCached = 0, kLaunchMemStream = 1, kLaunchMemStreamWriteThrough = 2;
+template <int MEM, int NIN> struct LaunchMem {
+  static constexpr int kLd = (MEM != kLaunchMemCached && NIN > 1) ? kMemStream : kMemCached;
+  static constexpr int kSt = MEM == kLaunchMemCached ? kMemCached : MEM == kLaunchMemStream ? kMemStream : kMemCoherent;
+};
+
+// Calls f(std::integral_constant<int, mem>) for mem in 0..2.
+template <class F>
+inline void with_launch_mem(int mem, F &&f) {
+  if (mem == kLaunchMemStreamWriteThrough) f(std::integral_constant<int, kLaunchMemStreamWriteThrough>{});
+  else if (mem == kLaunchMemStream) f(std::integral_constant<int, kLaunchMemStream>{});
+  else f(std::integral_constant<int, kLaunchMemCached>{});
+}
+
+template <int DT, class Op, int NIN, int UNROLL, bool ALIGNED, int MEM>
 __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
   typedef Dtype<DT> D;
   if constexpr (NIN > 1) D::wave_init();
@@ -37,7 +57,7 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_kernel(const RcLaunch p) {
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.ops.n_out) body.out[j] = p.ops.out[j] + p.head * D::kElemBytes;
-    body_packs<D, Op, NIN, UNROLL, ALIGNED, (NT && NIN > 1) ? kMemStream : kMemCached, NT ? kMemStream : kMemCached>(
+    body_packs<D, Op, NIN, UNROLL, ALIGNED, LaunchMem<MEM, NIN>::kLd, LaunchMem<MEM, NIN>::kSt>(
         body, p.n_packs, blockIdx.x, gridDim.x);
   }
   // head and tail elements: the last wavefront of the last workgroup
@@ -61,12 +81,12 @@ struct RcLean {
   long n_packs;
 };
 
-template <int DT, class Op, int NIN, int NOUT, bool NT>
+template <int DT, class Op, int NIN, int NOUT, int MEM>
 __global__ void __launch_bounds__(kBlock) reduce_copy_lean_kernel(const RcLean<NIN, NOUT> a) {
   typedef Dtype<DT> D;
   if constexpr (NIN > 1) D::wave_init();
-  constexpr int kLd = (NT && NIN > 1) ? kMemStream : kMemCached;
-  constexpr int kSt = NT ? kMemStream : kMemCached;
+  constexpr int kLd = LaunchMem<MEM, NIN>::kLd;
+  constexpr int kSt = LaunchMem<MEM, NIN>::kSt;
   const unsigned lane_off = threadIdx.x * 16u;
   const size_t wg_off = (size_t)blockIdx.x * (kBlock * 16);
   if ((long)blockIdx.x * kBlock + threadIdx.x < a.n_packs) {
@@ -80,14 +100,15 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_lean_kernel(const RcLean<N
 }
 
 template <int DT, class Op, int NIN, int NOUT>
-int launch_lean_nout(bool nt, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+int launch_lean_nout(int mem, unsigned lds, hipStream_t stream, const RcLaunch &p) {
   RcLean<NIN, NOUT> a;
   for (int k = 0; k < NIN; ++k) a.in[k] = p.ops.in[k];
   for (int j = 0; j < NOUT; ++j) a.out[j] = p.ops.out[j];
   a.n_packs = p.n_packs;
   const unsigned grid = (unsigned)((p.n_packs + kBlock - 1) / kBlock);
-  if (nt) hipLaunchKernelGGL((reduce_copy_lean_kernel<DT, Op, NIN, NOUT, true>), dim3(grid), dim3(kBlock), lds, stream, a);
-  else hipLaunchKernelGGL((reduce_copy_lean_kernel<DT, Op, NIN, NOUT, false>), dim3(grid), dim3(kBlock), lds, stream, a);
+  with_launch_mem(mem, [&](auto m) {
+    hipLaunchKernelGGL((reduce_copy_lean_kernel<DT, Op, NIN, NOUT, decltype(m)::value>), dim3(grid), dim3(kBlock), lds, stream, a);
+  });
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return pccl_host::fail(PCCL_ERR_HIP, "reduce_copy launch failed: %s", hipGetErrorString(e));
@@ -96,20 +117,18 @@ int launch_lean_nout(bool nt, unsigned lds, hipStream_t stream, const RcLaunch &
 
 // requires: p.head == 0, p.n_packs * pack == p.count, all streams aligned, n_out <= 2
 template <int DT, class Op, int NIN>
-int launch_lean(bool nt, unsigned lds, hipStream_t stream, const RcLaunch &p) {
-  if (p.ops.n_out == 1) return launch_lean_nout<DT, Op, NIN, 1>(nt, lds, stream, p);
-  return launch_lean_nout<DT, Op, NIN, 2>(nt, lds, stream, p);
+int launch_lean(int mem, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  if (p.ops.n_out == 1) return launch_lean_nout<DT, Op, NIN, 1>(mem, lds, stream, p);
+  return launch_lean_nout<DT, Op, NIN, 2>(mem, lds, stream, p);
 }
 
 template <int DT, class Op, int NIN, int UNROLL>
-int launch_shape(bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
-  if (aligned) {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, true>), dim3(grid), dim3(kBlock), lds, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, false>), dim3(grid), dim3(kBlock), lds, stream, p);
-  } else {
-    if (nt) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, true>), dim3(grid), dim3(kBlock), lds, stream, p);
-    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, false>), dim3(grid), dim3(kBlock), lds, stream, p);
-  }
+int launch_shape(bool aligned, int mem, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  with_launch_mem(mem, [&](auto m) {
+    constexpr int kMem = decltype(m)::value;
+    if (aligned) hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, true, kMem>), dim3(grid), dim3(kBlock), lds, stream, p);
+    else hipLaunchKernelGGL((reduce_copy_kernel<DT, Op, NIN, UNROLL, false, kMem>), dim3(grid), dim3(kBlock), lds, stream, p);
+  });
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return pccl_host::fail(PCCL_ERR_HIP, "reduce_copy launch failed: %s", hipGetErrorString(e));
@@ -118,47 +137,47 @@ int launch_shape(bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t
 
 // unroll is 0 (lean kernel), 1 or small_unroll_for(NIN); the last two coincide for n_in >= 3
 template <int DT, class Op, int NIN>
-int launch_nin(int unroll, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
-  if (unroll == 0) return launch_lean<DT, Op, NIN>(nt, lds, stream, p);
+int launch_nin(int unroll, bool aligned, int mem, unsigned grid, unsigned lds, hipStream_t stream, const RcLaunch &p) {
+  if (unroll == 0) return launch_lean<DT, Op, NIN>(mem, lds, stream, p);
   if constexpr (small_unroll_for(NIN) != 1) {
-    if (unroll != 1) return launch_shape<DT, Op, NIN, small_unroll_for(NIN)>(aligned, nt, grid, lds, stream, p);
+    if (unroll != 1) return launch_shape<DT, Op, NIN, small_unroll_for(NIN)>(aligned, mem, grid, lds, stream, p);
   }
-  return launch_shape<DT, Op, NIN, 1>(aligned, nt, grid, lds, stream, p);
+  return launch_shape<DT, Op, NIN, 1>(aligned, mem, grid, lds, stream, p);
 }
 
 template <int DT, class Op>
-int launch_op(int n_in, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds, hipStream_t stream,
+int launch_op(int n_in, int unroll, bool aligned, int mem, unsigned grid, unsigned lds, hipStream_t stream,
               const RcLaunch &p) {
   switch (n_in) {
-    case 2: return launch_nin<DT, Op, 2>(unroll, aligned, nt, grid, lds, stream, p);
-    case 3: return launch_nin<DT, Op, 3>(unroll, aligned, nt, grid, lds, stream, p);
-    case 4: return launch_nin<DT, Op, 4>(unroll, aligned, nt, grid, lds, stream, p);
-    case 5: return launch_nin<DT, Op, 5>(unroll, aligned, nt, grid, lds, stream, p);
-    case 6: return launch_nin<DT, Op, 6>(unroll, aligned, nt, grid, lds, stream, p);
-    case 7: return launch_nin<DT, Op, 7>(unroll, aligned, nt, grid, lds, stream, p);
-    case 8: return launch_nin<DT, Op, 8>(unroll, aligned, nt, grid, lds, stream, p);
+    case 2: return launch_nin<DT, Op, 2>(unroll, aligned, mem, grid, lds, stream, p);
+    case 3: return launch_nin<DT, Op, 3>(unroll, aligned, mem, grid, lds, stream, p);
+    case 4: return launch_nin<DT, Op, 4>(unroll, aligned, mem, grid, lds, stream, p);
+    case 5: return launch_nin<DT, Op, 5>(unroll, aligned, mem, grid, lds, stream, p);
+    case 6: return launch_nin<DT, Op, 6>(unroll, aligned, mem, grid, lds, stream, p);
+    case 7: return launch_nin<DT, Op, 7>(unroll, aligned, mem, grid, lds, stream, p);
+    case 8: return launch_nin<DT, Op, 8>(unroll, aligned, mem, grid, lds, stream, p);
     default: return pccl_host::fail(PCCL_ERR_INVALID_ARG, "n_in %d outside [1, 8]", n_in);
   }
 }
 
 // n_in >= 2.  Defined once per dtype (reduce_copy_inst_*.hip).
 template <int DT>
-int launch_typed(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
+int launch_typed(int compute, int n_in, int unroll, bool aligned, int mem, unsigned grid, unsigned lds,
                  hipStream_t stream, const RcLaunch &p);
 
 // n_in == 1: bytes move unchanged, so only the element size matters.
-int launch_copy(int elem_bytes, int unroll, bool aligned, bool nt, unsigned grid, unsigned lds,
+int launch_copy(int elem_bytes, int unroll, bool aligned, int mem, unsigned grid, unsigned lds,
                 hipStream_t stream, const RcLaunch &p);
 
 #define PCCL_DEFINE_LAUNCH_TYPED(DT)                                                            \
   template <>                                                                                   \
-  int launch_typed<DT>(int compute, int n_in, int unroll, bool aligned, bool nt, unsigned grid, \
+  int launch_typed<DT>(int compute, int n_in, int unroll, bool aligned, int mem, unsigned grid, \
                        unsigned lds, hipStream_t stream, const RcLaunch &p) {                   \
     switch (compute) {                                                                          \
-      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
-      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, unroll, aligned, nt, grid, lds, stream, p);         \
-      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
-      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, unroll, aligned, nt, grid, lds, stream, p);           \
+      case PCCL_SUM: return launch_op<DT, OpSum>(n_in, unroll, aligned, mem, grid, lds, stream, p);           \
+      case PCCL_PROD: return launch_op<DT, OpProd>(n_in, unroll, aligned, mem, grid, lds, stream, p);         \
+      case PCCL_MIN: return launch_op<DT, OpMin>(n_in, unroll, aligned, mem, grid, lds, stream, p);           \
+      case PCCL_MAX: return launch_op<DT, OpMax>(n_in, unroll, aligned, mem, grid, lds, stream, p);           \
       default: return pccl_host::fail(PCCL_ERR_UNSUPPORTED, "unknown compute code %d", compute); \
     }                                                                                           \
   }

@@ -61,3 +61,25 @@ def test_accumulate_errors(hip):
         hip.accumulate(7, "sum", t, [u], 8)
     assert e.value.code == hip.ERR_UNSUPPORTED
     hip.accumulate("f32", "sum", t, [u], 0)
+
+
+def test_cache_treatments_through_the_knob(hip, oracle):
+    """Cache treatment 0 / 1 / 2 (chosen from operand sizes in normal use) forced on small inputs."""
+    import torch
+    n = 70001
+    try:
+        for dtype, n_out, off in (("bf16", 1, 0), ("bf16", 3, 2), ("f32", 2, 4), ("f8e5m2", 7, 1)):
+            src = H.gen(dtype, n, 70, 0)
+            dst0 = [H.gen(dtype, n, 70, 1 + k) for k in range(n_out)]
+            for mem in (0, 1, 2):
+                hip.set_tuning(0, mem)
+                d_src = H.DevBuf(torch, dtype, n, src=src, offset=off)
+                d_dst = [H.DevBuf(torch, dtype, n, src=x, offset=(off * (k + 1)) % 64) for k, x in enumerate(dst0)]
+                hip.accumulate(dtype, "sum", d_src.ptr, [x.ptr for x in d_dst], n, torch.cuda.current_stream().cuda_stream)
+                torch.cuda.synchronize()
+                for k, x in enumerate(d_dst):
+                    H.assert_bits_equal(x.download(), oracle.reduce(dtype, "sum", [dst0[k], src]),
+                                        "%s 1->%d mem=%d dst %d" % (dtype, n_out, mem, k))
+                    assert x.guards_intact()
+    finally:
+        hip.set_tuning(0, -1)

@@ -162,3 +162,34 @@ def test_argument_errors(hip):
     assert e.value.code == hip.ERR_INVALID_ARG
     hip.reduce_copy("f32", "sum", [t], [t], 0)  # empty op is a no-op
     torch.cuda.synchronize()
+
+
+def test_every_kernel_variant_through_the_knobs(hip, oracle):
+    """The launch policy picks cache treatment, kernel shape and occupancy cap from operand sizes
+    that only large runs reach; the tuning knobs force each variant on small ragged inputs:
+    cache treatment 0 (cacheable) / 1 (non-temporal) / 2 (non-temporal loads, write-through
+    stores) x lean / 1 pack per lane / 4 packs per lane x full grid / persistent grid."""
+    import torch
+    cases = [("bf16", 8, 1, 256 * 8 * 5, 0), ("bf16", 3, 2, 70001, 2), ("f32", 2, 1, 4099, 4), ("f32", 2, 3, 1 << 16, 0),
+             ("i32", 4, 1, 131071, 12), ("f16", 1, 2, 50001, 6), ("f8e4m3", 5, 1, 30011, 3), ("bf16", 1, 1, 1 << 17, 0)]
+    try:
+        for dtype, n_in, n_out, count, off in cases:
+            ins = _inputs(dtype, "sum", n_in, count, seed=300 + n_in)
+            want = oracle.reduce(dtype, "sum", ins)
+            offs_in = [(off * (k + 1)) % 64 for k in range(n_in)]
+            offs_out = [(off * (k + 2)) % 64 for k in range(n_out)]
+            for mem in (0, 1, 2):
+                for unroll in (0, 1, 4):
+                    for wg in (0, 2):
+                        hip.set_tuning(wg, mem)
+                        hip.set_unroll(unroll)
+                        hip.set_occupancy_lds(65536 if wg == 0 else 0)
+                        got = H.hip_reduce(torch, hip, dtype, "sum", ins, n_out=n_out, in_offsets=offs_in,
+                                           out_offsets=offs_out)
+                        for g in got:
+                            H.assert_bits_equal(g, want, "%s %d->%d count=%d mem=%d unroll=%d wg=%d"
+                                                % (dtype, n_in, n_out, count, mem, unroll, wg))
+    finally:
+        hip.set_tuning(0, -1)
+        hip.set_unroll(-1)
+        hip.set_occupancy_lds(-1)
