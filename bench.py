@@ -186,8 +186,28 @@ def main():
         ring_bytes = 7 * 4 * ce * 2 + 7 * 2 * ce * 2
         tr = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[0], grad[:ce]], [result[:ce], send], ce, stream), 50, 5)
         tc = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[1]], [result[ce:2 * ce]], ce, stream), 50, 5)
+        # the same 14 steps as ONE persistent launch of the queue executor: independent, and with
+        # each step depending on the one before (what arrival order imposes in a real ring)
+        def ring_ops(chain):
+            o = []
+            for s in range(W - 1):
+                c = (W - 1 - s) % W
+                o.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]],
+                              outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(o) - 1] if chain and o else []))
+            for s in range(W - 1):
+                c = (W - s) % W
+                o.append(dict(dtype="bf16", compute="sum", ins=[peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce,
+                              deps=[len(o) - 1] if chain and o else []))
+            return o
+        tq = {}
+        for chain in (False, True):
+            g = hip.Graph(ring_ops(chain))
+            tq[chain] = event_times_us(torch, lambda: g.run(stream), 20, 3)
+            g.destroy()
         extras["ring_allreduce_rank_share"] = {
             "all_14_steps": dict(stats(t), GBps_median=gbps(ring_bytes, t[len(t) // 2])),
+            "all_14_steps_one_queue_launch": dict(stats(tq[False]), GBps_median=gbps(ring_bytes, tq[False][len(tq[False]) // 2])),
+            "all_14_steps_one_queue_launch_chained": dict(stats(tq[True]), GBps_median=gbps(ring_bytes, tq[True][len(tq[True]) // 2])),
             "reduce_step_2in_2out_32MiB": dict(stats(tr), GBps_median=gbps(4 * ce * 2, tr[len(tr) // 2])),
             "copy_step_1in_1out_32MiB": dict(stats(tc), GBps_median=gbps(2 * ce * 2, tc[len(tc) // 2])),
             "note": "single steps re-touch 128/64 MiB and are helped by the 256 MB Infinity Cache; "

@@ -14,7 +14,8 @@
 //     XCDs, so the ticket counter of a queue is hammered from one XCD only -- and
 //     moves on to the other queues when its own is exhausted;
 //   * a workgroup claims an entry by taking a ticket from RingBuffer::head_,
-//     reads the entry, and waits until the op's pre_dependencies_ is 0.  Every
+//     reads the entry, and waits until the op's dependencies are met (its ready word
+//     holds the number of this run; written by whoever takes pre_dependencies_ to 0).  Every
 //     dependency of a claimed entry lies earlier in the global order; each queue
 //     keeps at least one workgroup until it is exhausted; hence the unfinished
 //     claimed entry that comes first in the global order can always run, and the
@@ -53,6 +54,7 @@ namespace {
 
 constexpr int kQueues = 8;  // one per XCD of an MI355X
 constexpr long kDefaultTileBytes = 32 << 10;
+constexpr long kMaxDefaultParts = 1024;
 constexpr unsigned int kDefaultSpinLimit = 1u << 21;  // a few seconds of polling
 
 // Words that many workgroups update or poll, each alone on its 256-byte line.
@@ -77,12 +79,24 @@ struct GraphControl {
   char *slots;                            // PayloadSlot of op i at slots + i * kPayloadStride
   const int *succ;                        // all successor uid lists, back to back
   HotWord *hot;                           // kHot* words, see below
+  const int *group_base;                  // per op: first of its kPartGroups words in `groups`, or -1
+  HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
+  HotWord *ready;                         // per op: number of the run in which its dependencies were last met
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
   int queue_count[kQueues];
   unsigned int spin_limit;
   int total_tiles;
 };
+
+// An op of many parts does not count them on one word: atomics on one address are carried out
+// one after the other (about 11 ns each), and 1024 parts of a 32 MiB op finishing within a few
+// microseconds queued up behind each other (14 such ops took 690 us instead of 250).  Ops with
+// more than kGroupThreshold parts count part p on group word p % kPartGroups (each alone on its
+// line); the part that empties a group counts the group on the header's remaining_executors_,
+// which for these ops starts at kPartGroups instead of required_executors_.
+constexpr int kPartGroups = 8;
+constexpr int kGroupThreshold = 16;
 
 // indices into GraphControl::hot
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
@@ -207,18 +221,34 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // Thread 0, after a part of op `h` is complete: count it; the op's last part re-arms
 // the op's counters for the next run and releases its successors.
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const PayloadSlot *slot, int home) {
+                                            const PayloadSlot *slot, int uid, int part, int home,
+                                            unsigned int run_no) {
   const int parts = slot->parts;
+  int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
+  if (parts > kGroupThreshold) {
+    const int group = part % kPartGroups;
+    unsigned int *word = &g.groups[g.group_base[uid] + group].value;
+    if (__hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, AGENT) != 1u) return;
+    // this group is done: re-arm it (parts p < parts with p % kPartGroups == group)
+    __hip_atomic_store(word, (unsigned int)((parts - group + kPartGroups - 1) / kPartGroups), __ATOMIC_RELAXED, AGENT);
+    counted = kPartGroups;
+  }
   int old = 1;
-  if (parts > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
+  if (counted > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
   if (old != 1) return;
-  if (parts > 1) __hip_atomic_store(&h->remaining_executors_, parts, __ATOMIC_RELAXED, AGENT);
+  if (counted > 1) __hip_atomic_store(&h->remaining_executors_, counted, __ATOMIC_RELAXED, AGENT);
   const unsigned int w12 = slot->payload.initial_word12_;
   if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);
   const int n_next = (int)(w12 >> 24);
   const int *next = g.succ + slot->succ_start;
-  for (int s = 0; s < n_next; ++s)
-    __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
+  // Whoever takes a successor's count to zero announces it on the successor's own ready word:
+  // the workgroups that already hold parts of the successor poll that word, not the header,
+  // whose line the counting atomics of this and neighbouring ops need (with 1024 pollers on a
+  // header line a hand-over between two 32 MiB ops took 6 us longer).
+  for (int s = 0; s < n_next; ++s) {
+    const unsigned int before = __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
+    if ((before & 0xffu) == 1u) __hip_atomic_store(&g.ready[next[s]].value, run_no, __ATOMIC_RELAXED, AGENT);
+  }
   __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
 }
 
@@ -241,20 +271,22 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   // wavefront run ahead into the next barrier while thread 0 is parked.
   pccl_operation_layout_header *h = nullptr;
   const PayloadSlot *slot = nullptr;
+  int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   // Signal values are offset by (run number << 16).  The run number lives on the device (not
   // in the kernel arguments) so that a launch recorded into a HIP graph uses a fresh one on
   // every replay; it is read at the first signal op, always before the last workgroup out of
   // this run bumps it.
-  unsigned int signal_base = 0;
-  bool have_signal_base = false;
+  unsigned int run_no = 0;
+  if (threadIdx.x == 0) run_no = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT);
+  const unsigned int signal_base = run_no << 16;
   for (;;) {
     if (threadIdx.x == 0) {
       // The part executed in the previous iteration is complete (barrier below): every
       // wavefront waited for its write-through stores before that barrier, so the data is
       // at the point of coherence and relaxed device-scope atomics are enough to hand it
       // over; no L2 write-back / invalidate is involved.
-      if (h) finish_part(g, h, slot, home);
+      if (h) finish_part(g, h, slot, cur_uid, cur_part, home, run_no);
       int go = 0;
       unsigned long long e = 0;
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
@@ -278,21 +310,18 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         if (!go) break;
         const int uid = (int)(e & 0xffffffffu);
         pccl_operation_layout_header *hc = &g.headers[uid];
-        // wait for the op's dependencies
-        if (!bounded_wait(abort_flag, spin_limit, [&] {
-              return (__hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT) & 0xffu) == 0;
+        const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
+        // wait for the op's dependencies (none: nothing will ever write its ready word)
+        if ((sc->payload.initial_word12_ & 0xffu) != 0 &&
+            !bounded_wait(abort_flag, spin_limit, [&] {
+              return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == run_no;
             })) {
           go = 0;
           break;
         }
-        const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
         const int prim = sc->payload.primitive_;
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
-        if (!have_signal_base) {
-          signal_base = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT) << 16;
-          have_signal_base = true;
-        }
         const unsigned int want = signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
         if (prim == PCCL_NOTIFY) {
           // everything this op depends on is already at the point of coherence
@@ -303,7 +332,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           go = 0;
           break;
         }
-        finish_part(g, hc, sc, home);
+        finish_part(g, hc, sc, uid, 0, home, run_no);
       }
       s_entry = e;
       s_go = go;
@@ -312,6 +341,8 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
     const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
     const int part = __builtin_amdgcn_readfirstlane((int)(s_entry >> 32));
+    cur_uid = uid;
+    cur_part = part;
     h = &g.headers[uid];
     slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
     const pccl_op_payload *pl = &slot->payload;
@@ -404,7 +435,11 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   *graph = nullptr;
   if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_create: bad op array");
   if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
-  if (tile_bytes == 0) tile_bytes = kDefaultTileBytes;
+  // With the built-in part size an op is cut into at most kMaxDefaultParts parts: about one per
+  // workgroup of a full launch, so that one large op alone still fills the chip, while its
+  // parts grow with it instead of multiplying.
+  const bool default_tile = tile_bytes == 0;
+  if (default_tile) tile_bytes = kDefaultTileBytes;
   tile_bytes = std::max<long>(tile_bytes, 1024);
 
   // ---- validate; one (dtype, compute) pair for all REDUCE ops --------------
@@ -465,6 +500,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     n_edges += (size_t)o.n_deps;
     const long bytes = is_signal ? 0 : o.count * es;
     long p = (bytes + tile_bytes - 1) / tile_bytes;
+    if (default_tile) p = std::min<long>(p, kMaxDefaultParts);
     parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
     tiles += parts[i];
   }
@@ -531,6 +567,11 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   const size_t off_payload = off; off = align_up(off + kPayloadStride * (size_t)std::max(n_ops, 1), 256);
   const size_t off_succ = off;    off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_hot = off;     off = align_up(off + sizeof(HotWord) * kHotWords, 256);
+  int n_grouped = 0;  // ops that count their parts in groups
+  for (int i = 0; i < n_ops; ++i) n_grouped += parts[i] > kGroupThreshold;
+  const size_t off_ready = off;   off = align_up(off + sizeof(HotWord) * (size_t)std::max(n_ops, 1), 256);
+  const size_t off_gbase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
+  const size_t off_groups = off;  off = align_up(off + sizeof(HotWord) * (size_t)kPartGroups * (size_t)std::max(n_grouped, 1), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
   const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
@@ -564,6 +605,21 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   C->headers = (pccl_operation_layout_header *)(dev + off_hdr);
   C->slots = dev + off_payload;
   C->succ = (const int *)(dev + off_succ);
+  C->group_base = (const int *)(dev + off_gbase);
+  C->groups = (HotWord *)(dev + off_groups);
+  C->ready = (HotWord *)(dev + off_ready);
+  {
+    int *gbase = (int *)(img + off_gbase);
+    HotWord *groups = (HotWord *)(img + off_groups);
+    int next = 0;
+    for (int i = 0; i < n_ops; ++i) {
+      gbase[i] = -1;
+      if (parts[i] <= kGroupThreshold) continue;
+      gbase[i] = next;
+      for (int k = 0; k < kPartGroups; ++k) groups[next + k].value = (unsigned int)((parts[i] - k + kPartGroups - 1) / kPartGroups);
+      next += kPartGroups;
+    }
+  }
   C->spin_limit = kDefaultSpinLimit;
   C->total_tiles = (int)tiles;
   hot[kHotCompleted].value = 0;
@@ -609,7 +665,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     pccl_operation_layout_header *h = (pccl_operation_layout_header *)(img + off_hdr) + i;
     h->op_uid_ = i;
     h->required_executors_ = parts[i];
-    h->remaining_executors_ = parts[i];
+    h->remaining_executors_ = parts[i] > kGroupThreshold ? kPartGroups : parts[i];
     h->pre_dependencies_ = (unsigned char)n_pred[i];
     h->executor_type_ = 0;
     h->op_size_ = (unsigned char)(8 + sizeof(pccl_chunk_meta) * (size_t)(o.n_in + o.n_out));
