@@ -39,9 +39,11 @@ enum pccl_dtype {   /* element types with 16-byte packs in                      
   PCCL_BF16 = 2,    /* :71 (bf16x8)                                                */
   PCCL_F16 = 3,     /* :70 (f16x8)                                                 */
   PCCL_F8E4M3 = 4,  /* :75-77 (fp8_e4m3 packs): OCP E4M3FN, 16 per 16-byte pack     */
-  PCCL_F8E5M2 = 5   /* :78-80 (fp8_e5m2 packs): OCP E5M2                            */
+  PCCL_F8E5M2 = 5,  /* :78-80 (fp8_e5m2 packs): OCP E5M2                            */
+  PCCL_F64 = 6,     /* the f64 of multimemStore (utils/multimem.h:61-102); 2 per pack */
+  PCCL_U32 = 7      /* :66-68 (u32 packs) and multimem.h's u32 add; min / max unsigned */
 };
-#define PCCL_NUM_DTYPES 6
+#define PCCL_NUM_DTYPES 8
 
 /* Element size in bytes of a dtype code (the scalar types of vector_datatype.h:55-80),
  * 0 for an unknown code. */

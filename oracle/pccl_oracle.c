@@ -172,9 +172,20 @@ static inline uint32_t op_prod_i(uint32_t a, uint32_t b) { return a * b; }
 static inline uint32_t op_min_i(uint32_t a, uint32_t b) { return (int32_t)b < (int32_t)a ? b : a; }
 static inline uint32_t op_max_i(uint32_t a, uint32_t b) { return (int32_t)a < (int32_t)b ? b : a; }
 
+/* f64 accumulates in double; u32 differs from i32 only in the order min / max use */
+static inline double op_sum_d(double a, double b) { return a + b; }
+static inline double op_prod_d(double a, double b) { return a * b; }
+static inline double op_min_d(double a, double b) { return b < a ? b : a; }
+static inline double op_max_d(double a, double b) { return a < b ? b : a; }
+static inline uint32_t op_sum_u(uint32_t a, uint32_t b) { return a + b; }
+static inline uint32_t op_prod_u(uint32_t a, uint32_t b) { return a * b; }
+static inline uint32_t op_min_u(uint32_t a, uint32_t b) { return b < a ? b : a; }
+static inline uint32_t op_max_u(uint32_t a, uint32_t b) { return a < b ? b : a; }
+
 static size_t dtype_size(int dtype) {
   switch (dtype) {
-    case PCCL_ORACLE_F32: case PCCL_ORACLE_I32: return 4;
+    case PCCL_ORACLE_F64: return 8;
+    case PCCL_ORACLE_F32: case PCCL_ORACLE_I32: case PCCL_ORACLE_U32: return 4;
     case PCCL_ORACLE_BF16: case PCCL_ORACLE_F16: return 2;
     case PCCL_ORACLE_F8E4M3: case PCCL_ORACLE_F8E5M2: return 1;
     default: return 0;
@@ -215,6 +226,8 @@ static int reduce_range(int dtype, int op, const void *const *ins, int n_in,
   switch (dtype) {
     case PCCL_ORACLE_F32: BY_OP(float, float, IDENT, IDENT, f); break;
     case PCCL_ORACLE_I32: BY_OP(uint32_t, uint32_t, IDENT, IDENT, i); break;
+    case PCCL_ORACLE_U32: BY_OP(uint32_t, uint32_t, IDENT, IDENT, u); break;
+    case PCCL_ORACLE_F64: BY_OP(double, double, IDENT, IDENT, d); break;
     case PCCL_ORACLE_BF16:
       BY_OP(uint16_t, float, pccl_oracle_bf16_to_f32, pccl_oracle_f32_to_bf16, f);
       break;
@@ -389,8 +402,10 @@ void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64
     uint64_t b = pccl_oracle_rng_u64(seed, stream, 2 * (uint64_t)i + 1);
     double u1 = ((double)(a >> 11) + 1.0) * (1.0 / 9007199254740992.0); /* (0, 1] */
     double u2 = (double)(b >> 11) * (1.0 / 9007199254740992.0);         /* [0, 1) */
-    float z = (float)(mean + sigma * sqrt(-2.0 * log(u1)) * cos(two_pi * u2));
+    const double zd = mean + sigma * sqrt(-2.0 * log(u1)) * cos(two_pi * u2);
+    float z = (float)zd;
     switch (dtype) {
+      case PCCL_ORACLE_F64: ((double *)dst)[i] = zd; break;
       case PCCL_ORACLE_F32: ((float *)dst)[i] = z; break;
       case PCCL_ORACLE_BF16: ((uint16_t *)dst)[i] = pccl_oracle_f32_to_bf16(z); break;
       case PCCL_ORACLE_F16: ((uint16_t *)dst)[i] = pccl_oracle_f32_to_f16(z); break;

@@ -23,7 +23,8 @@
  *   out[j][i] = cvt_T( fold_op( up(in[0][i]), ..., up(in[n_in-1][i]) ) )
  *
  *   - strict left fold in input-index order, no tree, no FMA contraction;
- *   - accumulator float for f32/bf16/f16, uint32 two's-complement for i32;
+ *   - accumulator float for f32/bf16/f16/f8, double for f64, uint32 two's-complement for
+ *     i32 and u32 (u32 differs from i32 only in min / max comparing unsigned);
  *   - bf16/f16 are widened exactly, rounded to nearest-even ONCE at the end,
  *     NaN becomes a quiet NaN, overflow becomes +-inf;
  *   - min is (b < a ? b : a), max is (a < b ? b : a);
@@ -41,8 +42,9 @@
  *       saturating range (tests/test_oracle_convert.py).
  *   pccl_oracle_reduce_copy
  *       pinned against the mathematics: exact-rational brute force with one
- *       rounding per step, fold-order-sensitive known answers, int32
- *       wraparound closed form (tests/test_oracle_reduce.py).
+ *       rounding per step (binary32 and binary64), fold-order-sensitive known
+ *       answers, int32 / uint32 wraparound closed forms in Python integers
+ *       (tests/test_oracle_reduce.py).
  *       Parity against the reference's own arithmetic is UNPINNED because the
  *       reference contains none (no kernels, no tests, no golden vectors).
  *   pccl_oracle_topo_sort
@@ -60,7 +62,7 @@ extern "C" {
 
 /* dtype / compute / primitive codes: same numbering as include/pccl_hip.h. */
 enum { PCCL_ORACLE_F32 = 0, PCCL_ORACLE_I32 = 1, PCCL_ORACLE_BF16 = 2, PCCL_ORACLE_F16 = 3,
-       PCCL_ORACLE_F8E4M3 = 4, PCCL_ORACLE_F8E5M2 = 5 };
+       PCCL_ORACLE_F8E4M3 = 4, PCCL_ORACLE_F8E5M2 = 5, PCCL_ORACLE_F64 = 6, PCCL_ORACLE_U32 = 7 };
 enum { PCCL_ORACLE_SUM = 0, PCCL_ORACLE_PROD = 1, PCCL_ORACLE_MIN = 2, PCCL_ORACLE_MAX = 3 };
 
 /* ---- conversions -------------------------------------------------------- */
@@ -126,8 +128,8 @@ int pccl_oracle_topo_sort(int n_nodes, const int *edge_src, const int *edge_dst,
 uint64_t pccl_oracle_rng_u64(uint64_t seed, uint64_t stream, uint64_t index);
 void pccl_oracle_fill_uniform_f32(float *dst, long n, uint64_t seed, uint64_t stream,
                                   float lo, float hi);
-/* N(mean, sigma) by Box-Muller in double, then narrowed to dtype
- * (F32, BF16 or F16) with round-to-nearest-even. */
+/* N(mean, sigma) by Box-Muller in double, kept (F64) or narrowed to dtype
+ * (F32, BF16, F16, F8E4M3, F8E5M2) with round-to-nearest-even. */
 void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64_t stream,
                              double mean, double sigma);
 /* uniform integers in [lo, hi] */

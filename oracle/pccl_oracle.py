@@ -12,12 +12,13 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpccl_oracle.so")
 
-F32, I32, BF16, F16, F8E4M3, F8E5M2 = 0, 1, 2, 3, 4, 5
+F32, I32, BF16, F16, F8E4M3, F8E5M2, F64, U32 = 0, 1, 2, 3, 4, 5, 6, 7
 SUM, PROD, MIN, MAX = 0, 1, 2, 3
-DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16, "f8e4m3": F8E4M3, "f8e5m2": F8E5M2}
+DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16, "f8e4m3": F8E4M3, "f8e5m2": F8E5M2, "f64": F64, "u32": U32}
 COMPUTES = {"sum": SUM, "prod": PROD, "min": MIN, "max": MAX}
 # numpy storage type per dtype code (bf16/f16 travel as raw uint16 bit patterns)
-NP_STORAGE = {F32: np.float32, I32: np.int32, BF16: np.uint16, F16: np.uint16, F8E4M3: np.uint8, F8E5M2: np.uint8}
+NP_STORAGE = {F32: np.float32, I32: np.int32, BF16: np.uint16, F16: np.uint16, F8E4M3: np.uint8, F8E5M2: np.uint8,
+              F64: np.float64, U32: np.uint32}
 
 
 class OracleOp(ctypes.Structure):

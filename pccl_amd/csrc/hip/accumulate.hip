@@ -150,6 +150,8 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
     case PCCL_BF16: return launch_acc_op<PCCL_BF16>(compute, aligned, mem, grid, lds, s, p);
     case PCCL_F16: return launch_acc_op<PCCL_F16>(compute, aligned, mem, grid, lds, s, p);
     case PCCL_F8E4M3: return launch_acc_op<PCCL_F8E4M3>(compute, aligned, mem, grid, lds, s, p);
-    default: return launch_acc_op<PCCL_F8E5M2>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_F8E5M2: return launch_acc_op<PCCL_F8E5M2>(compute, aligned, mem, grid, lds, s, p);
+    case PCCL_F64: return launch_acc_op<PCCL_F64>(compute, aligned, mem, grid, lds, s, p);
+    default: return launch_acc_op<PCCL_U32>(compute, aligned, mem, grid, lds, s, p);
   }
 }

@@ -186,7 +186,8 @@ __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, lon
       // COPY moves bytes, and its element size is its own, not that of the graph's
       // REDUCE ops: run it as a copy of 1-byte units
       const int dt = pl->chunks_[0].dtype_;
-      const long units = (dt == PCCL_F32 || dt == PCCL_I32) ? 4 : (dt == PCCL_BF16 || dt == PCCL_F16) ? 2 : 1;
+      const long units = dt == PCCL_F64 ? 8 : (dt == PCCL_F32 || dt == PCCL_I32 || dt == PCCL_U32) ? 4
+                         : (dt == PCCL_BF16 || dt == PCCL_F16) ? 2 : 1;
       run_part_nin<Dtype<PCCL_F8E4M3>, OpSum, 1>(pl, lo * units, count * units);
       break;
     }
@@ -402,7 +403,9 @@ DrainKernel drain_for(int dtype, int compute) {
     case PCCL_BF16: return drain_for_compute<PCCL_BF16>(compute);
     case PCCL_F16: return drain_for_compute<PCCL_F16>(compute);
     case PCCL_F8E4M3: return drain_for_compute<PCCL_F8E4M3>(compute);
-    default: return drain_for_compute<PCCL_F8E5M2>(compute);
+    case PCCL_F8E5M2: return drain_for_compute<PCCL_F8E5M2>(compute);
+    case PCCL_F64: return drain_for_compute<PCCL_F64>(compute);
+    default: return drain_for_compute<PCCL_U32>(compute);
   }
 }
 

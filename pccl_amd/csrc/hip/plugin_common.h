@@ -17,8 +17,8 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
 inline int pccl_dtype_bytes(int dtype) {
-  return dtype == PCCL_F32 || dtype == PCCL_I32 ? 4 : dtype == PCCL_BF16 || dtype == PCCL_F16 ? 2
-         : dtype == PCCL_F8E4M3 || dtype == PCCL_F8E5M2 ? 1 : 0;
+  return dtype == PCCL_F64 ? 8 : dtype == PCCL_F32 || dtype == PCCL_I32 || dtype == PCCL_U32 ? 4
+         : dtype == PCCL_BF16 || dtype == PCCL_F16 ? 2 : dtype == PCCL_F8E4M3 || dtype == PCCL_F8E5M2 ? 1 : 0;
 }
 
 // Compute units of the current device (cached per device index).

@@ -21,6 +21,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // Same 16 bytes, but the compiler may only assume the stated alignment.  The
 // HSA ABI runs gfx9 in unaligned access mode, so these still compile to one
 // global_load_dwordx4 / global_store_dwordx4.
+typedef u32x4 u32x4_a8 __attribute__((aligned(8)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
@@ -36,25 +37,34 @@ __device__ __forceinline__ float as_f32(unsigned int u) { return __builtin_bit_c
 __device__ __forceinline__ unsigned int as_u32(float f) { return __builtin_bit_cast(unsigned int, f); }
 
 // ---- fold operators: a is the accumulator, b the next input ----------------
+// f: binary32 accumulator, d: binary64, i: int32 in two's complement, u: uint32
 struct OpSum {
   static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+  static __device__ __forceinline__ double d(double a, double b) { return a + b; }
   static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) { return a + b; }
+  static __device__ __forceinline__ unsigned int u(unsigned int a, unsigned int b) { return a + b; }
 };
 struct OpProd {
   static __device__ __forceinline__ float f(float a, float b) { return a * b; }
+  static __device__ __forceinline__ double d(double a, double b) { return a * b; }
   static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) { return a * b; }
+  static __device__ __forceinline__ unsigned int u(unsigned int a, unsigned int b) { return a * b; }
 };
 struct OpMin {
   static __device__ __forceinline__ float f(float a, float b) { return b < a ? b : a; }
+  static __device__ __forceinline__ double d(double a, double b) { return b < a ? b : a; }
   static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) {
     return (int)b < (int)a ? b : a;
   }
+  static __device__ __forceinline__ unsigned int u(unsigned int a, unsigned int b) { return b < a ? b : a; }
 };
 struct OpMax {
   static __device__ __forceinline__ float f(float a, float b) { return a < b ? b : a; }
+  static __device__ __forceinline__ double d(double a, double b) { return a < b ? b : a; }
   static __device__ __forceinline__ unsigned int i(unsigned int a, unsigned int b) {
     return (int)a < (int)b ? b : a;
   }
+  static __device__ __forceinline__ unsigned int u(unsigned int a, unsigned int b) { return a < b ? b : a; }
 };
 
 // ---- per-dtype: fold one 32-bit word of every input ------------------------
@@ -89,6 +99,36 @@ template <> struct Dtype<PCCL_I32> {
   }
   template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
     return word<Op, N>(e);
+  }
+};
+
+template <> struct Dtype<PCCL_U32> {
+  static constexpr int kElemBytes = 4;
+  typedef unsigned int elem_t;
+  typedef u32x4_a4 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
+  template <class Op, int N> static __device__ __forceinline__ unsigned int word(const unsigned int (&w)[N]) {
+    unsigned int acc = w[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::u(acc, w[k]);
+    return acc;
+  }
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    return word<Op, N>(e);
+  }
+};
+
+// binary64: an element spans two words, so the fold works on word pairs (fold_pack below)
+template <> struct Dtype<PCCL_F64> {
+  static constexpr int kElemBytes = 8;
+  typedef unsigned long long elem_t;
+  typedef u32x4_a8 pack_unaligned;
+  static __device__ __forceinline__ void wave_init() {}
+  template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
+    double acc = __builtin_bit_cast(double, e[0]);
+#pragma unroll
+    for (int k = 1; k < N; ++k) acc = Op::d(acc, __builtin_bit_cast(double, e[k]));
+    return __builtin_bit_cast(elem_t, acc);
   }
 };
 
@@ -299,12 +339,24 @@ __device__ __forceinline__ u32x4 fold_pack(const u32x4 (&v)[NIN]) {
     return v[0];  // COPY: bytes unchanged
   } else {
     u32x4 r;
+    if constexpr (D::kElemBytes == 8) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      unsigned int w[NIN];
+      for (int j = 0; j < 2; ++j) {
+        unsigned long long e[NIN];
 #pragma unroll
-      for (int k = 0; k < NIN; ++k) w[k] = v[k][j];
-      r[j] = D::template word<Op, NIN>(w);
+        for (int k = 0; k < NIN; ++k) e[k] = (unsigned long long)v[k][2 * j] | ((unsigned long long)v[k][2 * j + 1] << 32);
+        const unsigned long long x = D::template elem<Op, NIN>(e);
+        r[2 * j] = (unsigned int)x;
+        r[2 * j + 1] = (unsigned int)(x >> 32);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        unsigned int w[NIN];
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) w[k] = v[k][j];
+        r[j] = D::template word<Op, NIN>(w);
+      }
     }
     return r;
   }

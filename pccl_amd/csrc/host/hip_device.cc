@@ -41,8 +41,8 @@ struct HipPluginRegistration {
       t.primitive[TypeRegistry::registerPrimitive(prims[i])] = prim_codes[i];
       TypeRegistry::registerCompatibility("hip", prims[i]);
     }
-    const char *dtypes[] = {"f32", "i32", "bf16", "f16", "f8e4m3", "f8e5m2"};
-    const int dtype_codes[] = {PCCL_F32, PCCL_I32, PCCL_BF16, PCCL_F16, PCCL_F8E4M3, PCCL_F8E5M2};
+    const char *dtypes[] = {"f32", "i32", "bf16", "f16", "f8e4m3", "f8e5m2", "f64", "u32"};
+    const int dtype_codes[] = {PCCL_F32, PCCL_I32, PCCL_BF16, PCCL_F16, PCCL_F8E4M3, PCCL_F8E5M2, PCCL_F64, PCCL_U32};
     for (int i = 0; i < PCCL_NUM_DTYPES; ++i) {
       t.dtype[TypeRegistry::registerDataType(dtypes[i])] = dtype_codes[i];
       TypeRegistry::registerCompatibility("hip", dtypes[i]);

@@ -14,7 +14,8 @@ bool known_buffer(const std::string &b) { return b == "in" || b == "out" || b ==
 }  // namespace
 
 int Schedule::elemBytes() const {
-  if (dtype == "f32" || dtype == "i32") return 4;
+  if (dtype == "f64") return 8;
+  if (dtype == "f32" || dtype == "i32" || dtype == "u32") return 4;
   if (dtype == "bf16" || dtype == "f16") return 2;
   if (dtype == "f8e4m3" || dtype == "f8e5m2") return 1;
   bad("unknown dtype '" + dtype + "'");

@@ -11,12 +11,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpccl_hip.so")
 
 # codes of include/pccl_hip.h
-F32, I32, BF16, F16, F8E4M3, F8E5M2 = 0, 1, 2, 3, 4, 5
+F32, I32, BF16, F16, F8E4M3, F8E5M2, F64, U32 = 0, 1, 2, 3, 4, 5, 6, 7
 SUM, PROD, MIN, MAX = 0, 1, 2, 3
 COPY, REDUCE, NOTIFY, GET_NOTIFIED = 0, 1, 2, 3
-DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16, "f8e4m3": F8E4M3, "f8e5m2": F8E5M2}
+DTYPES = {"f32": F32, "i32": I32, "bf16": BF16, "f16": F16, "f8e4m3": F8E4M3, "f8e5m2": F8E5M2, "f64": F64, "u32": U32}
 COMPUTES = {"sum": SUM, "prod": PROD, "min": MIN, "max": MAX}
-ELEM_BYTES = {F32: 4, I32: 4, BF16: 2, F16: 2, F8E4M3: 1, F8E5M2: 1}
+ELEM_BYTES = {F32: 4, I32: 4, BF16: 2, F16: 2, F8E4M3: 1, F8E5M2: 1, F64: 8, U32: 4}
 
 OK = 0
 ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = -1, -2, -3, -4

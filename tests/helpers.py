@@ -4,17 +4,24 @@ import numpy as np
 
 import pccl_oracle as orc
 
-ELEM_BYTES = {"f32": 4, "i32": 4, "bf16": 2, "f16": 2, "f8e4m3": 1, "f8e5m2": 1}
+ELEM_BYTES = {"f32": 4, "i32": 4, "bf16": 2, "f16": 2, "f8e4m3": 1, "f8e5m2": 1, "f64": 8, "u32": 4}
 STORAGE = {"f32": np.float32, "i32": np.int32, "bf16": np.uint16, "f16": np.uint16,
-           "f8e4m3": np.uint8, "f8e5m2": np.uint8}
+           "f8e4m3": np.uint8, "f8e5m2": np.uint8, "f64": np.float64, "u32": np.uint32}
 
 
 def gen(dtype, count, seed, stream, kind="normal", **kw):
     """One seeded input buffer in its storage type."""
     if dtype == "i32":
         return orc.fill_int32(count, seed, stream, kw.get("lo", -(1 << 20)), kw.get("hi", 1 << 20))
+    if dtype == "u32":
+        # the whole range by default, so that values above 2^31 tell unsigned min / max from signed
+        lo, hi = kw.get("lo", 0), kw.get("hi", (1 << 32) - 1)
+        return orc.fill_int32(count, seed, stream, lo - (1 << 31), hi - (1 << 31)).view(np.uint32) ^ np.uint32(1 << 31)
     if kind == "uniform":
         a = orc.fill_uniform_f32(count, seed, stream, kw.get("lo", -1.0), kw.get("hi", 1.0))
+        if dtype == "f64":  # a second draw fills the mantissa bits a binary32 does not have
+            b = orc.fill_uniform_f32(count, seed, stream + 1000, 0.0, 1.0)
+            return a.astype(np.float64) * (1.0 + b.astype(np.float64) * 2.0 ** -24)
         return a if dtype == "f32" else orc.narrow(dtype, a)
     return orc.fill_normal(dtype, count, seed, stream, kw.get("mean", 0.0), kw.get("sigma", 1.0))
 
@@ -26,6 +33,8 @@ def bits(a):
         return a.view(np.uint32)
     if a.dtype == np.int32:
         return a.view(np.uint32)
+    if a.dtype == np.float64:
+        return a.view(np.uint64)
     return a
 
 

@@ -8,15 +8,16 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("dtype", ["f32", "i32", "bf16", "f16"])
+@pytest.mark.parametrize("dtype", ["f32", "i32", "bf16", "f16", "f64", "u32"])
 @pytest.mark.parametrize("compute", ["sum", "prod", "min", "max"])
 def test_accumulate_matches_checker(hip, oracle, dtype, compute):
     import torch
     es = H.ELEM_BYTES[dtype]
     for count, n_out, offs in ((1, 1, [0, 0]), (7, 2, [0, 0, 0]), (100003, 3, [0, 0, 0, 0]),
                                (70001, 2, [es, 3 * es, 5 * es]), (1 << 20, 8, [0] * 9), (4099, 8, [es * k for k in range(9)])):
-        kind = dict(kind="uniform", lo=0.5, hi=2.0) if compute == "prod" and dtype != "i32" else {}
+        kind = dict(kind="uniform", lo=0.5, hi=2.0) if compute == "prod" and dtype not in ("i32", "u32") else {}
         kw = dict(lo=-7, hi=7) if compute == "prod" and dtype == "i32" else kind
+        kw = dict(lo=0, hi=13) if compute == "prod" and dtype == "u32" else kw
         src = H.gen(dtype, count, 200, 0, **kw)
         dsts = [H.gen(dtype, count, 200, 1 + j, **kw) for j in range(n_out)]
         want = [oracle.reduce(dtype, compute, [d, src]) for d in dsts]
@@ -58,7 +59,7 @@ def test_accumulate_errors(hip):
         hip.accumulate("f32", "sum", t.data_ptr() + 2, [u], 8)
     assert e.value.code == hip.ERR_MISALIGNED
     with pytest.raises(hip.PcclError) as e:
-        hip.accumulate(7, "sum", t, [u], 8)
+        hip.accumulate(99, "sum", t, [u], 8)
     assert e.value.code == hip.ERR_UNSUPPORTED
     hip.accumulate("f32", "sum", t, [u], 0)
 

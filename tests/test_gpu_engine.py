@@ -163,7 +163,7 @@ def test_plugin_layer_reduce_copy(E, oracle):
     torch.cuda.synchronize()
     H.assert_bits_equal(d_out.cpu().numpy().view(np.int32), want, "plugin-layer reduce_copy")
     with pytest.raises(E.EngineError):
-        E.reduce_copy("f64", "sum", d_in, [d_out], 4)
+        E.reduce_copy("c64", "sum", d_in, [d_out], 4)
     p = E.allocate("rocm", 3 << 20)
     assert p and p % 256 == 0
     E.deallocate("rocm", p)

@@ -23,7 +23,7 @@ def _run_and_check(torch, hip, g, n_ops):
 
 def test_single_op_graph(hip, oracle):
     import torch
-    for dtype, count in (("bf16", 32768), ("f32", 70001), ("i32", 5), ("f16", 1 << 20)):
+    for dtype, count in (("bf16", 32768), ("f32", 70001), ("i32", 5), ("f16", 1 << 20), ("f64", 50001), ("u32", 7777)):
         ins = [H.gen(dtype, count, 31, k) for k in range(2)]
         want = oracle.reduce(dtype, "sum", ins)
         d_in = [H.DevBuf(torch, dtype, count, 0, src=a) for a in ins]

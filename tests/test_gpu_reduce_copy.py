@@ -13,9 +13,11 @@ COUNTS_SMALL = [1, 2, 3, 7, 8, 15, 16, 17, 63, 64, 65, 127, 255, 256, 257, 1023,
 
 def _inputs(dtype, compute, n_in, count, seed):
     if compute == "prod":
+        if dtype == "u32":
+            return [H.gen(dtype, count, seed, k, lo=0, hi=13) for k in range(n_in)]
         return [H.gen(dtype, count, seed, k, kind="uniform", lo=0.5, hi=2.0) if dtype != "i32"
                 else H.gen(dtype, count, seed, k, lo=-7, hi=7) for k in range(n_in)]
-    if dtype == "i32":
+    if dtype in ("i32", "u32"):
         return [H.gen(dtype, count, seed, k) for k in range(n_in)]
     return [H.gen(dtype, count, seed, k, kind="normal") for k in range(n_in)]
 
@@ -32,7 +34,7 @@ def test_config1_f32_sum_2in(hip, oracle):
     H.assert_bits_equal(want, ins[0] + ins[1], "oracle vs numpy")
 
 
-@pytest.mark.parametrize("dtype", ["f32", "i32", "bf16", "f16"])
+@pytest.mark.parametrize("dtype", ["f32", "i32", "bf16", "f16", "f64", "u32"])
 @pytest.mark.parametrize("compute", ["sum", "prod", "min", "max"])
 def test_all_dtype_op_nin(hip, oracle, dtype, compute):
     """Every (dtype, compute, n_in) instantiation on ragged counts, aligned buffers."""
@@ -45,7 +47,7 @@ def test_all_dtype_op_nin(hip, oracle, dtype, compute):
             H.assert_bits_equal(got, want, "%s %s n_in=%d count=%d" % (dtype, compute, n_in, count))
 
 
-@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f64"])
 def test_small_counts_every_offset(hip, oracle, dtype):
     """Counts around pack / wavefront / workgroup boundaries at every element offset of output 0."""
     import torch
@@ -140,7 +142,7 @@ def test_argument_errors(hip):
     import torch
     t = torch.zeros(1024, dtype=torch.float32, device="cuda")
     with pytest.raises(hip.PcclError) as e:
-        hip.reduce_copy(9, "sum", [t], [t], 4)
+        hip.reduce_copy(99, "sum", [t], [t], 4)
     assert e.value.code == hip.ERR_UNSUPPORTED
     with pytest.raises(hip.PcclError) as e:
         hip.reduce_copy("f32", 7, [t, t], [t], 4)

@@ -158,7 +158,7 @@ def test_direct_allreduce_schedule_shape(E, tmp_path):
 
 @pytest.mark.parametrize("text, why", [
     ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "version"),
-    ("pccl-schedule 1\nname x\ndtype f64\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "dtype"),
+    ("pccl-schedule 1\nname x\ndtype q7\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "dtype"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute xor\ndevices 1\nelems_per_device 4\nops 0\n", "compute"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
      "op 0 NOTIFY 4 deps 0 slot 256\n", "signal slot"),

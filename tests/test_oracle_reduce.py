@@ -175,7 +175,7 @@ def test_threaded_form_matches_scalar_form(oracle):
 def test_argument_checks(oracle):
     a = np.zeros(4, dtype=np.float32)
     with pytest.raises(ValueError):
-        oracle.reduce_copy(9, "sum", [a], [a])
+        oracle.reduce_copy(99, "sum", [a], [a])
     with pytest.raises(ValueError):
         oracle.reduce_copy("f32", "sum", [a] * 9, [a])
     with pytest.raises(ValueError):
@@ -258,3 +258,64 @@ def _ancestors(ops, i, memo):
             s |= _ancestors(ops, d, memo)
         memo[i] = s
     return memo[i]
+
+
+def test_u32_closed_form(oracle):
+    """u32: arithmetic mod 2^32 in Python integers; min / max compare unsigned (the same bits as
+    i32 give other answers as soon as a value exceeds 2^31)."""
+    n_in, count = 5, 4096
+    rng = np.random.default_rng(13)
+    ins = [rng.integers(0, 2 ** 32, size=count, dtype=np.uint64).astype(np.uint32) for _ in range(n_in)]
+    want_sum = np.array([sum(int(a[i]) for a in ins) % 2 ** 32 for i in range(count)], dtype=np.uint64).astype(np.uint32)
+    H.assert_bits_equal(oracle.reduce("u32", "sum", ins), want_sum, "u32 sum mod 2^32")
+    prod = [1] * count
+    for a in ins:
+        prod = [p * int(x) for p, x in zip(prod, a)]
+    H.assert_bits_equal(oracle.reduce("u32", "prod", ins), np.array([p % 2 ** 32 for p in prod], dtype=np.uint64).astype(np.uint32),
+                        "u32 prod mod 2^32")
+    H.assert_bits_equal(oracle.reduce("u32", "max", ins), np.maximum.reduce(ins), "u32 max")
+    H.assert_bits_equal(oracle.reduce("u32", "min", ins), np.minimum.reduce(ins), "u32 min")
+    as_i32 = [a.view(np.int32) for a in ins]
+    assert not np.array_equal(oracle.reduce("i32", "max", as_i32).view(np.uint32), oracle.reduce("u32", "max", ins))
+
+
+def _round_f64(q):
+    """Exact rational -> nearest binary64, ties to even: Python's Fraction -> float conversion
+    is correctly rounded (it is integer division with round-half-even)."""
+    return np.float64(float(q))
+
+
+@pytest.mark.parametrize("compute", ["sum", "prod", "min", "max"])
+def test_f64_fold_matches_exact_rational(oracle, compute):
+    count, n_in = 64, 5
+    lo, hi = (0.5, 2.0) if compute == "prod" else (-1.0, 1.0)
+    ins = [H.gen("f64", count, 910, k, kind="uniform", lo=lo, hi=hi) for k in range(n_in)]
+    if compute == "sum":
+        ins = [a * 10.0 ** (3 * (k % 4)) for k, a in enumerate(ins)]
+    want = np.empty(count, dtype=np.float64)
+    for i in range(count):
+        acc = ins[0][i]
+        for a in ins[1:]:
+            x, y = Fraction(float(acc)), Fraction(float(a[i]))
+            if compute == "sum":
+                acc = _round_f64(x + y)
+            elif compute == "prod":
+                acc = _round_f64(x * y)
+            elif compute == "min":
+                acc = a[i] if a[i] < acc else acc
+            else:
+                acc = a[i] if acc < a[i] else acc
+        want[i] = acc
+    H.assert_bits_equal(oracle.reduce("f64", compute, ins), want, "f64 %s" % compute)
+
+
+def test_f64_fold_order_and_width(oracle):
+    """Answers that need a binary64 accumulator and a left fold: 2^53 + 1 + 1 stays 2^53 from
+    the left (each +1 ties to even) and is 2^53 + 2 from the right; 1e8 + 1 - 1e8 is exactly 1
+    in binary64 where binary32 loses it."""
+    two53 = np.float64(2.0 ** 53)
+    one = np.float64(1.0)
+    for vals, want in (([two53, one, one], two53), ([one, one, two53], two53 + 2.0),
+                       ([np.float64(1e8), one, np.float64(-1e8)], one)):
+        ins = [np.full(3, v, dtype=np.float64) for v in vals]
+        H.assert_bits_equal(oracle.reduce("f64", "sum", ins), np.full(3, want, dtype=np.float64), "f64 %s" % (vals,))
