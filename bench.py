@@ -28,6 +28,10 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
+    ap.add_argument("--extras", default="all", metavar="LIST",
+                    help="comma-separated secondary workloads to run: nvls, accumulate, ring, plumbing, unaligned, "
+                         "op64k, schedule (one persistent launch), schedule_launches (the same ops as 4096 launches), "
+                         "or all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="N",
                     help="also launch N plain copies (1 input -> 1 output) of the same 256 MiB buffers: the "
@@ -147,128 +151,141 @@ def main():
     torch.cuda.synchronize()
 
     extras = {}
+    chosen = set(args.extras.split(","))
+
+    def want(name):
+        return "all" in chosen or name in chosen
+
     if not args.no_extras:
         # ---- 128 MiB variants: bf16 8->1 and fp16 8->2 ------------------------------------
-        c3 = 1 << 26
-        t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x[:c3] for x in ins], [out[:c3]], c3, stream), 30, 5)
-        extras["nvls_bf16_8in_1out_128MiB"] = dict(stats(t), GBps_median=gbps(9 * c3 * 2, t[len(t) // 2]))
-        ins16 = [randn(torch, c3, "f16") for _ in range(8)]
-        o16 = [torch.empty(c3, dtype=torch.float16, device="cuda") for _ in range(2)]
-        t = event_times_us(torch, lambda: hip.reduce_copy("f16", "sum", ins16, o16, c3, stream), 30, 5)
-        extras["nvls_f16_8in_2out_128MiB"] = dict(stats(t), GBps_median=gbps(10 * c3 * 2, t[len(t) // 2]))
-        assert torch.equal(o16[0], o16[1])
-        del ins16, o16
+        if want("nvls"):
+            c3 = 1 << 26
+            t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x[:c3] for x in ins], [out[:c3]], c3, stream), 30, 5)
+            extras["nvls_bf16_8in_1out_128MiB"] = dict(stats(t), GBps_median=gbps(9 * c3 * 2, t[len(t) // 2]))
+            ins16 = [randn(torch, c3, "f16") for _ in range(8)]
+            o16 = [torch.empty(c3, dtype=torch.float16, device="cuda") for _ in range(2)]
+            t = event_times_us(torch, lambda: hip.reduce_copy("f16", "sum", ins16, o16, c3, stream), 30, 5)
+            extras["nvls_f16_8in_2out_128MiB"] = dict(stats(t), GBps_median=gbps(10 * c3 * 2, t[len(t) // 2]))
+            assert torch.equal(o16[0], o16[1])
+            del ins16, o16
 
         # ---- fold one 128 MiB input into 7 destinations (the multimem.red role) -------------
-        src = randn(torch, c3, "bf16")
-        dsts = [randn(torch, c3, "bf16") for _ in range(7)]
-        t = event_times_us(torch, lambda: hip.accumulate("bf16", "sum", src, dsts, c3, stream), 20, 3)
-        extras["accumulate_bf16_1in_7dst_128MiB"] = dict(stats(t), GBps_median=gbps(15 * c3 * 2, t[len(t) // 2]))
-        del src, dsts
+        if want("accumulate"):
+            src = randn(torch, c3, "bf16")
+            dsts = [randn(torch, c3, "bf16") for _ in range(7)]
+            t = event_times_us(torch, lambda: hip.accumulate("bf16", "sum", src, dsts, c3, stream), 20, 3)
+            extras["accumulate_bf16_1in_7dst_128MiB"] = dict(stats(t), GBps_median=gbps(15 * c3 * 2, t[len(t) // 2]))
+            del src, dsts
 
         # ---- ring all-reduce, one rank's share at world 8: 7 reduce-copy + 7 copy steps ----
-        W, ce = 8, 1 << 24  # 32 MiB chunks of a 256 MiB gradient
-        grad = randn(torch, W * ce, "bf16", 1e-2)
-        peers = [randn(torch, ce, "bf16", 1e-2) for _ in range(W - 1)]
-        result = torch.empty(W * ce, dtype=torch.bfloat16, device="cuda")
-        send = torch.empty(ce, dtype=torch.bfloat16, device="cuda")
+        if want("ring"):
+            W, ce = 8, 1 << 24  # 32 MiB chunks of a 256 MiB gradient
+            grad = randn(torch, W * ce, "bf16", 1e-2)
+            peers = [randn(torch, ce, "bf16", 1e-2) for _ in range(W - 1)]
+            result = torch.empty(W * ce, dtype=torch.bfloat16, device="cuda")
+            send = torch.empty(ce, dtype=torch.bfloat16, device="cuda")
 
-        def ring():
-            for s in range(W - 1):  # local chunk + incoming -> output chunk + send buffer
-                c = (W - 1 - s) % W
-                hip.reduce_copy("bf16", "sum", [peers[s], grad[c * ce:(c + 1) * ce]],
-                                [result[c * ce:(c + 1) * ce], send], ce, stream)
-            for s in range(W - 1):  # incoming reduced chunk -> output chunk
-                c = (W - s) % W
-                hip.reduce_copy("bf16", "sum", [peers[s]], [result[c * ce:(c + 1) * ce]], ce, stream)
+            def ring():
+                for s in range(W - 1):  # local chunk + incoming -> output chunk + send buffer
+                    c = (W - 1 - s) % W
+                    hip.reduce_copy("bf16", "sum", [peers[s], grad[c * ce:(c + 1) * ce]],
+                                    [result[c * ce:(c + 1) * ce], send], ce, stream)
+                for s in range(W - 1):  # incoming reduced chunk -> output chunk
+                    c = (W - s) % W
+                    hip.reduce_copy("bf16", "sum", [peers[s]], [result[c * ce:(c + 1) * ce]], ce, stream)
 
-        t = event_times_us(torch, ring, 20, 3)
-        ring_bytes = 7 * 4 * ce * 2 + 7 * 2 * ce * 2
-        tr = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[0], grad[:ce]], [result[:ce], send], ce, stream), 50, 5)
-        tc = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[1]], [result[ce:2 * ce]], ce, stream), 50, 5)
-        # the same 14 steps as ONE persistent launch of the queue executor: independent, and with
-        # each step depending on the one before (what arrival order imposes in a real ring)
-        def ring_ops(chain):
-            o = []
-            for s in range(W - 1):
-                c = (W - 1 - s) % W
-                o.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]],
-                              outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(o) - 1] if chain and o else []))
-            for s in range(W - 1):
-                c = (W - s) % W
-                o.append(dict(dtype="bf16", compute="sum", ins=[peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce,
-                              deps=[len(o) - 1] if chain and o else []))
-            return o
-        tq = {}
-        for chain in (False, True):
-            g = hip.Graph(ring_ops(chain))
-            tq[chain] = event_times_us(torch, lambda: g.run(stream), 20, 3)
-            g.destroy()
-        extras["ring_allreduce_rank_share"] = {
-            "all_14_steps": dict(stats(t), GBps_median=gbps(ring_bytes, t[len(t) // 2])),
-            "all_14_steps_one_queue_launch": dict(stats(tq[False]), GBps_median=gbps(ring_bytes, tq[False][len(tq[False]) // 2])),
-            "all_14_steps_one_queue_launch_chained": dict(stats(tq[True]), GBps_median=gbps(ring_bytes, tq[True][len(tq[True]) // 2])),
-            "reduce_step_2in_2out_32MiB": dict(stats(tr), GBps_median=gbps(4 * ce * 2, tr[len(tr) // 2])),
-            "copy_step_1in_1out_32MiB": dict(stats(tc), GBps_median=gbps(2 * ce * 2, tc[len(tc) // 2])),
-            "note": "single steps re-touch 128/64 MiB and are helped by the 256 MB Infinity Cache; "
-                    "the 14-step figure walks 1.3 GiB of distinct data"}
-        del grad, peers, result, send
+            t = event_times_us(torch, ring, 20, 3)
+            ring_bytes = 7 * 4 * ce * 2 + 7 * 2 * ce * 2
+            tr = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[0], grad[:ce]], [result[:ce], send], ce, stream), 50, 5)
+            tc = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[1]], [result[ce:2 * ce]], ce, stream), 50, 5)
+            # the same 14 steps as ONE persistent launch of the queue executor: independent, and with
+            # each step depending on the one before (what arrival order imposes in a real ring)
+            def ring_ops(chain):
+                o = []
+                for s in range(W - 1):
+                    c = (W - 1 - s) % W
+                    o.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]],
+                                  outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(o) - 1] if chain and o else []))
+                for s in range(W - 1):
+                    c = (W - s) % W
+                    o.append(dict(dtype="bf16", compute="sum", ins=[peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce,
+                                  deps=[len(o) - 1] if chain and o else []))
+                return o
+            tq = {}
+            for chain in (False, True):
+                g = hip.Graph(ring_ops(chain))
+                tq[chain] = event_times_us(torch, lambda: g.run(stream), 20, 3)
+                g.destroy()
+            extras["ring_allreduce_rank_share"] = {
+                "all_14_steps": dict(stats(t), GBps_median=gbps(ring_bytes, t[len(t) // 2])),
+                "all_14_steps_one_queue_launch": dict(stats(tq[False]), GBps_median=gbps(ring_bytes, tq[False][len(tq[False]) // 2])),
+                "all_14_steps_one_queue_launch_chained": dict(stats(tq[True]), GBps_median=gbps(ring_bytes, tq[True][len(tq[True]) // 2])),
+                "reduce_step_2in_2out_32MiB": dict(stats(tr), GBps_median=gbps(4 * ce * 2, tr[len(tr) // 2])),
+                "copy_step_1in_1out_32MiB": dict(stats(tc), GBps_median=gbps(2 * ce * 2, tc[len(tc) // 2])),
+                "note": "single steps re-touch 128/64 MiB and are helped by the 256 MB Infinity Cache; "
+                        "the 14-step figure walks 1.3 GiB of distinct data"}
+            del grad, peers, result, send
 
         # ---- plumbing config: f32 2 -> 1, 4 MiB ---------------------------------------------
-        a, b = randn(torch, 1 << 20, "f32"), randn(torch, 1 << 20, "f32")
-        o = torch.empty_like(a)
-        t = event_times_us(torch, lambda: hip.reduce_copy("f32", "sum", [a, b], [o], 1 << 20, stream), 100, 10)
-        assert torch.equal(o, a + b)
-        extras["f32_2in_1out_4MiB"] = stats(t)
+        if want("plumbing"):
+            a, b = randn(torch, 1 << 20, "f32"), randn(torch, 1 << 20, "f32")
+            o = torch.empty_like(a)
+            t = event_times_us(torch, lambda: hip.reduce_copy("f32", "sum", [a, b], [o], 1 << 20, stream), 100, 10)
+            assert torch.equal(o, a + b)
+            extras["f32_2in_1out_4MiB"] = stats(t)
 
         # ---- unaligned operands: i32 4 -> 1, 2^28-57 elements, every buffer 4..60 bytes off 64 ----
-        cu = (1 << 28) - 57
-        pool = [torch.randint(-(1 << 20), 1 << 20, (cu + 64,), dtype=torch.int32, device="cuda") for _ in range(4)]
-        ou = torch.empty(cu + 64, dtype=torch.int32, device="cuda")
-        offs = [4, 12, 20, 60, 8]
-        ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
-        t = event_times_us(torch, lambda: hip.reduce_copy("i32", "sum", ptr_in, [ou.data_ptr() + offs[4]], cu, stream), 10, 2)
-        extras["unaligned_i32_4in_1out_1GiB"] = dict(stats(t), GBps_median=gbps(5 * 4 * cu, t[len(t) // 2]), byte_offsets=offs)
-        del pool, ou
+        if want("unaligned"):
+            cu = (1 << 28) - 57
+            pool = [torch.randint(-(1 << 20), 1 << 20, (cu + 64,), dtype=torch.int32, device="cuda") for _ in range(4)]
+            ou = torch.empty(cu + 64, dtype=torch.int32, device="cuda")
+            offs = [4, 12, 20, 60, 8]
+            ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
+            t = event_times_us(torch, lambda: hip.reduce_copy("i32", "sum", ptr_in, [ou.data_ptr() + offs[4]], cu, stream), 10, 2)
+            extras["unaligned_i32_4in_1out_1GiB"] = dict(stats(t), GBps_median=gbps(5 * 4 * cu, t[len(t) // 2]), byte_offsets=offs)
+            del pool, ou
 
         # ---- small ops: 64 KiB direct launch and through the queue --------------------------
-        n64 = 32768
-        x, y = randn(torch, n64, "bf16"), randn(torch, n64, "bf16")
-        z = torch.empty_like(x)
-        t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x, y], [z], n64, stream), 200, 20)
-        extras["op_64KiB_direct_launch"] = stats(t)
-        g1 = hip.Graph([dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)])
-        t = event_times_us(torch, lambda: g1.run(stream), 200, 20)
-        extras["op_64KiB_via_queue"] = stats(t)
-        g1.destroy()
+        if want("op64k"):
+            n64 = 32768
+            x, y = randn(torch, n64, "bf16"), randn(torch, n64, "bf16")
+            z = torch.empty_like(x)
+            t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x, y], [z], n64, stream), 200, 20)
+            extras["op_64KiB_direct_launch"] = stats(t)
+            g1 = hip.Graph([dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)])
+            t = event_times_us(torch, lambda: g1.run(stream), 200, 20)
+            extras["op_64KiB_via_queue"] = stats(t)
+            g1.destroy()
 
         # ---- the 4096-op small-message schedule: one persistent launch ----------------------
-        ir, per_rank = lang.small_message_allreduce()
-        low = ir.lower()
-        bufs = {"in": [randn(torch, per_rank, "bf16") for _ in range(8)],
-                "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
-        bound = lang.bind(low, lambda b, r, e: bufs[b][r].data_ptr() + 2 * e)
-        sched_bytes = sum((len(o["ins"]) + len(o["outs"])) * o["count"] * 2 for o in low)
-        g = hip.Graph(bound)
-        t = event_times_us(torch, lambda: g.run(stream), 30, 5)
-        done, total = g.status(stream)
-        assert done == total == len(low)
-        for r in range(1, 8):  # all-reduce invariant on the ring part
-            assert torch.equal(bufs["out"][r][:per_rank // 2], bufs["out"][0][:per_rank // 2])
-        ginfo = g.info()
-        med = t[len(t) // 2]
+        if want("schedule"):
+            ir, per_rank = lang.small_message_allreduce()
+            low = ir.lower()
+            bufs = {"in": [randn(torch, per_rank, "bf16") for _ in range(8)],
+                    "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
+            bound = lang.bind(low, lambda b, r, e: bufs[b][r].data_ptr() + 2 * e)
+            sched_bytes = sum((len(o["ins"]) + len(o["outs"])) * o["count"] * 2 for o in low)
+            g = hip.Graph(bound)
+            t = event_times_us(torch, lambda: g.run(stream), 30, 5)
+            done, total = g.status(stream)
+            assert done == total == len(low)
+            for r in range(1, 8):  # all-reduce invariant on the ring part
+                assert torch.equal(bufs["out"][r][:per_rank // 2], bufs["out"][0][:per_rank // 2])
+            ginfo = g.info()
+            med = t[len(t) // 2]
 
-        def individually():
-            for o in bound:
-                hip.reduce_copy("bf16", "sum", o["ins"], o["outs"], o["count"], stream)
+            def individually():
+                for o in bound:
+                    hip.reduce_copy("bf16", "sum", o["ins"], o["outs"], o["count"], stream)
 
-        t2 = event_times_us(torch, individually, 5, 1)
-        extras["schedule_4096_ops"] = {
-            "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med)),
-            "as_4096_launches": dict(stats(t2), us_per_op=round(t2[len(t2) // 2] / len(low), 4)),
-            "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
-            "algorithmic_bytes": sched_bytes}
-        g.destroy()
+            extras["schedule_4096_ops"] = {
+                "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med)),
+                "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
+                "algorithmic_bytes": sched_bytes}
+            if want("schedule_launches"):  # the same ops as one launch each ("all" includes it)
+                t2 = event_times_us(torch, individually, 5, 1)
+                extras["schedule_4096_ops"]["as_4096_launches"] = dict(stats(t2), us_per_op=round(t2[len(t2) // 2] / len(low), 4))
+            g.destroy()
 
     result = {
         "metric": "reduce_copy_hbm_bandwidth", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
