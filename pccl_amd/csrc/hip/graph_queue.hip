@@ -44,357 +44,13 @@
 #include <mutex>
 #include <vector>
 
-#include "plugin_common.h"
-#include "reduce_copy_device.h"
+#include "graph_queue_device.h"
 
 using namespace pccl_dev;
+using namespace pccl_queue;
 using pccl_host::fail;
 
 namespace {
-
-constexpr int kQueues = 8;  // one per XCD of an MI355X
-constexpr long kDefaultTileBytes = 32 << 10;
-constexpr long kMaxDefaultParts = 1024;
-constexpr unsigned int kDefaultSpinLimit = 1u << 21;  // a few seconds of polling
-
-// Words that many workgroups update or poll, each alone on its 256-byte line.
-// Device-scope atomics and sc1 loads are served at the memory side; an ordinary
-// cached load of the same line parks a copy in an XCD's L2 that every later
-// atomic must first probe out again.  Measured: with immutable fields (queue
-// length, entry pointer, part count) sharing lines with ticket counters and
-// dependency counts, a claim took 25 us and a part 13 us under 768 workgroups,
-// against 1.7 us and 1.9 us with 64.  So: lines that are written during a run
-// are touched by atomics / sc1 only, and everything a workgroup reads with
-// ordinary loads lives on lines that no one writes during a run.
-struct alignas(256) HotWord {
-  unsigned int value;
-};
-
-// Device-resident control block; read-only during a run.  The reference's
-// GraphBufferLayout is its first member, so the arena's base address is a
-// GraphBufferLayout*.
-struct GraphControl {
-  pccl_graph_buffer_layout layout;
-  pccl_operation_layout_header *headers;  // contiguous; layout.operators[i] == &headers[i]
-  char *slots;                            // PayloadSlot of op i at slots + i * kPayloadStride
-  const int *succ;                        // all successor uid lists, back to back
-  HotWord *hot;                           // kHot* words, see below
-  const int *group_base;                  // per op: first of its kPartGroups words in `groups`, or -1
-  HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
-  HotWord *ready;                         // per op: number of the run in which its dependencies were last met
-  int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
-  const unsigned long long *queue_entries[kQueues];
-  int queue_count[kQueues];
-  unsigned int spin_limit;
-  int total_tiles;
-};
-
-// An op of many parts does not count them on one word: atomics on one address are carried out
-// one after the other (about 11 ns each), and 1024 parts of a 32 MiB op finishing within a few
-// microseconds queued up behind each other (14 such ops took 690 us instead of 250).  Ops with
-// more than kGroupThreshold parts count part p on group word p % kPartGroups (each alone on its
-// line); the part that empties a group counts the group on the header's remaining_executors_,
-// which for these ops starts at kPartGroups instead of required_executors_.
-constexpr int kPartGroups = 8;
-constexpr int kGroupThreshold = 16;
-
-// indices into GraphControl::hot
-constexpr int kHotCompleted = 0;  // *layout.completed_operator
-constexpr int kHotTotal = 1;      // *layout.total_operator (never written during a run)
-constexpr int kHotAbort = 2;      // set when a bounded wait gave up
-constexpr int kHotExit = 3;       // workgroups that have left the current run
-constexpr int kHotDone = 4;       // kQueues counters of finished ops, summed at the end
-constexpr int kHotRun = kHotDone + kQueues;  // number of the current run (first run = 1), bumped by the last workgroup out
-constexpr int kHotWords = kHotRun + 1;
-
-// What a workgroup needs to run a part, on lines nothing writes during a run: the
-// op's payload plus the two header facts (part count, successor list) it would
-// otherwise have to read from the header, whose line is under atomic fire.
-constexpr size_t kPayloadStride = 256;
-struct PayloadSlot {
-  pccl_op_payload payload;  // 248 bytes; what OperationLayoutHeader::op_buffer_ points to
-  int parts;                // == required_executors_
-  int succ_start;           // successors at GraphControl::succ + succ_start
-};
-static_assert(sizeof(PayloadSlot) == kPayloadStride, "payload slot stride");
-
-__device__ __forceinline__ unsigned int *word12(pccl_operation_layout_header *h) {
-  return (unsigned int *)((char *)h + 12);
-}
-
-// elements per part: the count split evenly, rounded up to 64 elements so that
-// every part of an op keeps the alignment of the op's first element
-__host__ __device__ inline long part_elems(long count, int parts) {
-  long per = (count + parts - 1) / parts;
-  return (per + 63) / 64 * 64;
-}
-
-template <class D, class Op, int NIN, bool ALIGNED>
-__device__ __forceinline__ void run_part_body(const RcOperands &a, long head, long n_packs, long count) {
-  constexpr int kEpp = 16 / D::kElemBytes;
-  if (n_packs > 0) {
-    RcOperands body;
-    body.n_out = a.n_out;
-#pragma unroll
-    for (int k = 0; k < NIN; ++k) body.in[k] = a.in[k] + head * D::kElemBytes;
-#pragma unroll
-    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
-      if (j < a.n_out) body.out[j] = a.out[j] + head * D::kElemBytes;
-    // Every access of a part is device-coherent: its inputs may have been written
-    // by a workgroup on another XCD moments ago, and its outputs may be read by one.
-    constexpr int kUnroll = NIN >= 3 ? 1 : 2;
-    body_packs<D, Op, NIN, kUnroll, ALIGNED, kMemCoherent, kMemCoherent>(body, n_packs, 0, 1);
-  }
-  if (threadIdx.x >= kBlock - kWave)
-    edge_elems<D, Op, NIN, kMemCoherent>(a, head, head + n_packs * kEpp, count, (int)threadIdx.x - (kBlock - kWave));
-  settle_stores();
-}
-
-template <class D, class Op, int NIN>
-__device__ __forceinline__ void run_part_nin(const pccl_op_payload *pl, long lo, long count) {
-  RcOperands a;
-  a.n_out = pl->n_out_;
-  a.out[0] = (char *)pl->chunks_[NIN].addr_ + lo * D::kElemBytes;
-  // bits in which some stream's address differs from output 0's
-  unsigned long long mis = 0;
-#pragma unroll
-  for (int k = 0; k < NIN; ++k) {
-    a.in[k] = (const char *)pl->chunks_[k].addr_ + lo * D::kElemBytes;
-    mis |= (unsigned long long)a.in[k] ^ (unsigned long long)a.out[0];
-  }
-#pragma unroll
-  for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-    if (j < a.n_out) {
-      a.out[j] = (char *)pl->chunks_[NIN + j].addr_ + lo * D::kElemBytes;
-      mis |= (unsigned long long)a.out[j] ^ (unsigned long long)a.out[0];
-    }
-  // same peel as the direct launch: make output 0 start on 16 bytes; the other
-  // streams are 16-byte aligned after it exactly when they share its low bits
-  long head = (long)((16 - ((unsigned long long)a.out[0] & 15)) & 15) / D::kElemBytes;
-  if (head > count) head = count;
-  const long n_packs = (count - head) / (16 / D::kElemBytes);
-  const bool aligned = (mis & 15) == 0;
-  if (aligned) run_part_body<D, Op, NIN, true>(a, head, n_packs, count);
-  else run_part_body<D, Op, NIN, false>(a, head, n_packs, count);
-}
-
-template <int DT, class Op>
-__device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, long count) {
-  typedef Dtype<DT> D;
-  switch (pl->n_in_) {
-    case 1: {
-      // COPY moves bytes, and its element size is its own, not that of the graph's
-      // REDUCE ops: run it as a copy of 1-byte units
-      const int dt = pl->chunks_[0].dtype_;
-      const long units = dt == PCCL_F64 ? 8 : (dt == PCCL_F32 || dt == PCCL_I32 || dt == PCCL_U32) ? 4
-                         : (dt == PCCL_BF16 || dt == PCCL_F16) ? 2 : 1;
-      run_part_nin<Dtype<PCCL_F8E4M3>, OpSum, 1>(pl, lo * units, count * units);
-      break;
-    }
-    case 2: run_part_nin<D, Op, 2>(pl, lo, count); break;
-    case 3: run_part_nin<D, Op, 3>(pl, lo, count); break;
-    case 4: run_part_nin<D, Op, 4>(pl, lo, count); break;
-    case 5: run_part_nin<D, Op, 5>(pl, lo, count); break;
-    case 6: run_part_nin<D, Op, 6>(pl, lo, count); break;
-    case 7: run_part_nin<D, Op, 7>(pl, lo, count); break;
-    default: run_part_nin<D, Op, 8>(pl, lo, count); break;
-  }
-}
-
-#define AGENT __HIP_MEMORY_SCOPE_AGENT
-
-// Polls `ready` until it holds.  Gives up (and raises the abort word, so that every
-// workgroup leaves) after spin_limit polls or when another workgroup has given up.
-template <class Ready>
-__device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned int spin_limit, Ready ready) {
-  unsigned int spins = 0;
-  while (!ready()) {
-    __builtin_amdgcn_s_sleep(1);
-    if ((++spins & 63u) == 0 &&
-        (spins >= spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0)) {
-      __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
-      return false;
-    }
-  }
-  return true;
-}
-
-// Thread 0, after a part of op `h` is complete: count it; the op's last part re-arms
-// the op's counters for the next run and releases its successors.
-__device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const PayloadSlot *slot, int uid, int part, int home,
-                                            unsigned int run_no) {
-  const int parts = slot->parts;
-  int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
-  if (parts > kGroupThreshold) {
-    const int group = part % kPartGroups;
-    unsigned int *word = &g.groups[g.group_base[uid] + group].value;
-    if (__hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, AGENT) != 1u) return;
-    // this group is done: re-arm it (parts p < parts with p % kPartGroups == group)
-    __hip_atomic_store(word, (unsigned int)((parts - group + kPartGroups - 1) / kPartGroups), __ATOMIC_RELAXED, AGENT);
-    counted = kPartGroups;
-  }
-  int old = 1;
-  if (counted > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
-  if (old != 1) return;
-  if (counted > 1) __hip_atomic_store(&h->remaining_executors_, counted, __ATOMIC_RELAXED, AGENT);
-  const unsigned int w12 = slot->payload.initial_word12_;
-  if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);
-  const int n_next = (int)(w12 >> 24);
-  const int *next = g.succ + slot->succ_start;
-  // Whoever takes a successor's count to zero announces it on the successor's own ready word:
-  // the workgroups that already hold parts of the successor poll that word, not the header,
-  // whose line the counting atomics of this and neighbouring ops need (with 1024 pollers on a
-  // header line a hand-over between two 32 MiB ops took 6 us longer).
-  for (int s = 0; s < n_next; ++s) {
-    const unsigned int before = __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
-    if ((before & 0xffu) == 1u) __hip_atomic_store(&g.ready[next[s]].value, run_no, __ATOMIC_RELAXED, AGENT);
-  }
-  __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
-}
-
-template <int DT, class Op>
-__global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
-  __shared__ unsigned long long s_entry;
-  __shared__ int s_go;
-  __shared__ int s_last;
-  Dtype<DT>::wave_init();
-  HotWord *hot = g.hot;
-  unsigned int *abort_flag = &hot[kHotAbort].value;
-  const unsigned int spin_limit = g.spin_limit;
-  const int home = blockIdx.x % kQueues;
-
-  // Loop shape matters: thread 0's bookkeeping for the part just finished and its
-  // claim of the next entry sit in ONE conditional block per iteration, and the
-  // loop exit is a scalar branch (readfirstlane).  With two thread-0 blocks (one
-  // before the back edge, one after it) the compiler threads the jump between
-  // them, the back edge becomes divergent, and the other lanes of thread 0's
-  // wavefront run ahead into the next barrier while thread 0 is parked.
-  pccl_operation_layout_header *h = nullptr;
-  const PayloadSlot *slot = nullptr;
-  int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
-  unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
-  // Signal values are offset by (run number << 16).  The run number lives on the device (not
-  // in the kernel arguments) so that a launch recorded into a HIP graph uses a fresh one on
-  // every replay; it is read at the first signal op, always before the last workgroup out of
-  // this run bumps it.
-  unsigned int run_no = 0;
-  if (threadIdx.x == 0) run_no = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT);
-  const unsigned int signal_base = run_no << 16;
-  for (;;) {
-    if (threadIdx.x == 0) {
-      // The part executed in the previous iteration is complete (barrier below): every
-      // wavefront waited for its write-through stores before that barrier, so the data is
-      // at the point of coherence and relaxed device-scope atomics are enough to hand it
-      // over; no L2 write-back / invalidate is involved.
-      if (h) finish_part(g, h, slot, cur_uid, cur_part, home, run_no);
-      int go = 0;
-      unsigned long long e = 0;
-      // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
-      // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
-      for (;;) {
-        go = 0;
-        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0) break;
-        for (int i = 0; i < kQueues && !go; ++i) {
-          const int q = (home + i) % kQueues;
-          if (exhausted & (1u << q)) continue;
-          const int n = g.queue_count[q];
-          const int t = n > 0 ? __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT) : n;
-          if (t < n) {
-            e = g.queue_entries[q][t];
-            go = 1;
-            if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
-          } else {
-            exhausted |= 1u << q;
-          }
-        }
-        if (!go) break;
-        const int uid = (int)(e & 0xffffffffu);
-        pccl_operation_layout_header *hc = &g.headers[uid];
-        const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
-        // wait for the op's dependencies (none: nothing will ever write its ready word)
-        if ((sc->payload.initial_word12_ & 0xffu) != 0 &&
-            !bounded_wait(abort_flag, spin_limit, [&] {
-              return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == run_no;
-            })) {
-          go = 0;
-          break;
-        }
-        const int prim = sc->payload.primitive_;
-        if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
-        unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
-        const unsigned int want = signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
-        if (prim == PCCL_NOTIFY) {
-          // everything this op depends on is already at the point of coherence
-          __hip_atomic_store(sig, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        } else if (!bounded_wait(abort_flag, spin_limit, [&] {
-                     return (int)(__hip_atomic_load(sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
-                   })) {
-          go = 0;
-          break;
-        }
-        finish_part(g, hc, sc, uid, 0, home, run_no);
-      }
-      s_entry = e;
-      s_go = go;
-    }
-    __syncthreads();
-    if (!__builtin_amdgcn_readfirstlane(s_go)) break;
-    const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
-    const int part = __builtin_amdgcn_readfirstlane((int)(s_entry >> 32));
-    cur_uid = uid;
-    cur_part = part;
-    h = &g.headers[uid];
-    slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
-    const pccl_op_payload *pl = &slot->payload;
-    const long count = pl->chunks_[0].num_elems_;
-    const long per = part_elems(count, slot->parts);
-    const long lo = (long)part * per;
-    long n = count - lo;
-    if (n > per) n = per;
-    if (n > 0) run_part<DT, Op>(pl, lo, n);
-    // every store of this part has reached the point of coherence (run_part waits)
-    // before thread 0 hands the part over at the top of the next iteration; the
-    // barrier also keeps s_entry / s_go from being rewritten while still being read
-    __syncthreads();
-  }
-
-  // leave: the last workgroup out re-arms the graph for the next run
-  if (threadIdx.x == 0) {
-    settle_stores();  // this workgroup's counter updates land before it counts as gone
-    const unsigned int e = __hip_atomic_fetch_add(&hot[kHotExit].value, 1u, __ATOMIC_RELAXED, AGENT);
-    s_last = (e == gridDim.x - 1);
-  }
-  __syncthreads();
-  if (!__builtin_amdgcn_readfirstlane(s_last)) return;
-  if (threadIdx.x == 0) {
-    const bool aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0;
-    unsigned int done = 0;
-    for (int q = 0; q < kQueues; ++q) {
-      done += __hip_atomic_load(&hot[kHotDone + q].value, __ATOMIC_RELAXED, AGENT);
-      // after an abort the per-op state is inconsistent: leave it for the host to restore
-      if (!aborted) {
-        __hip_atomic_store(&hot[kHotDone + q].value, 0u, __ATOMIC_RELAXED, AGENT);
-        __hip_atomic_store(g.queue_head[q], 0, __ATOMIC_RELAXED, AGENT);
-      }
-    }
-    __hip_atomic_store(&hot[kHotCompleted].value, done, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&hot[kHotExit].value, 0u, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_fetch_add(&hot[kHotRun].value, 1u, __ATOMIC_RELAXED, AGENT);
-  }
-}
-
-typedef void (*DrainKernel)(const GraphControl);
-
-template <int DT>
-DrainKernel drain_for_compute(int compute) {
-  switch (compute) {
-    case PCCL_SUM: return drain_graph_kernel<DT, OpSum>;
-    case PCCL_PROD: return drain_graph_kernel<DT, OpProd>;
-    case PCCL_MIN: return drain_graph_kernel<DT, OpMin>;
-    default: return drain_graph_kernel<DT, OpMax>;
-  }
-}
 
 DrainKernel drain_for(int dtype, int compute) {
   switch (dtype) {
@@ -446,7 +102,8 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   tile_bytes = std::max<long>(tile_bytes, 1024);
 
   // ---- validate; one (dtype, compute) pair for all REDUCE ops --------------
-  int g_dtype = -1, g_compute = -1;
+  int g_dtype = -1, g_compute = -1;  // the (dtype, compute) pair of the REDUCE ops, if they share one
+  bool mixed = false;
   std::vector<int> n_succ(n_ops, 0), n_pred(n_ops, 0), parts(n_ops, 1), signal_ops;
   size_t n_edges = 0;
   long long tiles = 0;
@@ -488,8 +145,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
       }
       if (o.n_in > 1) {
         if (g_dtype < 0) { g_dtype = o.dtype; g_compute = o.compute; }
-        else if (g_dtype != o.dtype || g_compute != o.compute)
-          return fail(PCCL_ERR_UNSUPPORTED, "op %d: a graph holds REDUCE ops of one (dtype, compute) pair only", i);
+        else if (g_dtype != o.dtype || g_compute != o.compute) mixed = true;
       }
     }
     if (o.n_deps < 0 || (o.n_deps > 0 && !o.deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
@@ -584,7 +240,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   G->n_ops = n_ops;
   G->total_tiles = (int)tiles;
   G->payload_off = off_payload;
-  G->kernel = drain_for(g_dtype, g_compute);
+  G->kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute);
   if (hipGetDevice(&G->device) != hipSuccess) { delete G; return fail(PCCL_ERR_NO_DEVICE, "no current device"); }
   hipError_t e = hipMalloc((void **)&G->dev, arena_bytes);
   if (e != hipSuccess) {

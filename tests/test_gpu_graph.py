@@ -167,9 +167,6 @@ def test_graph_errors(hip):
     with pytest.raises(hip.PcclError) as e:  # self dependency
         hip.Graph([dict(op, deps=[0])])
     assert e.value.code == hip.ERR_GRAPH
-    with pytest.raises(hip.PcclError) as e:  # two (dtype, compute) pairs
-        hip.Graph([op, dict(op, compute="max")])
-    assert e.value.code == hip.ERR_UNSUPPORTED
     with pytest.raises(hip.PcclError) as e:  # unknown primitive code
         hip.Graph([dict(op, primitive=9)])
     assert e.value.code == hip.ERR_UNSUPPORTED
@@ -374,3 +371,49 @@ def test_copy_ops_keep_their_own_element_size(hip, oracle):
         H.assert_bits_equal(dbo.download(), want_b, name + ": bf16 copy")
         assert dfo.guards_intact() and dbo.guards_intact()
         g.destroy()
+
+
+def test_mixed_dtypes_and_computes_in_one_graph(hip, oracle):
+    """REDUCE ops of different (dtype, compute) pairs in one graph run the kernel instance that
+    picks the fold per part.  The f16 product overflows to infinity and the f8 sums saturate:
+    both depend on the same hardware mode bit, which that instance switches per part; small
+    parts make workgroups alternate between the two."""
+    import torch
+    n = 100_003
+    s = _stream(torch)
+    def dev(dtype, a, off=0):
+        return H.DevBuf(torch, dtype, n, off, src=a)
+    specs = [("bf16", "sum", 3, {}), ("f32", "max", 2, {}), ("f16", "prod", 4, dict(mean=0.0, sigma=40.0)),
+             ("f8e4m3", "sum", 4, dict(sigma=200.0)), ("i32", "min", 5, {}), ("f64", "sum", 2, {}),
+             ("u32", "max", 3, {}), ("f8e5m2", "prod", 3, dict(sigma=300.0)), ("f16", "sum", 8, dict(sigma=3e4))]
+    ops, checks = [], []
+    for k, (dtype, compute, n_in, kw) in enumerate(specs):
+        ins = [H.gen(dtype, n, 500 + k, j, **kw) for j in range(n_in)]
+        d_in = [dev(dtype, a, (2 * j * H.ELEM_BYTES[dtype]) % 16 if k % 2 else 0) for j, a in enumerate(ins)]
+        d_out = H.DevBuf(torch, dtype, n, 0)
+        ops.append(dict(dtype=dtype, compute=compute, ins=[b.ptr for b in d_in], outs=[d_out.ptr], count=n))
+        checks.append((dtype, compute, d_out, oracle.reduce(dtype, compute, ins), d_in))
+    # a dependent pair across dtypes' instances: copy of the f32 result, then f32 sum with itself
+    f32_out = checks[1][2]
+    cp, tw = H.DevBuf(torch, "f32", n, 4), H.DevBuf(torch, "f32", n, 0)
+    ops.append(dict(dtype="f32", compute="sum", ins=[f32_out.ptr], outs=[cp.ptr], count=n, deps=[1]))
+    ops.append(dict(dtype="f32", compute="sum", ins=[cp.ptr, f32_out.ptr], outs=[tw.ptr], count=n, deps=[len(ops) - 1]))
+    g = hip.Graph(ops, tile_bytes=8192)
+    for it in range(2):
+        for _, _, d_out, _, _ in checks:
+            d_out.view().fill_(0xFF)
+        _run_and_check(torch, hip, g, len(ops))
+        for dtype, compute, d_out, want, _ in checks:
+            got = d_out.download()
+            if dtype.startswith("f8") or dtype == "f16":
+                nan_w, nan_g = np.isnan(oracle.widen(dtype, want)), np.isnan(oracle.widen(dtype, got))
+                assert np.array_equal(nan_w, nan_g), "%s %s NaN positions" % (dtype, compute)
+                got, want = np.where(nan_w, 0, got), np.where(nan_w, 0, want)
+            H.assert_bits_equal(got, want, "run %d %s %s" % (it, dtype, compute))
+            assert d_out.guards_intact()
+        H.assert_bits_equal(cp.download(), checks[1][3], "copy")
+        H.assert_bits_equal(tw.download(), oracle.reduce("f32", "sum", [checks[1][3], checks[1][3]]), "sum after copy")
+    # the f16 cases did overflow to infinity and the f8 cases did saturate
+    assert np.isinf(oracle.widen("f16", checks[2][3])).any() and np.isinf(oracle.widen("f16", checks[8][3])).any()
+    assert (checks[3][3] & 0x7f == 0x7e).any() and (checks[7][3] & 0x7f == 0x7b).any()
+    g.destroy()
