@@ -168,3 +168,24 @@ def test_plugin_layer_reduce_copy(E, oracle):
     assert p and p % 256 == 0
     E.deallocate("rocm", p)
     assert E.allocate("rocm", 0) is None
+
+
+@pytest.mark.parametrize("dtype,compute", [("f32", "max"), ("f64", "sum"), ("u32", "min"), ("f8e4m3", "sum"), ("f16", "prod")])
+def test_ring_schedule_other_dtypes(E, eng, oracle, tmp_path, dtype, compute):
+    """The schedule file, engine and queue carry every dtype / compute name the plugin registers."""
+    import torch
+    p = str(tmp_path / "ring.sched")
+    E.write_ring_allreduce(p, dtype, compute, 4, 5001)
+    eng.regOp("ring_" + dtype, p)
+    info = eng.opInfo("ring_" + dtype)
+    assert info["elem_bytes"] == H.ELEM_BYTES[dtype]
+    n = info["devices"] * info["elems_per_device"]
+    kw = dict(kind="uniform", lo=0.7, hi=1.4) if compute == "prod" else {}
+    host_in = H.gen(dtype, n, 75, 0, **kw)
+    hdr, want = _oracle_replay(oracle, open(p).read(), host_in)
+    d_in = _to_dev(torch, host_in)
+    d_out = torch.zeros(n * H.ELEM_BYTES[dtype], dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    eng.exeOp("ring_" + dtype, d_in, d_out, stream)
+    eng.waitOp("ring_" + dtype, stream)
+    H.assert_bits_equal(d_out.cpu().numpy().view(H.STORAGE[dtype]), want, "engine ring %s %s" % (dtype, compute))
