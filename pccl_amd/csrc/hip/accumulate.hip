@@ -39,13 +39,19 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   const long pack = (long)blockIdx.x * kBlock + threadIdx.x;
   if (pack < p.n_packs) {
     const long off = p.head * D::kElemBytes + pack * 16;
-    u32x4 v[2];
-    v[1] = load_pack<D, ALIGNED, kLd>(p.in + off);
+    // All loads first, then the stores: the destinations are distinct buffers (checked by the
+    // host; partial overlap is outside the contract), so nothing written here is read here,
+    // and a lane keeps 1 + n_out loads in flight instead of two.
+    const u32x4 x = load_pack<D, ALIGNED, kLd>(p.in + off);
+    u32x4 d[PCCL_MAX_OUTPUTS];
+#pragma unroll
+    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
+      if (j < p.n_out)  // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
+        d[j] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + off) : load_pack<D, ALIGNED, kLd>(p.out[j] + off);
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.n_out) {
-        // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
-        v[0] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + off) : load_pack<D, ALIGNED, kLd>(p.out[j] + off);
+        const u32x4 v[2] = {d[j], x};
         const u32x4 r = fold_pack<D, Op, 2>(v);
         if (j == 0) store_pack<D, true, kSt>(p.out[0] + off, r);
         else store_pack<D, ALIGNED, kSt>(p.out[j] + off, r);
@@ -123,26 +129,32 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
   bool aligned = (((uintptr_t)in + (uintptr_t)p.head * es) & 15) == 0;
   for (int j = 0; j < n_out; ++j) aligned = aligned && (((uintptr_t)outs[j] + (uintptr_t)p.head * es) & 15) == 0;
   const unsigned grid = (unsigned)std::max<long>(1, (p.n_packs + kBlock - 1) / kBlock);
-  // Launch policy, measured on MI355X.  A lane handles its destinations one after the
-  // other (a store to one may alias a load of the next), so only two loads are in flight
-  // per lane and the kernel wants more resident workgroups than reduce_copy does.  One
-  // destination: the read-modify-write prefers cached accesses (7.2 vs 6.5 TB/s at
-  // 128 MiB).  Two: streaming loads with write-through stores beyond the Infinity Cache
-  // (7.1 vs 6.5 with non-temporal stores, 5.8 cached), non-temporal stores below.  Three and more: cached while input and
-  // destinations fit the 256 MB Infinity Cache together (1 -> 7 at 32 MiB: 7.05 vs 6.1),
-  // else non-temporal loads and stores (1 -> 7 at 128 MiB: 6.45 vs 6.2 write-through,
-  // 5.85 cached) under a cap of 5 workgroups per compute unit (6.4 vs 5.5 uncapped).
+  // Launch policy, measured on MI355X (128 MiB operands unless noted).  A lane has 1 + n_out
+  // loads in flight, then n_out stores.  Cache treatment: one destination, or input and
+  // destinations fitting the 256 MB Infinity Cache together, prefer cached accesses (1 -> 1:
+  // 7.3 vs 6.5 TB/s; 1 -> 7 at 32 MiB: 6.8 vs 5.7); two destinations streaming loads with
+  // write-through stores (7.1 vs 5.9 non-temporal, 5.6 cached); three and more non-temporal
+  // loads and stores (1 -> 7: 6.3 vs 6.0 cached or write-through).  Beyond the cache the
+  // occupancy cap of reduce_copy applies with 1 + 2 n_out streams per workgroup: about 20
+  // (workgroups x streams) per compute unit, at least 2 workgroups (1 -> 7: 6.3 with 2 or 3
+  // workgroups resident, 5.6-5.8 with 4 and more; 1 -> 3: 6.25 with 3, 5.9-6.0 otherwise).
   const pccl_host::Tuning t = pccl_host::tuning();
   const long total_bytes = (long)(1 + 2 * n_out) * count * es;
   const long working_set = (long)(1 + n_out) * count * es;
+  const bool beyond_cache = total_bytes > (192l << 20) && (n_out <= 2 || working_set > (256l << 20));
   int mem = kLaunchMemCached;
   if (n_out == 2 && total_bytes >= (48l << 20))
     mem = total_bytes > (192l << 20) ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
   else if (n_out >= 3 && working_set > (256l << 20)) mem = kLaunchMemStream;
   if (t.nontemporal >= 0) mem = std::min(t.nontemporal, (int)kLaunchMemStreamWriteThrough);
   unsigned lds = 0;
-  if (t.lds_bytes >= 0) lds = (unsigned)t.lds_bytes;
-  else if (n_out >= 3 && total_bytes > (192l << 20)) lds = 160 * 1024 / 5 - 256;
+  if (t.lds_bytes >= 0) {
+    lds = (unsigned)t.lds_bytes;
+  } else if (beyond_cache) {
+    const int streams = 1 + 2 * n_out;
+    const int wgs = std::max(2, std::min(8, (20 + streams / 2) / streams));
+    if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
+  }
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, mem, grid, lds, s, p);
