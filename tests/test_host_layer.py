@@ -284,3 +284,19 @@ def test_collective_ir_container():
     x = bad.create_operation(PrimitiveOpType.COPY, c, c, 0, 0)
     bad.op_dag.add_edge(x, x)
     assert not bad.validate_dag() and bad.get_operation_sequence() == []
+
+
+def test_tensor_overload_header_compiles_against_torch(tmp_path):
+    """engine_torch.h gives Engine::exeOp the reference's at::Tensor signature (include/engine.h:19);
+    it is header-only, so the check is that it compiles against this image's torch headers."""
+    import subprocess
+    from torch.utils import cpp_extension
+    src = tmp_path / "t.cc"
+    src.write_text('#include "engine_torch.h"\n'
+                   'void run(engine_c::TorchEngine &e, at::Tensor &a, at::Tensor b) { e.exeOp("op", a, b); }\n'
+                   'void run2(engine_c::Engine &e, at::Tensor &a, at::Tensor b) { engine_c::exeOp(e, "op", a, b); }\n')
+    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+           "-I", os.path.join(ROOT, "pccl_amd", "csrc", "host"), "-I", os.path.join(ROOT, "include")]
+    for inc in cpp_extension.include_paths():
+        cmd += ["-I", inc]
+    subprocess.run(cmd + [str(src)], check=True)
