@@ -1,0 +1,121 @@
+"""Seeded random sweep over everything a caller can vary at once: dtype, compute op, number of
+inputs and outputs, element count (log-uniform, so the small counts around pack and workgroup
+boundaries are as frequent as large ones), byte offsets of every buffer, an output aliasing an
+input, and the three entry points (direct launch, queue executor, accumulate).  Every case is
+compared bit for bit with the CPU checker, and the guard bands around every output are checked."""
+import numpy as np
+import pytest
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["f32", "i32", "bf16", "f16", "f8e4m3", "f8e5m2", "f64", "u32"]
+COMPUTES = ["sum", "prod", "min", "max"]
+
+
+def _gen(dtype, compute, count, seed, k):
+    if compute == "prod":
+        if dtype == "i32":
+            return H.gen(dtype, count, seed, k, lo=-7, hi=7)
+        if dtype == "u32":
+            return H.gen(dtype, count, seed, k, lo=0, hi=13)
+        return H.gen(dtype, count, seed, k, kind="uniform", lo=0.5, hi=2.0)
+    return H.gen(dtype, count, seed, k)
+
+
+def _equal(oracle, dtype, got, want, what):
+    if dtype in ("f8e4m3", "f8e5m2"):  # any NaN encoding of the format counts as NaN
+        wn, gn = np.isnan(oracle.widen(dtype, want)), np.isnan(oracle.widen(dtype, got))
+        assert np.array_equal(wn, gn), what + ": NaN positions"
+        got, want = np.where(wn, 0, got), np.where(wn, 0, want)
+    H.assert_bits_equal(got, want, what)
+
+
+def _cases(seed, n):
+    rng = np.random.default_rng(seed)
+    for i in range(n):
+        dtype = DTYPES[rng.integers(len(DTYPES))]
+        compute = COMPUTES[rng.integers(len(COMPUTES))]
+        es = H.ELEM_BYTES[dtype]
+        count = int(np.exp(rng.uniform(0, np.log(300_000))))
+        n_in, n_out = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+        aligned = rng.random() < 0.3
+        offs = lambda m: [0 if aligned else int(rng.integers(0, 64 // es)) * es for _ in range(m)]
+        yield i, dtype, compute, count, n_in, n_out, offs(n_in), offs(n_out), rng
+
+
+def test_direct_launch_random(hip, oracle):
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    for i, dtype, compute, count, n_in, n_out, in_offs, out_offs, rng in _cases(2024, 600):
+        ins = [_gen(dtype, compute, count, 700 + i, k) for k in range(n_in)]
+        want = oracle.reduce(dtype, compute, ins)
+        what = "case %d: %s %s %d->%d count=%d in_offs=%s out_offs=%s" % (i, dtype, compute, n_in, n_out, count, in_offs, out_offs)
+        d_in = [H.DevBuf(torch, dtype, count, off, src=a) for a, off in zip(ins, in_offs)]
+        d_out = [H.DevBuf(torch, dtype, count, off) for off in out_offs]
+        alias = rng.random() < 0.25      # output 0 is input k itself (in place)
+        out_ptrs = [b.ptr for b in d_out]
+        if alias:
+            k = int(rng.integers(n_in))
+            out_ptrs[0] = d_in[k].ptr
+        hip.reduce_copy(dtype, compute, [b.ptr for b in d_in], out_ptrs, count, stream)
+        torch.cuda.synchronize()
+        for j in range(n_out):
+            got = d_in[k].download() if (alias and j == 0) else d_out[j].download()
+            _equal(oracle, dtype, got, want, what + " out %d%s" % (j, " (in place)" if alias and j == 0 else ""))
+        for b in d_out + d_in:
+            assert b.guards_intact(), what + ": wrote outside a buffer"
+
+
+def test_queue_random(hip, oracle):
+    """Graphs of 1..12 independent random ops each (mixed dtypes), random part sizes."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = _cases(2025, 300)
+    g_no = 0
+    while True:
+        batch = []
+        try:
+            for _ in range(1 + g_no % 12):
+                batch.append(next(gen))
+        except StopIteration:
+            pass
+        if not batch:
+            break
+        ops, checks = [], []
+        for i, dtype, compute, count, n_in, n_out, in_offs, out_offs, rng in batch:
+            n_out = min(n_out, 10 - n_in)  # a queue op names at most 10 operands (payload of at most 255 bytes)
+            out_offs = out_offs[:n_out]
+            ins = [_gen(dtype, compute, count, 900 + i, k) for k in range(n_in)]
+            d_in = [H.DevBuf(torch, dtype, count, off, src=a) for a, off in zip(ins, in_offs)]
+            d_out = [H.DevBuf(torch, dtype, count, off) for off in out_offs]
+            ops.append(dict(dtype=dtype, compute=compute, ins=[b.ptr for b in d_in], outs=[b.ptr for b in d_out], count=count))
+            checks.append((dtype, oracle.reduce(dtype, compute, ins), d_out, d_in,
+                           "graph %d op %d: %s %s %d->%d count=%d" % (g_no, len(ops) - 1, dtype, compute, n_in, n_out, count)))
+        tile = [0, 1024, 4096, 16384][g_no % 4]
+        g = hip.Graph(ops, tile_bytes=tile)
+        g.run(stream)
+        assert g.status(stream) == (len(ops), len(ops))
+        for dtype, want, d_out, d_in, what in checks:
+            for j, b in enumerate(d_out):
+                _equal(oracle, dtype, b.download(), want, what + " out %d" % j)
+                assert b.guards_intact(), what
+        g.destroy()
+        g_no += 1
+
+
+def test_accumulate_random(hip, oracle):
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    for i, dtype, compute, count, _, n_out, in_offs, out_offs, rng in _cases(2026, 300):
+        src = _gen(dtype, compute, count, 1100 + i, 0)
+        dsts = [_gen(dtype, compute, count, 1100 + i, 1 + j) for j in range(n_out)]
+        d_src = H.DevBuf(torch, dtype, count, in_offs[0], src=src)
+        d_dst = [H.DevBuf(torch, dtype, count, off, src=a) for a, off in zip(dsts, out_offs)]
+        hip.accumulate(dtype, compute, d_src.ptr, [b.ptr for b in d_dst], count, stream)
+        torch.cuda.synchronize()
+        for j, b in enumerate(d_dst):
+            _equal(oracle, dtype, b.download(), oracle.reduce(dtype, compute, [dsts[j], src]),
+                   "case %d: %s %s 1->%d count=%d dst %d" % (i, dtype, compute, n_out, count, j))
+            assert b.guards_intact()
