@@ -195,9 +195,9 @@ __device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, long lo,
   }
   const int dt = pl->chunks_[0].dtype_;
   if (dt == PCCL_F8E4M3 || dt == PCCL_F8E5M2) {
-    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1" ::: "memory");
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1\n\ts_nop 1" ::: "memory");
   } else {
-    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 0" ::: "memory");
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 0\n\ts_nop 1" ::: "memory");
   }
   switch (dt) {
     case PCCL_F32: run_part_any_compute<PCCL_F32>(pl, lo, count); break;

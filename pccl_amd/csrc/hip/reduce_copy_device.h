@@ -191,7 +191,7 @@ template <bool E5M2> struct F8Fmt {
   static __device__ __forceinline__ void wave_init() {
     // MODE register (hwreg 1), bit 23 = FP16_OVFL; the clobber keeps loads (and so every
     // conversion of loaded data) behind the mode change
-    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1" ::: "memory");
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1\n\ts_nop 1" ::: "memory");
   }
   static __device__ __forceinline__ float up(unsigned int w, int byte) {
     if constexpr (E5M2) {
@@ -295,7 +295,13 @@ __device__ __forceinline__ u32x4 load_pack(const char *p) {
 template <class D, bool ALIGNED, int MEM>
 __device__ __forceinline__ void store_pack(char *p, u32x4 v) {
   if constexpr (MEM == kMemCoherent) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    // The s_nop is part of the store: a VMEM store of more than 64 bits of data needs two
+    // wait states before a VALU instruction may overwrite its data registers.  The compiler
+    // inserts them after the stores it generates itself, but it cannot see what this string
+    // is; without them the instruction after the LAST store of a pack (when the data is dead
+    // and its registers are reused at once, e.g. for the next address) corrupted 8 bytes of
+    // that store in a quarter of the lanes.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
   } else if constexpr (ALIGNED) {
     if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (u32x4 *)p);
     else *(u32x4 *)p = v;

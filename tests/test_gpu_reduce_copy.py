@@ -172,7 +172,7 @@ def test_every_kernel_variant_through_the_knobs(hip, oracle):
     cache treatment 0 (cacheable) / 1 (non-temporal) / 2 (non-temporal loads, write-through
     stores) x lean / 1 pack per lane / 4 packs per lane x full grid / persistent grid."""
     import torch
-    cases = [("bf16", 8, 1, 256 * 8 * 5, 0), ("bf16", 3, 2, 70001, 2), ("f32", 2, 1, 4099, 4), ("f32", 2, 3, 1 << 16, 0),
+    cases = [("bf16", 8, 1, 256 * 8 * 5, 0), ("bf16", 3, 2, 70001, 2), ("f8e4m3", 1, 8, 93744, 1), ("f32", 2, 8, 50001, 4), ("f32", 2, 1, 4099, 4), ("f32", 2, 3, 1 << 16, 0),
              ("i32", 4, 1, 131071, 12), ("f16", 1, 2, 50001, 6), ("f8e4m3", 5, 1, 30011, 3), ("bf16", 1, 1, 1 << 17, 0)]
     try:
         for dtype, n_in, n_out, count, off in cases:
