@@ -38,23 +38,25 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   constexpr int kEpp = 16 / D::kElemBytes;
   const long pack = (long)blockIdx.x * kBlock + threadIdx.x;
   if (pack < p.n_packs) {
-    const long off = p.head * D::kElemBytes + pack * 16;
+    // (wave-uniform base, lane offset) addressing: the workgroup's 4 KiB of every stream
+    const size_t wg = (size_t)p.head * D::kElemBytes + (size_t)blockIdx.x * (kBlock * 16);
+    const unsigned int off = threadIdx.x * 16u;
     // All loads first, then the stores: the destinations are distinct buffers (checked by the
     // host; partial overlap is outside the contract), so nothing written here is read here,
     // and a lane keeps 1 + n_out loads in flight instead of two.
-    const u32x4 x = load_pack<D, ALIGNED, kLd>(p.in + off);
+    const u32x4 x = load_pack<D, ALIGNED, kLd>(p.in + wg, off);
     u32x4 d[PCCL_MAX_OUTPUTS];
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.n_out)  // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
-        d[j] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + off) : load_pack<D, ALIGNED, kLd>(p.out[j] + off);
+        d[j] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + wg, off) : load_pack<D, ALIGNED, kLd>(p.out[j] + wg, off);
 #pragma unroll
     for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
       if (j < p.n_out) {
         const u32x4 v[2] = {d[j], x};
         const u32x4 r = fold_pack<D, Op, 2>(v);
-        if (j == 0) store_pack<D, true, kSt>(p.out[0] + off, r);
-        else store_pack<D, ALIGNED, kSt>(p.out[j] + off, r);
+        if (j == 0) store_pack<D, true, kSt>(p.out[0] + wg, off, r);
+        else store_pack<D, ALIGNED, kSt>(p.out[j] + wg, off, r);
       }
   }
   // head and tail elements: the last wavefront of the last workgroup

@@ -94,9 +94,8 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   *graph = nullptr;
   if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_create: bad op array");
   if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
-  // With the built-in part size an op is cut into at most kMaxDefaultParts parts: about one per
-  // workgroup of a full launch, so that one large op alone still fills the chip, while its
-  // parts grow with it instead of multiplying.
+  // With the built-in part size the parts of a large op grow with it instead of multiplying
+  // (see the part count below).
   const bool default_tile = tile_bytes == 0;
   if (default_tile) tile_bytes = kDefaultTileBytes;
   tile_bytes = std::max<long>(tile_bytes, 1024);
@@ -107,6 +106,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   std::vector<int> n_succ(n_ops, 0), n_pred(n_ops, 0), parts(n_ops, 1), signal_ops;
   size_t n_edges = 0;
   long long tiles = 0;
+  std::vector<long> op_bytes(n_ops, 0);
   for (int i = 0; i < n_ops; ++i) {
     const pccl_op_desc &o = ops[i];
     if (o.op_uid != i) return fail(PCCL_ERR_GRAPH, "op %d: op_uid %d is not its index (uids are dense from 0)", i, o.op_uid);
@@ -157,17 +157,30 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     }
     n_pred[i] = o.n_deps;
     n_edges += (size_t)o.n_deps;
-    const long bytes = is_signal ? 0 : o.count * es;
-    long p = (bytes + tile_bytes - 1) / tile_bytes;
-    if (default_tile) p = std::min<long>(p, kMaxDefaultParts);
-    parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
-    tiles += parts[i];
+    op_bytes[i] = is_signal ? 0 : o.count * es;
   }
   for (int i = 0; i < n_ops; ++i)
     if (n_succ[i] > 255) return fail(PCCL_ERR_GRAPH, "op %d: %d successors exceed num_next_ops_ (unsigned char)", i, n_succ[i]);
-  if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
   // copy-only graphs: element size of the ops decides nothing but alignment assumptions
   if (g_dtype < 0) { g_dtype = PCCL_BF16; g_compute = PCCL_SUM; }
+  // launch width: as many workgroups as the chip holds of this kernel instance
+  const DrainKernel kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute);
+  int occ = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)kernel, kBlock, 0) != hipSuccess || occ < 1) {
+    (void)hipGetLastError();
+    occ = 4;
+  }
+  occ = std::min(occ, 8);
+  const long long cap = (long long)pccl_host::compute_units() * occ;
+  // parts: with the built-in part size an op is cut into at most one part per resident
+  // workgroup, so that one large op alone fills the chip in a single round of parts
+  for (int i = 0; i < n_ops; ++i) {
+    long p = (op_bytes[i] + tile_bytes - 1) / tile_bytes;
+    if (default_tile) p = std::min<long>(p, (long)cap);
+    parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
+    tiles += parts[i];
+  }
+  if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
 
   // ---- acyclicity (Kahn) -----------------------------------------------------
   std::vector<int> succ_start(n_ops + 1, 0);
@@ -240,7 +253,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   G->n_ops = n_ops;
   G->total_tiles = (int)tiles;
   G->payload_off = off_payload;
-  G->kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute);
+  G->kernel = kernel;
   if (hipGetDevice(&G->device) != hipSuccess) { delete G; return fail(PCCL_ERR_NO_DEVICE, "no current device"); }
   hipError_t e = hipMalloc((void **)&G->dev, arena_bytes);
   if (e != hipSuccess) {
@@ -345,14 +358,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
   }
   if (n_edges) memcpy(img + off_succ, succ.data(), sizeof(int) * n_edges);
-  // launch width: enough workgroups to fill the chip, never more than entries
-  int occ = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)G->kernel, kBlock, 0) != hipSuccess || occ < 1) {
-    (void)hipGetLastError();
-    occ = 4;
-  }
-  occ = std::min(occ, 8);
-  const long long cap = (long long)pccl_host::compute_units() * occ;
+  // never more workgroups than entries
   G->n_wg = (int)std::max<long long>(1, std::min<long long>(tiles, cap));
 
   e = hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);

@@ -260,6 +260,8 @@ template <> struct Dtype<PCCL_F8E4M3> : DtypeF8<false> {};
 template <> struct Dtype<PCCL_F8E5M2> : DtypeF8<true> {};
 
 // ---- pack load / store -------------------------------------------------------
+// A pack is addressed as (base, off): `base` is the same for every lane of the wavefront
+// (it sits in scalar registers), `off` is the lane's byte offset, below 4 GiB.
 // ALIGNED: every stream is 16-byte aligned.  Otherwise only output 0 is (the
 // host peels a head so that it is) and the others are element-aligned.
 //
@@ -270,56 +272,57 @@ template <> struct Dtype<PCCL_F8E5M2> : DtypeF8<true> {};
 //                 through, this XCD's L2, which is not coherent with the L2s of the
 //                 other seven XCDs.  Used where workgroups on different XCDs hand
 //                 data to each other inside one kernel, so that no L2-wide
-//                 write-back / invalidate is needed at every hand-over.  Written
-//                 as inline assembly because the compiler offers sc1 only on
-//                 atomics of at most 8 bytes; the loads are invisible to its
-//                 wait-count tracking, so settle_loads() must precede their use.
+//                 write-back / invalidate is needed at every hand-over, and for the
+//                 stores of large reductions.  The compiler offers sc1 on global
+//                 accesses only for atomics of at most 8 bytes, so these go through
+//                 the buffer instructions, whose cache-policy operand it exposes
+//                 (buffer_load_dwordx4 / buffer_store_dwordx4 ... sc1); wait counts and
+//                 instruction hazards stay the compiler's business.
 constexpr int kMemCached = 0, kMemStream = 1, kMemCoherent = 2;
 
+// cache-policy operand of the buffer builtins on this target: 1 = sc0, 2 = nt, 16 = sc1
+constexpr int kCachePolicySc1 = 16;
+
+// Buffer resource over the whole address space above `base`: no stride, no bounds
+// clamp below 4 GiB, raw 32-bit data (word 3 as for every gfx9-family part).
+// `base` is wave-uniform by contract; reading it from the first lane tells the compiler so
+// where it cannot prove it (the descriptor must sit in scalar registers, and for a base
+// it takes to be lane-varying it would build a loop over the distinct values).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_buffer(const void *base) {
+  const unsigned long long b = (unsigned long long)base;
+  // readfirstlane returns int: go through unsigned int, or a low word with its top bit set
+  // would sign-extend into the high word
+  const unsigned int lo = (unsigned int)__builtin_amdgcn_readfirstlane((int)(unsigned int)b);
+  const unsigned int hi = (unsigned int)__builtin_amdgcn_readfirstlane((int)(unsigned int)(b >> 32));
+  const unsigned long long uniform = (unsigned long long)lo | ((unsigned long long)hi << 32);
+  return __builtin_amdgcn_make_buffer_rsrc((void *)uniform, 0, (int)0xffffffffu, 0x00020000);
+}
+
 template <class D, bool ALIGNED, int MEM>
-__device__ __forceinline__ u32x4 load_pack(const char *p) {
+__device__ __forceinline__ u32x4 load_pack(const char *base, unsigned int off) {
   if constexpr (MEM == kMemCoherent) {
-    u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-    return v;
+    return __builtin_amdgcn_raw_buffer_load_b128(whole_buffer(base), (int)off, 0, kCachePolicySc1);
   } else if constexpr (ALIGNED) {
-    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const u32x4 *)p);
-    else return *(const u32x4 *)p;
+    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const u32x4 *)(base + off));
+    else return *(const u32x4 *)(base + off);
   } else {
     typedef typename D::pack_unaligned P;
-    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const P *)p);
-    else return *(const P *)p;
+    if constexpr (MEM == kMemStream) return __builtin_nontemporal_load((const P *)(base + off));
+    else return *(const P *)(base + off);
   }
 }
 
 template <class D, bool ALIGNED, int MEM>
-__device__ __forceinline__ void store_pack(char *p, u32x4 v) {
+__device__ __forceinline__ void store_pack(char *base, unsigned int off, u32x4 v) {
   if constexpr (MEM == kMemCoherent) {
-    // The s_nop is part of the store: a VMEM store of more than 64 bits of data needs two
-    // wait states before a VALU instruction may overwrite its data registers.  The compiler
-    // inserts them after the stores it generates itself, but it cannot see what this string
-    // is; without them the instruction after the LAST store of a pack (when the data is dead
-    // and its registers are reused at once, e.g. for the next address) corrupted 8 bytes of
-    // that store in a quarter of the lanes.
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    __builtin_amdgcn_raw_buffer_store_b128(v, whole_buffer(base), (int)off, 0, kCachePolicySc1);
   } else if constexpr (ALIGNED) {
-    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (u32x4 *)p);
-    else *(u32x4 *)p = v;
+    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (u32x4 *)(base + off));
+    else *(u32x4 *)(base + off) = v;
   } else {
     typedef typename D::pack_unaligned P;
-    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (P *)p);
-    else *(P *)p = v;
-  }
-}
-
-// Makes the values of coherent loads usable: waits for all outstanding vector
-// memory operations and ties every loaded register to the wait, so that the
-// compiler cannot schedule a use above it.  Nothing to do for the other policies.
-template <int MEM, int N>
-__device__ __forceinline__ void settle_loads(u32x4 (&v)[N]) {
-  if constexpr (MEM == kMemCoherent) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[k]) : : "memory");
+    if constexpr (MEM == kMemStream) __builtin_nontemporal_store(v, (P *)(base + off));
+    else *(P *)(base + off) = v;
   }
 }
 
@@ -387,39 +390,36 @@ template <class D, class Op, int NIN, int UNROLL, bool ALIGNED, int LD, int ST>
 __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, long wg, long n_wg) {
   constexpr long kChunk = (long)kBlock * UNROLL;
   for (long base = wg * kChunk; base < n_packs; base += n_wg * kChunk) {
-    const long p0 = base + threadIdx.x;
+    const size_t chunk = (size_t)base * 16;  // byte offset of the chunk: the same for every lane
     if (base + kChunk <= n_packs) {
       u32x4 v[UNROLL][NIN];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
         for (int k = 0; k < NIN; ++k)
-          v[u][k] = load_pack<D, ALIGNED, LD>(a.in[k] + (p0 + (long)u * kBlock) * 16);
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) settle_loads<LD>(v[u]);
+          v[u][k] = load_pack<D, ALIGNED, LD>(a.in[k] + chunk, (threadIdx.x + (unsigned)u * kBlock) * 16u);
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const u32x4 r = fold_pack<D, Op, NIN>(v[u]);
-        const long off = (p0 + (long)u * kBlock) * 16;
-        store_pack<D, true, ST>(a.out[0] + off, r);
+        const unsigned int off = (threadIdx.x + (unsigned)u * kBlock) * 16u;
+        store_pack<D, true, ST>(a.out[0] + chunk, off, r);
 #pragma unroll
         for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-          if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + off, r);
+          if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + chunk, off, r);
       }
     } else {  // last, partial chunk: same shape, every pack guarded
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        const long p = p0 + (long)u * kBlock;
-        if (p < n_packs) {
+        const unsigned int off = (threadIdx.x + (unsigned)u * kBlock) * 16u;
+        if (base + threadIdx.x + (long)u * kBlock < n_packs) {
           u32x4 v[NIN];
 #pragma unroll
-          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, LD>(a.in[k] + p * 16);
-          settle_loads<LD>(v);
+          for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, ALIGNED, LD>(a.in[k] + chunk, off);
           const u32x4 r = fold_pack<D, Op, NIN>(v);
-          store_pack<D, true, ST>(a.out[0] + p * 16, r);
+          store_pack<D, true, ST>(a.out[0] + chunk, off, r);
 #pragma unroll
           for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
-            if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + p * 16, r);
+            if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + chunk, off, r);
         }
       }
     }

@@ -92,10 +92,10 @@ __global__ void __launch_bounds__(kBlock) reduce_copy_lean_kernel(const RcLean<N
   if ((long)blockIdx.x * kBlock + threadIdx.x < a.n_packs) {
     u32x4 v[NIN];
 #pragma unroll
-    for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, true, kLd>(a.in[k] + wg_off + lane_off);
+    for (int k = 0; k < NIN; ++k) v[k] = load_pack<D, true, kLd>(a.in[k] + wg_off, lane_off);
     const u32x4 r = fold_pack<D, Op, NIN>(v);
 #pragma unroll
-    for (int j = 0; j < NOUT; ++j) store_pack<D, true, kSt>(a.out[j] + wg_off + lane_off, r);
+    for (int j = 0; j < NOUT; ++j) store_pack<D, true, kSt>(a.out[j] + wg_off, lane_off, r);
   }
 }
 
