@@ -177,8 +177,10 @@ __device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, lon
 // instance sets the bit for exactly the parts that need it.
 constexpr int kAnyDtype = -1;
 
+// Not inlined: one function per dtype keeps the any-dtype kernel a small caller of eight
+// mid-sized functions (as one flat function its compilation took minutes).
 template <int DT>
-__device__ __forceinline__ void run_part_any_compute(const pccl_op_payload *pl, long lo, long count) {
+__device__ __attribute__((noinline)) void run_part_any_compute(const pccl_op_payload *pl, long lo, long count) {
   switch (pl->compute_) {
     case PCCL_SUM: run_reduce_part<DT, OpSum, true>(pl, lo, count); break;
     case PCCL_PROD: run_reduce_part<DT, OpProd, true>(pl, lo, count); break;
