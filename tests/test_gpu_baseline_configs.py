@@ -163,3 +163,43 @@ def test_config5_small_message_schedule_full_size(hip, oracle):
         for t in d_out:
             t.zero_()
     g.destroy()
+
+
+def test_buffers_beyond_4_gib(hip):
+    """Single operands larger than 4 GiB: every byte offset inside the kernels must be 64-bit.
+    Checked on the device against torch (i32 sums wrap the same way; a copy is byte equality),
+    at both ends and around the 4 GiB mark, for the direct launch and the queue executor."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    n = (1 << 30) + 4099                      # int32 elements: 4 GiB + 16 KiB + 12 B
+    a = torch.randint(-(1 << 31), (1 << 31) - 1, (n + 1,), dtype=torch.int32, device="cuda")
+    b = torch.randint(-(1 << 31), (1 << 31) - 1, (n + 1,), dtype=torch.int32, device="cuda")
+    out = torch.zeros(n + 2, dtype=torch.int32, device="cuda")
+    windows = [slice(0, 1 << 20), slice((1 << 30) - (1 << 19), (1 << 30) + 4099)]
+
+    def check(got, want, what):
+        for w in windows:
+            assert torch.equal(got[w], want[w]), what
+        # and a strided sample across the whole range
+        assert torch.equal(got[::4099], want[::4099]), what
+
+    # aligned operands
+    hip.reduce_copy("i32", "sum", [a[:n], b[:n]], [out[:n]], n, stream)
+    torch.cuda.synchronize()
+    check(out[:n], a[:n] + b[:n], "aligned 2 -> 1 beyond 4 GiB")
+    # unaligned operands (4 bytes off) and a copy
+    out.zero_()
+    hip.reduce_copy("i32", "sum", [a[1:]], [out[2:]], n, stream)
+    torch.cuda.synchronize()
+    check(out[2:], a[1:], "unaligned copy beyond 4 GiB")
+    assert int(out[0]) == 0 and int(out[1]) == 0
+    # the queue executor on the same operands
+    out.zero_()
+    g = hip.Graph([dict(dtype="i32", compute="sum", ins=[a[1:], b[:n]], outs=[out[:n]], count=n)])
+    g.run(stream)
+    assert g.status(stream) == (1, 1)
+    check(out[:n], a[1:] + b[:n], "queue 2 -> 1 beyond 4 GiB")
+    assert int(out[n]) == 0
+    g.destroy()
+    del a, b, out
+    torch.cuda.empty_cache()
