@@ -107,7 +107,7 @@ int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *out
 /* Launch-shape overrides for tuning runs: workgroups per compute unit
  * (0 = built-in choice) and cache treatment (-1 = built-in choice, 0 = cacheable,
  * 1 = non-temporal loads and stores, 2 = non-temporal loads and write-through stores). */
-int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal);
+int pccl_hip_set_tuning(int workgroups_per_cu, int cache_treatment);
 
 /* Occupancy override for tuning runs: bytes of (unused) dynamic LDS requested per
  * workgroup, which caps the workgroups resident on a compute unit at

@@ -148,7 +148,7 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
   if (n_out == 2 && total_bytes >= (48l << 20))
     mem = total_bytes > (192l << 20) ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
   else if (n_out >= 3 && working_set > (256l << 20)) mem = kLaunchMemStream;
-  if (t.nontemporal >= 0) mem = std::min(t.nontemporal, (int)kLaunchMemStreamWriteThrough);
+  if (t.cache_treatment >= 0) mem = std::min(t.cache_treatment, (int)kLaunchMemStreamWriteThrough);
   unsigned lds = 0;
   if (t.lds_bytes >= 0) {
     lds = (unsigned)t.lds_bytes;

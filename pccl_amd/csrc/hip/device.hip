@@ -49,7 +49,7 @@ Tuning tuning() {
   if (!g_tuning_env_read) {  // same knobs the host plugin lists as launch options
     g_tuning_env_read = true;
     if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tuning.workgroups_per_cu = atoi(s);
-    if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.nontemporal = std::max(0, std::min(2, atoi(s)));
+    if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.cache_treatment = std::max(0, std::min(2, atoi(s)));
     if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tuning.lds_bytes = atoi(s);
     if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tuning.unroll = atoi(s);
   }
@@ -129,14 +129,14 @@ int pccl_hip_free(void *p) {
   return PCCL_OK;
 }
 
-int pccl_hip_set_tuning(int workgroups_per_cu, int nontemporal) {
+int pccl_hip_set_tuning(int workgroups_per_cu, int cache_treatment) {
   clear_error();
   if (workgroups_per_cu < 0 || workgroups_per_cu > 64)
     return fail(PCCL_ERR_INVALID_ARG, "workgroups_per_cu %d outside [0, 64]", workgroups_per_cu);
   (void)tuning();  // make sure the environment was read before overriding it
   std::lock_guard<std::mutex> lock(g_tuning_mutex);
   g_tuning.workgroups_per_cu = workgroups_per_cu;
-  g_tuning.nontemporal = nontemporal < 0 ? -1 : std::min(nontemporal, 2);
+  g_tuning.cache_treatment = cache_treatment < 0 ? -1 : std::min(cache_treatment, 2);
   return PCCL_OK;
 }
 

@@ -26,7 +26,7 @@ int compute_units();
 
 struct Tuning {
   int workgroups_per_cu;  // 0 = built-in choice
-  int nontemporal;        // -1 = built-in choice, else 0 cacheable / 1 streaming / 2 streaming loads + write-through stores
+  int cache_treatment;        // -1 = built-in choice, else 0 cacheable / 1 streaming / 2 streaming loads + write-through stores
   int lds_bytes;          // -1 = built-in choice, else dynamic LDS requested per workgroup
   int unroll;             // -1 = built-in choice, 0 = lean kernel where it applies, else packs per lane (1 or 4)
 };

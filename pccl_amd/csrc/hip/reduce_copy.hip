@@ -94,7 +94,7 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
     const bool write_through = n_in > 1 && big && total_bytes <= (4l << 30);
     mem = write_through ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
   }
-  if (t.nontemporal >= 0) mem = std::min(t.nontemporal, (int)kLaunchMemStreamWriteThrough);
+  if (t.cache_treatment >= 0) mem = std::min(t.cache_treatment, (int)kLaunchMemStreamWriteThrough);
   // one pack per lane beyond the Infinity Cache; a copy already from 32 MiB in all (cold walk
   // over 16 MiB copies: 4.55 vs 4.29 TB/s, 64 MiB: 5.8 vs 5.7)
   int unroll = (big || (n_in == 1 && total_bytes >= (32l << 20))) ? 1 : small_unroll_for(n_in);

@@ -129,8 +129,8 @@ def free(ptr):
     _check(lib().pccl_hip_free(ctypes.c_void_p(ptr)))
 
 
-def set_tuning(workgroups_per_cu=0, nontemporal=-1):
-    _check(lib().pccl_hip_set_tuning(workgroups_per_cu, nontemporal))
+def set_tuning(workgroups_per_cu=0, cache_treatment=-1):
+    _check(lib().pccl_hip_set_tuning(workgroups_per_cu, cache_treatment))
 
 
 def set_occupancy_lds(lds_bytes=-1):
