@@ -3,12 +3,18 @@ inputs and outputs, element count (log-uniform, so the small counts around pack 
 boundaries are as frequent as large ones), byte offsets of every buffer, an output aliasing an
 input, and the three entry points (direct launch, queue executor, accumulate).  Every case is
 compared bit for bit with the CPU checker, and the guard bands around every output are checked."""
+import os
+
 import numpy as np
 import pytest
 
 import helpers as H
 
 pytestmark = pytest.mark.gpu
+
+# PCCL_TEST_SWEEP_SCALE=10 runs ten times as many cases from other seeds (a soak, not the default)
+SCALE = max(1, int(os.environ.get("PCCL_TEST_SWEEP_SCALE", "1")))
+SEED_SHIFT = 0 if SCALE == 1 else 7919
 
 DTYPES = ["f32", "i32", "bf16", "f16", "f8e4m3", "f8e5m2", "f64", "u32"]
 COMPUTES = ["sum", "prod", "min", "max"]
@@ -45,13 +51,38 @@ def _cases(seed, n):
         yield i, dtype, compute, count, n_in, n_out, offs(n_in), offs(n_out), rng
 
 
-def test_direct_launch_random(hip, oracle):
+@pytest.fixture
+def restore_knobs(hip):
+    yield
+    hip.set_tuning(0, -1)
+    hip.set_unroll(-1)
+    hip.set_occupancy_lds(-1)
+
+
+def _random_knobs(hip, rng):
+    """Every second case forces a kernel variant that the built-in policy would only pick for
+    much larger operands: cache treatment, packs per lane / lean kernel, persistent grid, LDS cap."""
+    if rng.random() < 0.5:
+        hip.set_tuning(0, -1)
+        hip.set_unroll(-1)
+        hip.set_occupancy_lds(-1)
+        return "policy"
+    mem, unroll = int(rng.integers(0, 3)), [-1, 0, 1, 4][rng.integers(4)]
+    wg, lds = [0, 0, 1, 3][rng.integers(4)], [-1, 0, 32512, 65536][rng.integers(4)]
+    hip.set_tuning(wg, mem)
+    hip.set_unroll(unroll)
+    hip.set_occupancy_lds(lds)
+    return "mem=%d unroll=%d wg=%d lds=%d" % (mem, unroll, wg, lds)
+
+
+def test_direct_launch_random(hip, oracle, restore_knobs):
     import torch
     stream = torch.cuda.current_stream().cuda_stream
-    for i, dtype, compute, count, n_in, n_out, in_offs, out_offs, rng in _cases(2024, 600):
+    for i, dtype, compute, count, n_in, n_out, in_offs, out_offs, rng in _cases(2024 + SEED_SHIFT, 600 * SCALE):
+        knobs = _random_knobs(hip, rng)
         ins = [_gen(dtype, compute, count, 700 + i, k) for k in range(n_in)]
         want = oracle.reduce(dtype, compute, ins)
-        what = "case %d: %s %s %d->%d count=%d in_offs=%s out_offs=%s" % (i, dtype, compute, n_in, n_out, count, in_offs, out_offs)
+        what = "case %d: %s %s %d->%d count=%d in_offs=%s out_offs=%s [%s]" % (i, dtype, compute, n_in, n_out, count, in_offs, out_offs, knobs)
         d_in = [H.DevBuf(torch, dtype, count, off, src=a) for a, off in zip(ins, in_offs)]
         d_out = [H.DevBuf(torch, dtype, count, off) for off in out_offs]
         alias = rng.random() < 0.25      # output 0 is input k itself (in place)
@@ -72,7 +103,7 @@ def test_queue_random(hip, oracle):
     """Graphs of 1..12 independent random ops each (mixed dtypes), random part sizes."""
     import torch
     stream = torch.cuda.current_stream().cuda_stream
-    gen = _cases(2025, 300)
+    gen = _cases(2025 + SEED_SHIFT, 300 * SCALE)
     g_no = 0
     while True:
         batch = []
@@ -105,10 +136,11 @@ def test_queue_random(hip, oracle):
         g_no += 1
 
 
-def test_accumulate_random(hip, oracle):
+def test_accumulate_random(hip, oracle, restore_knobs):
     import torch
     stream = torch.cuda.current_stream().cuda_stream
-    for i, dtype, compute, count, _, n_out, in_offs, out_offs, rng in _cases(2026, 300):
+    for i, dtype, compute, count, _, n_out, in_offs, out_offs, rng in _cases(2026 + SEED_SHIFT, 300 * SCALE):
+        knobs = _random_knobs(hip, rng)
         src = _gen(dtype, compute, count, 1100 + i, 0)
         dsts = [_gen(dtype, compute, count, 1100 + i, 1 + j) for j in range(n_out)]
         d_src = H.DevBuf(torch, dtype, count, in_offs[0], src=src)
@@ -117,5 +149,5 @@ def test_accumulate_random(hip, oracle):
         torch.cuda.synchronize()
         for j, b in enumerate(d_dst):
             _equal(oracle, dtype, b.download(), oracle.reduce(dtype, compute, [dsts[j], src]),
-                   "case %d: %s %s 1->%d count=%d dst %d" % (i, dtype, compute, n_out, count, j))
+                   "case %d: %s %s 1->%d count=%d dst %d [%s]" % (i, dtype, compute, n_out, count, j, knobs))
             assert b.guards_intact()
