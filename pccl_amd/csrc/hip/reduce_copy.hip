@@ -78,21 +78,23 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   // pack per lane under an occupancy cap (below).  Streaming treatment starts earlier,
   // at 48 MiB: a collective step works on data that just arrived and will not be
   // touched again soon; smaller operands stay cacheable.  Which streaming treatment
-  // (measured on MI355X in steady state, TB/s with non-temporal vs write-through
-  // stores): reductions beyond the Infinity Cache prefer write-through stores (8 -> 1 at
-  // 256 MiB 6.5 vs 6.6, 8 -> 2 at 128 MiB 6.5 vs 6.8, 4 -> 1 6.3 vs 6.7, 2 -> 1 6.6 vs
-  // 7.2); copies prefer non-temporal stores (1 -> 1 at 256 MiB 7.3 vs 6.1), and so do
-  // reductions over several GiB (i32 4 -> 1 at 1 GiB per operand 6.1 vs 6.0, unaligned
-  // 5.9 vs 5.4).  Between 48 and 192 MiB write-through stores look better on a step
-  // that is repeated in place (2 -> 2 at 32 MiB 6.0 vs 6.9) but leave the caches in a
-  // state the NEXT kernel pays for: a walk over 14 ring steps of 32 MiB takes 239 us
-  // with non-temporal stores throughout and 256 us with write-through reductions.
+  // (measured on MI355X, TB/s with non-temporal stores vs write-through stores):
+  //  - same buffers every launch: 8 -> 1 at 256 MiB 6.5 vs 6.6, 8 -> 2 at 128 MiB 6.5 vs
+  //    6.9, 4 -> 1 6.3 vs 6.7, 2 -> 1 6.6 vs 7.2;
+  //  - walks over distinct buffers (nothing in any cache): copy 1 -> 1 at 96 MiB .. 1 GiB
+  //    6.0-6.4 vs 6.3-6.7, 1 -> 2 6.1 vs 6.3, but 1 -> 4 and 1 -> 8 6.6 vs 6.0-6.3;
+  //  - a walk over 14 ring steps (7 reductions 2 -> 2, 7 copies): 243 vs 229 us at 32 MiB
+  //    chunks, 452 vs 433 us at 64 MiB, when every step uses the same treatment; MIXING
+  //    them is worse than either (write-through reductions followed by non-temporal
+  //    copies: 249 and 467 us), which is why one rule covers reductions and copies;
+  //  - reductions over several GiB: i32 4 -> 1 at 1 GiB per operand 6.1 vs 6.0, unaligned
+  //    5.9 vs 5.4.
   const long total_bytes = (long)(n_in + n_out) * count * es;
   const bool big = total_bytes > (192l << 20);
   int mem = kLaunchMemCached;
   if (total_bytes >= (48l << 20)) {
-    const bool write_through = n_in > 1 && big && total_bytes <= (4l << 30);
-    mem = write_through ? kLaunchMemStreamWriteThrough : kLaunchMemStream;
+    const bool non_temporal_stores = (n_in == 1 && n_out >= 3) || total_bytes > (4l << 30);
+    mem = non_temporal_stores ? kLaunchMemStream : kLaunchMemStreamWriteThrough;
   }
   if (t.cache_treatment >= 0) mem = std::min(t.cache_treatment, (int)kLaunchMemStreamWriteThrough);
   // one pack per lane beyond the Infinity Cache; a copy already from 32 MiB in all (cold walk

@@ -27,12 +27,13 @@ __host__ __device__ constexpr int small_unroll_for(int n_in) { return n_in <= 2 
 // MEM: how the launch treats the caches (host-side choice by operand size and shape).
 //   0  everything cacheable;
 //   1  streaming: non-temporal loads and stores (a copy: stores only);
-//   2  streaming loads (a copy: cacheable loads), write-through (sc1) stores.  Measured on
-//      MI355X this beats 1 wherever the stores compete with many load streams for the
-//      L2: bf16 8 -> 1 at 256 MiB 6.62 -> 6.86 TB/s, 2 -> 2 at 32 MiB 5.5 -> 6.4 TB/s.
+//   2  non-temporal loads (a copy too), write-through (sc1) stores.  Measured on MI355X this
+//      beats 1 for reductions beyond the caches (bf16 8 -> 2 at 128 MiB 6.5 -> 6.9 TB/s,
+//      2 -> 1 at 256 MiB 6.6 -> 7.2) and for the steps of a ring walk, copies included.
 constexpr int kLaunchMemCached = 0, kLaunchMemStream = 1, kLaunchMemStreamWriteThrough = 2;
 template <int MEM, int NIN> struct LaunchMem {
-  static constexpr int kLd = (MEM != kLaunchMemCached && NIN > 1) ? kMemStream : kMemCached;
+  static constexpr int kLd =
+      (MEM == kLaunchMemStreamWriteThrough || (MEM == kLaunchMemStream && NIN > 1)) ? kMemStream : kMemCached;
   static constexpr int kSt = MEM == kLaunchMemCached ? kMemCached : MEM == kLaunchMemStream ? kMemStream : kMemCoherent;
 };
 
