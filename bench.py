@@ -19,7 +19,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size (figures and commands in
 # profiles/reduce_copy_bf16_8in_256MiB.md).
-MEASURED_TRAFFIC_BYTES = 2415507280
+MEASURED_TRAFFIC_BYTES = 2415785223
 
 
 def parse():
