@@ -8,6 +8,10 @@ import math
 from .ir import Chunk, CollectiveIR, Device, DeviceType, Link, PrimitiveOpType
 
 
+# element sizes of the dtype names the device plugin registers
+ELEM_BYTES = {"f64": 8, "f32": 4, "i32": 4, "u32": 4, "bf16": 2, "f16": 2, "f8e4m3": 1, "f8e5m2": 1}
+
+
 def _ring_ir(name, world, dtype, compute):
     ir = CollectiveIR(name, dtype=dtype, compute=compute)
     for r in range(world):
@@ -57,6 +61,95 @@ def ring_allreduce(world, chunk_elems, dtype="bf16", compute="sum", name="ring_a
                 metadata={"src_buffer": "out", "tgt_buffer": "out", "level": W - 1 + step})
         prev = cur
     return ir, base + W * chunk_elems
+
+
+def ring_reduce_scatter(world, chunk_elems, dtype="bf16", compute="sum", name="ring_reduce_scatter"):
+    """The reduce-scatter half of the ring: after W-1 steps rank r holds, in "out" at chunk
+    (r+1) mod W, the fold of that chunk over all ranks (in ring order starting at the chunk's
+    own rank).  Other chunks of "out" are partial sums or untouched.  Returns (ir, elems)."""
+    W = world
+    ir = _ring_ir(name, W, dtype, compute)
+    prev = {}
+    for step in range(1, W):
+        cur = {}
+        for r in range(W):
+            c, p = (r - step) % W, (r - 1) % W
+            off = c * chunk_elems
+            incoming = ("in" if step == 1 else "out", p, off)
+            ranks = {(c + i) % W for i in range(step + 1)}
+            cur[r] = ir.create_operation(
+                PrimitiveOpType.REDUCE,
+                src_chunk=Chunk(ranks - {r}, p, chunk_elems, off), tgt_chunk=Chunk(ranks, r, chunk_elems, off),
+                src_device=p, tgt_device=r, dependencies=[prev[p]] if step > 1 else [],
+                metadata={"srcs": [incoming, ("in", r, off)], "tgt_buffer": "out", "level": step})
+        prev = cur
+    return ir, W * chunk_elems
+
+
+def ring_all_gather(world, chunk_elems, dtype="bf16", name="ring_all_gather"):
+    """Rank r contributes chunk r of its "in"; afterwards every rank's "out" holds all W chunks.
+    Level 1: every rank copies its own chunk in -> out; levels 2..W: rank r copies chunk
+    (r-s+1) mod W from rank r-1's "out".  Returns (ir, elems)."""
+    W = world
+    ir = _ring_ir(name, W, dtype, "sum")
+    prev = {}
+    for r in range(W):
+        off = r * chunk_elems
+        prev[r] = ir.create_operation(
+            PrimitiveOpType.COPY, src_chunk=Chunk({r}, r, chunk_elems, off), tgt_chunk=Chunk({r}, r, chunk_elems, off),
+            src_device=r, tgt_device=r, dependencies=[], metadata={"src_buffer": "in", "tgt_buffer": "out", "level": 1})
+    for step in range(1, W):
+        cur = {}
+        for r in range(W):
+            c, p = (r - step) % W, (r - 1) % W
+            off = c * chunk_elems
+            cur[r] = ir.create_operation(
+                PrimitiveOpType.COPY, src_chunk=Chunk({c}, p, chunk_elems, off), tgt_chunk=Chunk({c}, r, chunk_elems, off),
+                src_device=p, tgt_device=r, dependencies=[prev[p]],
+                metadata={"src_buffer": "out", "tgt_buffer": "out", "level": 1 + step})
+        prev = cur
+    return ir, W * chunk_elems
+
+
+def direct_allreduce(world, slice_elems, dtype="bf16", compute="sum", name="direct_allreduce"):
+    """The one-exchange all-reduce for a fully connected node: rank d folds slice d of all W
+    "in" buffers in rank order (one W-input REDUCE, W <= 8), then one COPY stores the result
+    into the other ranks' "out" (W-1 destinations).  Same ops as the native generator
+    ``pccl_schedule_write_direct_allreduce``.  Returns (ir, elems)."""
+    W = world
+    if W > 8:
+        raise ValueError("direct all-reduce folds one input per rank: at most 8 ranks")
+    ir = _ring_ir(name, W, dtype, compute)
+    full = set(range(W))
+    for d in range(W):
+        off = d * slice_elems
+        red = ir.create_operation(
+            PrimitiveOpType.REDUCE if W > 1 else PrimitiveOpType.COPY,
+            src_chunk=Chunk(full, d, slice_elems, off), tgt_chunk=Chunk(full, d, slice_elems, off),
+            src_device=d, tgt_device=d, dependencies=[],
+            metadata={"srcs": [("in", r, off) for r in range(W)], "src_buffer": "in", "tgt_buffer": "out", "level": 1})
+        if W > 1:
+            others = [r for r in range(W) if r != d]
+            ir.create_operation(
+                PrimitiveOpType.COPY, src_chunk=Chunk(full, d, slice_elems, off), tgt_chunk=Chunk(full, others[0], slice_elems, off),
+                src_device=d, tgt_device=others[0], dependencies=[red],
+                metadata={"src_buffer": "out", "tgt_buffer": "out", "dsts": [("out", r, off) for r in others[1:]], "level": 2})
+    return ir, W * slice_elems
+
+
+def broadcast(world, elems, root=0, dtype="bf16", name="broadcast"):
+    """Root's "in" to every rank's "out": one COPY with W destinations (W <= 8)."""
+    W = world
+    if W > 8:
+        raise ValueError("one COPY names at most 8 destinations")
+    ir = _ring_ir(name, W, dtype, "sum")
+    full = {root}
+    others = [r for r in range(W) if r != root]
+    ir.create_operation(
+        PrimitiveOpType.COPY, src_chunk=Chunk(full, root, elems, 0), tgt_chunk=Chunk(full, root, elems, 0),
+        src_device=root, tgt_device=root, dependencies=[],
+        metadata={"src_buffer": "in", "tgt_buffer": "out", "dsts": [("out", r, 0) for r in others], "level": 1})
+    return ir, elems
 
 
 def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", name="ring_allreduce_signalled",
@@ -120,7 +213,7 @@ def small_message_allreduce(world=8, n_slices=36, n_extra=64, seed=4, lo_bytes=8
     share it), plus `n_extra` independent level-1 COPY ops in -> out with sizes drawn the same
     way.  world=8, 36 slices, 64 extras: 36*112 + 64 = 4096 ops, DAG depth 14.
     Returns (ir, elements_per_rank)."""
-    es = 4 if dtype in ("f32", "i32") else 2
+    es = ELEM_BYTES[dtype]
     sizes = log_uniform_sizes(n_slices + n_extra, seed, lo_bytes, hi_bytes, es)
     ir = _ring_ir("small_message_allreduce", world, dtype, compute)
     base = 0

@@ -189,3 +189,26 @@ def test_ring_schedule_other_dtypes(E, eng, oracle, tmp_path, dtype, compute):
     eng.exeOp("ring_" + dtype, d_in, d_out, stream)
     eng.waitOp("ring_" + dtype, stream)
     H.assert_bits_equal(d_out.cpu().numpy().view(H.STORAGE[dtype]), want, "engine ring %s %s" % (dtype, compute))
+
+
+@pytest.mark.parametrize("which", ["reduce_scatter", "all_gather", "direct", "broadcast"])
+def test_python_emitted_collectives(E, eng, oracle, tmp_path, which):
+    """The other emitters of pccl_amd.lang through regOp / exeOp, against the CPU replay of the
+    same schedule file."""
+    import torch
+    from pccl_amd import lang
+    W, n, dtype = 8, 20011, "bf16"
+    ir, per = {"reduce_scatter": lambda: lang.ring_reduce_scatter(W, n, dtype, "sum"),
+               "all_gather": lambda: lang.ring_all_gather(W, n, dtype),
+               "direct": lambda: lang.direct_allreduce(W, n, dtype, "sum"),
+               "broadcast": lambda: lang.broadcast(W, 3 * n, root=5, dtype=dtype)}[which]()
+    p = str(tmp_path / (which + ".sched"))
+    ir.save(p, per)
+    eng.regOp(which, p)
+    total = W * per
+    host_in = H.gen(dtype, total, 77, 0)
+    hdr, want = _oracle_replay(oracle, open(p).read(), host_in)
+    d_in, d_out = _to_dev(torch, host_in), torch.zeros(total * 2, dtype=torch.uint8, device="cuda")
+    eng.exeOp(which, d_in, d_out)
+    eng.waitOp(which)
+    H.assert_bits_equal(d_out.cpu().numpy().view(np.uint16), want, which)

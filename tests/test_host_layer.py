@@ -4,8 +4,10 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
+import helpers as H
 import schedules as S
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -144,6 +146,64 @@ def test_schedule_order_matches_reference_rule(E, oracle, tmp_path):
     assert info["order"] == [o.op_id for o in ir.get_operation_sequence()]
     pos = {op: i for i, op in enumerate(info["order"])}
     assert all(pos[d] < pos[i] for i, o in enumerate(ops) for d in o["deps"])
+
+
+def _replay_ir(oracle, ir, per, dtype, host_in):
+    """Runs a Python-emitted schedule on the CPU checker: returns the "out" buffers of all ranks."""
+    hdr, ops = S.parse_schedule_text(ir.serialize(per))
+    W = hdr["devices"]
+    out = np.zeros(W * per, dtype=H.STORAGE[dtype])
+    bufs = {"in": host_in, "out": out}
+    order = oracle.topo_sort(len(ops), S.edges_of(ops))
+    oracle.run_ops(S.materialise(ops, lambda b, r, e, n: bufs[b][r * per + e:r * per + e + n]), order)
+    return out.reshape(W, per)
+
+
+def test_python_collectives_compute_what_they_say(E, oracle, tmp_path):
+    """reduce-scatter, all-gather, direct all-reduce and broadcast emitters, replayed on the CPU
+    checker and compared with their definitions in numpy terms."""
+    from pccl_amd import lang
+    W, n = 5, 37
+    x = H.gen("f32", W * W * n, 60, 0).reshape(W, W * n)          # rank r's "in": W chunks of n
+    flat = x.reshape(-1)
+    # reduce-scatter: rank r ends with chunk (r+1) mod W folded around the ring from the chunk's own rank
+    ir, per = lang.ring_reduce_scatter(W, n, "f32", "sum")
+    out = _replay_ir(oracle, ir, per, "f32", flat)
+    for r in range(W):
+        c = (r + 1) % W
+        acc = x[c, c * n:(c + 1) * n].copy()
+        for i in range(1, W):
+            acc = (x[(c + i) % W, c * n:(c + 1) * n] + acc).astype(np.float32)     # incoming first, then own
+        H.assert_bits_equal(out[r, c * n:(c + 1) * n], acc, "reduce-scatter rank %d" % r)
+    # all-gather: every rank's out = concatenation of chunk r of rank r
+    ir, per = lang.ring_all_gather(W, n, "f32")
+    out = _replay_ir(oracle, ir, per, "f32", flat)
+    want = np.concatenate([x[r, r * n:(r + 1) * n] for r in range(W)])
+    for r in range(W):
+        H.assert_bits_equal(out[r], want, "all-gather rank %d" % r)
+    # direct all-reduce: every rank's out = fold over ranks 0..W-1 in that order; same text as the native generator
+    ir, per = lang.direct_allreduce(W, n, "f32", "sum")
+    out = _replay_ir(oracle, ir, per, "f32", flat)
+    want = oracle.reduce("f32", "sum", [x[r].copy() for r in range(W)])
+    for r in range(W):
+        H.assert_bits_equal(out[r], want, "direct all-reduce rank %d" % r)
+    p = str(tmp_path / "d.sched")
+    for world in (1, 2, 8):
+        E.write_direct_allreduce(p, "f32", "sum", world, n)
+        ir, per = lang.direct_allreduce(world, n, "f32", "sum")
+        assert open(p).read().replace("name direct_allreduce_%d" % world, "name direct_allreduce") == ir.serialize(per) \
+            or open(p).read().split("\n", 2)[2] == ir.serialize(per).split("\n", 2)[2]
+    # broadcast from rank 3
+    ir, per = lang.broadcast(W, 3 * n, root=3, dtype="f32")
+    out = _replay_ir(oracle, ir, per, "f32", x[:, :3 * n].copy().reshape(-1))
+    for r in range(W):
+        H.assert_bits_equal(out[r], x[3, :3 * n], "broadcast rank %d" % r)
+    with pytest.raises(ValueError):
+        lang.direct_allreduce(9, 4)
+    # element sizes of every dtype name
+    for dt, es in lang.ELEM_BYTES.items():
+        ir, per = lang.small_message_allreduce(world=2, n_slices=2, n_extra=1, lo_bytes=64, hi_bytes=128, dtype=dt)
+        assert 64 // es <= per
 
 
 def test_direct_allreduce_schedule_shape(E, tmp_path):
