@@ -269,6 +269,28 @@ int pccl_schedule_write_direct_allreduce(const char *path, const char *dtype, co
   });
 }
 
+int pccl_schedule_write_collective(const char *path, const char *kind, const char *dtype, const char *compute,
+                                   int devices, long elems, int root) {
+  if (!path || !kind || !dtype || !compute) return bad_arg("null argument");
+  return guarded([&] {
+    if (devices < 1 || elems < 0) throw std::runtime_error("devices must be >= 1 and elems >= 0");
+    Schedule s;
+    s.name = kind;
+    s.dtype = dtype;
+    s.compute = compute;
+    s.devices = devices;
+    const std::string k = kind;
+    if (k == "ring_allreduce") appendRingAllReduce(s, elems, 0);
+    else if (k == "direct_allreduce") appendDirectAllReduce(s, elems, 0);
+    else if (k == "ring_reduce_scatter") appendRingReduceScatter(s, elems, 0);
+    else if (k == "ring_all_gather") appendRingAllGather(s, elems, 0);
+    else if (k == "broadcast") appendBroadcast(s, elems, root, 0);
+    else throw std::runtime_error("unknown collective '" + k + "'");
+    s.validate();
+    s.save(path);
+  });
+}
+
 int pccl_schedule_write_small_message(const char *path, const char *dtype, int devices, int n_slices, int n_extra,
                                       unsigned long seed, long lo_bytes, long hi_bytes) {
   if (!path || !dtype) return bad_arg("null argument");

@@ -270,6 +270,79 @@ long appendRingAllReduce(Schedule &s, long chunk_elems, long base) {
   return end;
 }
 
+long appendRingReduceScatter(Schedule &s, long chunk_elems, long base) {
+  const int W = s.devices;
+  std::vector<int> prev(W, -1), cur(W, -1);
+  auto mod = [W](int x) { return ((x % W) + W) % W; };
+  for (int step = 1; step < W; ++step) {
+    for (int r = 0; r < W; ++r) {
+      const int c = mod(r - step), p = mod(r - 1);
+      const long off = base + (long)c * chunk_elems;
+      ScheduleOp o;
+      o.kind = ScheduleOp::REDUCE;
+      o.reduce = true;
+      o.count = chunk_elems;
+      o.srcs.push_back({step == 1 ? "in" : "out", p, off});
+      o.srcs.push_back({"in", r, off});
+      o.dsts.push_back({"out", r, off});
+      if (step > 1) o.deps.push_back(prev[p]);
+      cur[r] = (int)s.ops.size();
+      s.ops.push_back(std::move(o));
+    }
+    prev = cur;
+  }
+  const long end = base + (long)W * chunk_elems;
+  if (end > s.elems_per_device) s.elems_per_device = end;
+  return end;
+}
+
+long appendRingAllGather(Schedule &s, long chunk_elems, long base) {
+  const int W = s.devices;
+  std::vector<int> prev(W, -1), cur(W, -1);
+  auto mod = [W](int x) { return ((x % W) + W) % W; };
+  for (int r = 0; r < W; ++r) {  // own chunk: in -> out
+    ScheduleOp o;
+    o.count = chunk_elems;
+    o.srcs.push_back({"in", r, base + (long)r * chunk_elems});
+    o.dsts.push_back({"out", r, base + (long)r * chunk_elems});
+    prev[r] = (int)s.ops.size();
+    s.ops.push_back(std::move(o));
+  }
+  for (int step = 1; step < W; ++step) {
+    for (int r = 0; r < W; ++r) {
+      const int c = mod(r - step), p = mod(r - 1);
+      const long off = base + (long)c * chunk_elems;
+      ScheduleOp o;
+      o.count = chunk_elems;
+      o.srcs.push_back({"out", p, off});
+      o.dsts.push_back({"out", r, off});
+      o.deps.push_back(prev[p]);
+      cur[r] = (int)s.ops.size();
+      s.ops.push_back(std::move(o));
+    }
+    prev = cur;
+  }
+  const long end = base + (long)W * chunk_elems;
+  if (end > s.elems_per_device) s.elems_per_device = end;
+  return end;
+}
+
+long appendBroadcast(Schedule &s, long elems, int root, long base) {
+  const int W = s.devices;
+  if (W > 8) bad("broadcast names one destination per device: at most 8 devices");
+  if (root < 0 || root >= W) bad("broadcast root outside the devices");
+  ScheduleOp o;
+  o.count = elems;
+  o.srcs.push_back({"in", root, base});
+  o.dsts.push_back({"out", root, base});
+  for (int r = 0; r < W; ++r)
+    if (r != root) o.dsts.push_back({"out", r, base});
+  s.ops.push_back(std::move(o));
+  const long end = base + elems;
+  if (end > s.elems_per_device) s.elems_per_device = end;
+  return end;
+}
+
 long appendDirectAllReduce(Schedule &s, long slice_elems, long base) {
   const int W = s.devices;
   if (W > 8) bad("direct all-reduce supports at most 8 devices (8 inputs per op)");

@@ -80,6 +80,16 @@ long appendRingAllReduce(Schedule &s, long chunk_elems, long base);
 // W-input op and writes it to every device's output (W outputs), W ops, no dependencies.
 long appendDirectAllReduce(Schedule &s, long slice_elems, long base);
 
+// The two halves of the ring on their own.  Reduce-scatter: after W-1 steps device r holds the
+// fold of chunk (r+1) mod W in its "out".  All-gather: device r contributes chunk r of its "in";
+// afterwards every "out" holds all W chunks.
+long appendRingReduceScatter(Schedule &s, long chunk_elems, long base);
+long appendRingAllGather(Schedule &s, long chunk_elems, long base);
+
+// Broadcast of `elems` elements of device `root`'s "in" into every device's "out": one COPY
+// with W destinations (W <= 8).
+long appendBroadcast(Schedule &s, long elems, int root, long base);
+
 // The small-message program: n_slices ring all-reduces with log-uniform chunk sizes in
 // [lo_bytes, hi_bytes] plus n_extra independent copies; seed selects the sizes.
 Schedule makeSmallMessageSchedule(int devices, int n_slices, int n_extra, unsigned long seed,

@@ -58,6 +58,7 @@ def lib():
             "pccl_env_register_opt": [cs],
             "pccl_schedule_write_ring_allreduce": [cs, cs, cs, ci, cl],
             "pccl_schedule_write_direct_allreduce": [cs, cs, cs, ci, cl],
+            "pccl_schedule_write_collective": [cs, cs, cs, cs, ci, cl, ci],
             "pccl_schedule_write_small_message": [cs, cs, ci, ci, ci, ctypes.c_ulong, cl, cl],
             "pccl_schedule_inspect": [cs, P(ci), P(ci), P(cl), P(ci), ci],
         }
@@ -239,6 +240,10 @@ def write_ring_allreduce(path, dtype, compute, devices, chunk_elems):
 
 def write_direct_allreduce(path, dtype, compute, devices, slice_elems):
     _check(lib().pccl_schedule_write_direct_allreduce(_b(path), _b(dtype), _b(compute), devices, slice_elems))
+
+
+def write_collective(path, kind, dtype, compute, devices, elems, root=0):
+    _check(lib().pccl_schedule_write_collective(_b(path), _b(kind), _b(dtype), _b(compute), devices, elems, root))
 
 
 def write_small_message(path, dtype="bf16", devices=8, n_slices=36, n_extra=64, seed=4, lo_bytes=8 << 10,

@@ -130,6 +130,16 @@ def test_native_and_python_emitters_agree(E, tmp_path):
         E.write_ring_allreduce(p, dt, op, world, n)
         ir, per = lang.ring_allreduce(world, n, dt, op)
         assert open(p).read() == ir.serialize(per)
+        for kind, emit in (("ring_allreduce", lambda: lang.ring_allreduce(world, n, dt, op)),
+                           ("direct_allreduce", lambda: lang.direct_allreduce(world, n, dt, op)),
+                           ("ring_reduce_scatter", lambda: lang.ring_reduce_scatter(world, n, dt, op)),
+                           ("ring_all_gather", lambda: lang.ring_all_gather(world, n, dt)),
+                           ("broadcast", lambda: lang.broadcast(world, n, root=world - 1, dtype=dt))):
+            E.write_collective(p, kind, dt, op if kind not in ("ring_all_gather", "broadcast") else "sum", world, n, world - 1)
+            ir, per = emit()
+            assert open(p).read() == ir.serialize(per), kind
+    with pytest.raises(E.EngineError):
+        E.write_collective(p, "all_to_all", "f32", "sum", 4, 8)
 
 
 def test_schedule_order_matches_reference_rule(E, oracle, tmp_path):
