@@ -78,8 +78,8 @@ int pccl_schedule_write_ring_allreduce(const char *path, const char *dtype, cons
                                        long chunk_elems);
 int pccl_schedule_write_direct_allreduce(const char *path, const char *dtype, const char *compute, int devices,
                                          long slice_elems);
-/* kind: "ring_allreduce", "direct_allreduce", "ring_reduce_scatter", "ring_all_gather" (elems = per
- * chunk / slice) or "broadcast" (elems in all, from device `root`; root is ignored otherwise). */
+/* kind: "ring_allreduce", "direct_allreduce", "ring_reduce_scatter", "ring_all_gather", "all_to_all"
+ * (elems = per chunk / slice) or "broadcast" (elems in all, from device `root`; root is ignored otherwise). */
 int pccl_schedule_write_collective(const char *path, const char *kind, const char *dtype, const char *compute,
                                    int devices, long elems, int root);
 int pccl_schedule_write_small_message(const char *path, const char *dtype, int devices, int n_slices, int n_extra,

@@ -285,6 +285,7 @@ int pccl_schedule_write_collective(const char *path, const char *kind, const cha
     else if (k == "ring_reduce_scatter") appendRingReduceScatter(s, elems, 0);
     else if (k == "ring_all_gather") appendRingAllGather(s, elems, 0);
     else if (k == "broadcast") appendBroadcast(s, elems, root, 0);
+    else if (k == "all_to_all") appendAllToAll(s, elems, 0);
     else throw std::runtime_error("unknown collective '" + k + "'");
     s.validate();
     s.save(path);

@@ -343,6 +343,21 @@ long appendBroadcast(Schedule &s, long elems, int root, long base) {
   return end;
 }
 
+long appendAllToAll(Schedule &s, long chunk_elems, long base) {
+  const int W = s.devices;
+  for (int r = 0; r < W; ++r)
+    for (int d = 0; d < W; ++d) {
+      ScheduleOp o;
+      o.count = chunk_elems;
+      o.srcs.push_back({"in", r, base + (long)d * chunk_elems});
+      o.dsts.push_back({"out", d, base + (long)r * chunk_elems});
+      s.ops.push_back(std::move(o));
+    }
+  const long end = base + (long)W * chunk_elems;
+  if (end > s.elems_per_device) s.elems_per_device = end;
+  return end;
+}
+
 long appendDirectAllReduce(Schedule &s, long slice_elems, long base) {
   const int W = s.devices;
   if (W > 8) bad("direct all-reduce supports at most 8 devices (8 inputs per op)");

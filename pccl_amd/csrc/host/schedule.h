@@ -90,6 +90,9 @@ long appendRingAllGather(Schedule &s, long chunk_elems, long base);
 // with W destinations (W <= 8).
 long appendBroadcast(Schedule &s, long elems, int root, long base);
 
+// All-to-all: device r's "in" chunk d goes to device d's "out" chunk r; W*W independent copies.
+long appendAllToAll(Schedule &s, long chunk_elems, long base);
+
 // The small-message program: n_slices ring all-reduces with log-uniform chunk sizes in
 // [lo_bytes, hi_bytes] plus n_extra independent copies; seed selects the sizes.
 Schedule makeSmallMessageSchedule(int devices, int n_slices, int n_extra, unsigned long seed,

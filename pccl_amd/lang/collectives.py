@@ -152,6 +152,20 @@ def broadcast(world, elems, root=0, dtype="bf16", name="broadcast"):
     return ir, elems
 
 
+def all_to_all(world, chunk_elems, dtype="bf16", name="all_to_all"):
+    """Rank r's "in" chunk d goes to rank d's "out" chunk r: W*W independent COPY ops (the
+    diagonal ones stay on their rank)."""
+    W = world
+    ir = _ring_ir(name, W, dtype, "sum")
+    for r in range(W):
+        for d in range(W):
+            ir.create_operation(
+                PrimitiveOpType.COPY, src_chunk=Chunk({r}, r, chunk_elems, d * chunk_elems),
+                tgt_chunk=Chunk({r}, d, chunk_elems, r * chunk_elems), src_device=r, tgt_device=d, dependencies=[],
+                metadata={"src_buffer": "in", "tgt_buffer": "out", "level": 1})
+    return ir, W * chunk_elems
+
+
 def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", name="ring_allreduce_signalled",
                              first_slot=0):
     """The same ring all-reduce written the way ranks on different GPUs have to write it:

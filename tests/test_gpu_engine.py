@@ -191,7 +191,7 @@ def test_ring_schedule_other_dtypes(E, eng, oracle, tmp_path, dtype, compute):
     H.assert_bits_equal(d_out.cpu().numpy().view(H.STORAGE[dtype]), want, "engine ring %s %s" % (dtype, compute))
 
 
-@pytest.mark.parametrize("which", ["reduce_scatter", "all_gather", "direct", "broadcast"])
+@pytest.mark.parametrize("which", ["reduce_scatter", "all_gather", "direct", "broadcast", "all_to_all"])
 def test_python_emitted_collectives(E, eng, oracle, tmp_path, which):
     """The other emitters of pccl_amd.lang through regOp / exeOp, against the CPU replay of the
     same schedule file."""
@@ -201,7 +201,8 @@ def test_python_emitted_collectives(E, eng, oracle, tmp_path, which):
     ir, per = {"reduce_scatter": lambda: lang.ring_reduce_scatter(W, n, dtype, "sum"),
                "all_gather": lambda: lang.ring_all_gather(W, n, dtype),
                "direct": lambda: lang.direct_allreduce(W, n, dtype, "sum"),
-               "broadcast": lambda: lang.broadcast(W, 3 * n, root=5, dtype=dtype)}[which]()
+               "broadcast": lambda: lang.broadcast(W, 3 * n, root=5, dtype=dtype),
+               "all_to_all": lambda: lang.all_to_all(W, n, dtype)}[which]()
     p = str(tmp_path / (which + ".sched"))
     ir.save(p, per)
     eng.regOp(which, p)

@@ -134,12 +134,13 @@ def test_native_and_python_emitters_agree(E, tmp_path):
                            ("direct_allreduce", lambda: lang.direct_allreduce(world, n, dt, op)),
                            ("ring_reduce_scatter", lambda: lang.ring_reduce_scatter(world, n, dt, op)),
                            ("ring_all_gather", lambda: lang.ring_all_gather(world, n, dt)),
+                           ("all_to_all", lambda: lang.all_to_all(world, n, dt)),
                            ("broadcast", lambda: lang.broadcast(world, n, root=world - 1, dtype=dt))):
-            E.write_collective(p, kind, dt, op if kind not in ("ring_all_gather", "broadcast") else "sum", world, n, world - 1)
+            E.write_collective(p, kind, dt, op if kind not in ("ring_all_gather", "broadcast", "all_to_all") else "sum", world, n, world - 1)
             ir, per = emit()
             assert open(p).read() == ir.serialize(per), kind
     with pytest.raises(E.EngineError):
-        E.write_collective(p, "all_to_all", "f32", "sum", 4, 8)
+        E.write_collective(p, "all_to_some", "f32", "sum", 4, 8)
 
 
 def test_schedule_order_matches_reference_rule(E, oracle, tmp_path):
@@ -203,6 +204,12 @@ def test_python_collectives_compute_what_they_say(E, oracle, tmp_path):
         ir, per = lang.direct_allreduce(world, n, "f32", "sum")
         assert open(p).read().replace("name direct_allreduce_%d" % world, "name direct_allreduce") == ir.serialize(per) \
             or open(p).read().split("\n", 2)[2] == ir.serialize(per).split("\n", 2)[2]
+    # all-to-all: out[d] chunk r = in[r] chunk d
+    ir, per = lang.all_to_all(W, n, "f32")
+    out = _replay_ir(oracle, ir, per, "f32", flat)
+    for d in range(W):
+        for r in range(W):
+            H.assert_bits_equal(out[d, r * n:(r + 1) * n], x[r, d * n:(d + 1) * n], "all-to-all %d <- %d" % (d, r))
     # broadcast from rank 3
     ir, per = lang.broadcast(W, 3 * n, root=3, dtype="f32")
     out = _replay_ir(oracle, ir, per, "f32", x[:, :3 * n].copy().reshape(-1))
