@@ -91,10 +91,28 @@ def cpu_baseline(count_sample):
             orc.reduce_copy("bf16", "sum", ins, [out], count_sample, nthreads=threads)
             ts.append(time.perf_counter() - t0)
         best[threads] = nbytes / min(ts) / 1e9
+    # the two other shapes of the measurement plan, same code: f32 2 -> 1 at 4 MiB per buffer and one
+    # ring reduce step (bf16 2 -> 2, 32 MiB per buffer)
+    other = {}
+    a32 = [np.random.default_rng(20 + k).random(1 << 20, dtype=np.float32) for k in range(2)]
+    o32 = np.empty(1 << 20, dtype=np.float32)
+    ring_in = [x[:1 << 24] if count_sample >= (1 << 24) else np.resize(x, 1 << 24) for x in ins[:2]]
+    ring_out = [np.empty(1 << 24, dtype=np.uint16) for _ in range(2)]
+    for name, dt, i_, o_, n_, nb in (("f32_2in_1out_4MiB", "f32", a32, [o32], 1 << 20, 3 * 4 << 20),
+                                     ("bf16_2in_2out_32MiB_ring_step", "bf16", ring_in, ring_out, 1 << 24, 4 * 32 << 20)):
+        r = {}
+        for threads in (1, cores):
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                orc.reduce_copy(dt, "sum", i_, o_, n_, nthreads=threads)
+                ts.append(time.perf_counter() - t0)
+            r["GBps_%d_thread%s" % (threads, "" if threads == 1 else "s")] = round(nb / min(ts) / 1e9, 2)
+        other[name] = r
     return {"value": round(best[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": "bf16 8->1 sum, %d elements per buffer (1/%d of the headline buffers), best of 5; "
                       "single thread: %.2f GB/s" % (count_sample, (1 << 27) // count_sample, best[1]),
-            "host_cpus_visible": os.cpu_count()}
+            "other_shapes": other, "host_cpus_visible": os.cpu_count()}
 
 
 def main():
