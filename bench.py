@@ -29,7 +29,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--extras", default="all", metavar="LIST",
-                    help="comma-separated secondary workloads to run: nvls, accumulate, ring, plumbing, unaligned, "
+                    help="comma-separated secondary workloads to run: layout, nvls, accumulate, ring, plumbing, unaligned, "
                          "op64k, schedule (one persistent launch), schedule_launches (the same ops as 4096 launches), "
                          "or all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -175,6 +175,23 @@ def main():
         return "all" in chosen or name in chosen
 
     if not args.no_extras:
+        # ---- the headline shape on buffers out of one staggered allocation --------------------
+        if want("layout"):
+            ptrs = hip.alloc_group(9, count * 2)      # built-in stagger between the nine buffers
+            for k in range(8):
+                hip.reduce_copy("bf16", "sum", [ins[k]], [ptrs[k]], count, stream)
+            t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", ptrs[:8], [ptrs[8]], count, stream), 30, 5)
+            chk = torch.empty_like(out)
+            hip.reduce_copy("bf16", "sum", [ptrs[8]], [chk], count, stream)
+            torch.cuda.synchronize()
+            assert torch.equal(chk, out), "staggered-layout run differs from the headline output"
+            extras["headline_shape_staggered_group"] = dict(
+                stats(t), GBps_median=gbps(step_bytes, t[len(t) // 2]),
+                note="same kernel and data as the headline, operands from pccl_hip_alloc_group (one allocation, "
+                     "buffers %d bytes apart) instead of nine separate allocations" % (ptrs[1] - ptrs[0]))
+            hip.free(ptrs[0])
+            del chk
+
         # ---- 128 MiB variants: bf16 8->1 and fp16 8->2 ------------------------------------
         if want("nvls"):
             c3 = 1 << 26

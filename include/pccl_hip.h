@@ -81,6 +81,16 @@ int pccl_hip_device_info(int *compute_units, long *hbm_bytes, char *name, int na
 int pccl_hip_alloc(void **p, long nbytes);
 int pccl_hip_free(void *p);
 
+/* n buffers of nbytes_each out of ONE allocation, ptrs[k] = base + k * (nbytes_each rounded to 256
+ * + pad_bytes rounded to 256); pad_bytes < 0 = built-in choice.  For operands that a reduce-copy
+ * reads at the same offset at the same time: buffers whose addresses agree in the bits that select
+ * HBM stack, channel and bank (what separately allocated, 2 MiB-aligned buffers do) collide there,
+ * and a stagger of a few hundred KiB between them is worth 2-4 % of bandwidth
+ * (bf16 8 -> 1 at 256 MiB: 6.5 -> 6.8 TB/s).  The best stagger depends on the buffer size; this is
+ * an option for callers that measure, not something pccl_hip_alloc does on its own.
+ * Free the whole group with pccl_hip_free(ptrs[0]).  No counterpart in the reference. */
+int pccl_hip_alloc_group(void **ptrs, int n, long nbytes_each, long pad_bytes);
+
 /* ---- the hot path: one reduce-copy ---------------------------------------- */
 
 /* out[j][i] = cvt(fold_op(up(in[0][i]) ... up(in[n_in-1][i]))) for j < n_out,

@@ -56,6 +56,13 @@ Tuning tuning() {
   return g_tuning;
 }
 
+// Distance added between the buffers of a group when the caller leaves the choice open.
+// Measured with bf16 reductions on group allocations (TB/s at pad 0 -> at this pad): 8 -> 1 at
+// 256 MiB 6.5 -> 6.8, at 128 MiB 6.6 -> 6.75, 8 -> 2 at 128 MiB 6.65 -> 6.9, 2 -> 2 at 32 MiB
+// 7.1 -> 7.1.  Pads of 4-68 KiB help the 256 MiB case as much but cost the 128 MiB cases 10 %,
+// and 1028 KiB does the opposite, so the effect is not monotonic in the pad.
+constexpr long kDefaultGroupPad = (576l << 10) + 4096;
+
 static std::mutex g_mem_mutex;
 static std::unordered_map<void *, long> &mem_map() {
   static std::unordered_map<void *, long> m;
@@ -112,6 +119,28 @@ int pccl_hip_alloc(void **p, long nbytes) {
   std::lock_guard<std::mutex> lock(g_mem_mutex);
   mem_map()[q] = rounded;
   *p = q;
+  return PCCL_OK;
+}
+
+int pccl_hip_alloc_group(void **ptrs, int n, long nbytes_each, long pad_bytes) {
+  clear_error();
+  if (!ptrs || n < 1) return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_alloc_group: ptrs is null or n %d < 1", n);
+  for (int k = 0; k < n; ++k) ptrs[k] = nullptr;
+  if (nbytes_each <= 0) return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_alloc_group: nbytes_each %ld <= 0", nbytes_each);
+  if (pad_bytes < 0) pad_bytes = kDefaultGroupPad;
+  pad_bytes = (pad_bytes + 255) / 256 * 256;
+  const long stride = (nbytes_each + 255) / 256 * 256 + pad_bytes;
+  const long gran = 2l << 20;
+  const long rounded = ((long)n * stride + gran - 1) / gran * gran;
+  void *q = nullptr;
+  hipError_t e = hipMalloc(&q, (size_t)rounded);
+  if (e != hipSuccess || !q) {
+    (void)hipGetLastError();
+    return fail(PCCL_ERR_NOMEM, "hipMalloc(%ld): %s", rounded, hipGetErrorString(e));
+  }
+  std::lock_guard<std::mutex> lock(g_mem_mutex);
+  mem_map()[q] = rounded;  // the group is freed through its first buffer
+  for (int k = 0; k < n; ++k) ptrs[k] = (char *)q + (long)k * stride;
   return PCCL_OK;
 }
 

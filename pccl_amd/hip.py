@@ -67,6 +67,7 @@ def lib():
         L.pccl_hip_device_info.argtypes = [ctypes.POINTER(ci), ctypes.POINTER(cl), ctypes.c_char_p, ci]
         L.pccl_hip_alloc.argtypes = [ctypes.POINTER(vp), cl]
         L.pccl_hip_free.argtypes = [vp]
+        L.pccl_hip_alloc_group.argtypes = [ctypes.POINTER(vp), ci, cl, cl]
         L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_accumulate.argtypes = [ci, ci, vp, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_set_tuning.argtypes = [ci, ci]
@@ -123,6 +124,13 @@ def alloc(nbytes):
     p = ctypes.c_void_p(None)
     _check(lib().pccl_hip_alloc(ctypes.byref(p), nbytes))
     return p.value
+
+
+def alloc_group(n, nbytes_each, pad_bytes=-1):
+    """n buffers out of one allocation, staggered by pad_bytes; free the group with free(ptrs[0])."""
+    arr = (ctypes.c_void_p * n)()
+    _check(lib().pccl_hip_alloc_group(arr, n, nbytes_each, pad_bytes))
+    return [arr[k] for k in range(n)]
 
 
 def free(ptr):
