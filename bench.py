@@ -19,7 +19,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size (figures and commands in
 # profiles/reduce_copy_bf16_8in_256MiB.md).
-MEASURED_TRAFFIC_BYTES = 2415785223
+MEASURED_TRAFFIC_BYTES = 2415753079
 
 
 def parse():
@@ -136,9 +136,17 @@ def main():
     ins = [randn(torch, count, "bf16") for _ in range(8)]
     out = torch.empty(count, dtype=torch.bfloat16, device="cuda")
     step_bytes = 9 * count * 2
+    # The timed operands come from the device plugin's own allocator, as PCCL's operands do (its
+    # BufferManager sub-allocates one plugin-allocated workspace): nine buffers of one allocation,
+    # the built-in stagger apart.  The same data in nine separately allocated torch tensors is timed
+    # below as "headline_shape_separate_allocations".
+    operands = hip.alloc_group(9, count * 2)
+    for k in range(8):
+        hip.reduce_copy("bf16", "sum", [ins[k]], [operands[k]], count, stream)
+    torch.cuda.synchronize()
 
     def step():
-        hip.reduce_copy("bf16", "sum", ins, [out], count, stream)
+        hip.reduce_copy("bf16", "sum", operands[:8], [operands[8]], count, stream)
 
     for _ in range(args.warmup):
         step()
@@ -160,12 +168,14 @@ def main():
                 "launch_us": stats(ts)}
 
     # quick self-check of the timed buffers against torch's fp32 accumulate (same fold order)
+    hip.reduce_copy("bf16", "sum", [operands[8]], [out], count, stream)
+    torch.cuda.synchronize()
     ref = ins[0][:1 << 20].float()
     for k in range(1, 8):
         ref = ref + ins[k][:1 << 20].float()
     assert torch.equal(ref.to(torch.bfloat16), out[:1 << 20]), "headline output differs from fp32-accumulated fold"
     for _ in range(args.calibration_copy):
-        hip.reduce_copy("bf16", "sum", [ins[0]], [out], count, stream)
+        hip.reduce_copy("bf16", "sum", [operands[0]], [operands[8]], count, stream)
     torch.cuda.synchronize()
 
     extras = {}
@@ -175,22 +185,16 @@ def main():
         return "all" in chosen or name in chosen
 
     if not args.no_extras:
-        # ---- the headline shape on buffers out of one staggered allocation --------------------
+        # ---- the headline shape on nine separately allocated torch tensors ---------------------
         if want("layout"):
-            ptrs = hip.alloc_group(9, count * 2)      # built-in stagger between the nine buffers
-            for k in range(8):
-                hip.reduce_copy("bf16", "sum", [ins[k]], [ptrs[k]], count, stream)
-            t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", ptrs[:8], [ptrs[8]], count, stream), 30, 5)
-            chk = torch.empty_like(out)
-            hip.reduce_copy("bf16", "sum", [ptrs[8]], [chk], count, stream)
-            torch.cuda.synchronize()
-            assert torch.equal(chk, out), "staggered-layout run differs from the headline output"
-            extras["headline_shape_staggered_group"] = dict(
+            full = out.clone()
+            t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", ins, [out], count, stream), 30, 5)
+            assert torch.equal(full, out), "separate-allocation run differs from the headline output"
+            extras["headline_shape_separate_allocations"] = dict(
                 stats(t), GBps_median=gbps(step_bytes, t[len(t) // 2]),
-                note="same kernel and data as the headline, operands from pccl_hip_alloc_group (one allocation, "
-                     "buffers %d bytes apart) instead of nine separate allocations" % (ptrs[1] - ptrs[0]))
-            hip.free(ptrs[0])
-            del chk
+                note="same kernel and data as the headline, operands in nine separate 2 MiB-aligned allocations "
+                     "instead of one pccl_hip_alloc_group allocation (buffers %d bytes apart)" % (operands[1] - operands[0]))
+            del full
 
         # ---- 128 MiB variants: bf16 8->1 and fp16 8->2 ------------------------------------
         if want("nvls"):
@@ -322,12 +326,16 @@ def main():
                 extras["schedule_4096_ops"]["as_4096_launches"] = dict(stats(t2), us_per_op=round(t2[len(t2) // 2] / len(low), 4))
             g.destroy()
 
+    torch.cuda.synchronize()
+    hip.free(operands[0])
+
     result = {
         "metric": "reduce_copy_hbm_bandwidth", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 sum of 8 inputs -> 1 output, 134217728 elements (256 MiB) per buffer, "
-                               "N(0,1) from torch seed 2, fp32 accumulate, one launch per step",
+                               "N(0,1) from torch seed 2, fp32 accumulate, one launch per step, operands allocated by the "
+                               "plugin's group allocator (one allocation, buffers the built-in 580 KiB apart)",
                    "n_in": 8, "n_out": 1, "count": count, "bytes_per_step": step_bytes},
         "pct_of_peak_hbm": round(100.0 * value / PEAK_HBM_GBPS, 2),
         "roofline": roofline,
