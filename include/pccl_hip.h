@@ -85,9 +85,11 @@ int pccl_hip_free(void *p);
  * + pad_bytes rounded to 256); pad_bytes < 0 = built-in choice.  For operands that a reduce-copy
  * reads at the same offset at the same time: buffers whose addresses agree in the bits that select
  * HBM stack, channel and bank (what separately allocated, 2 MiB-aligned buffers do) collide there,
- * and a stagger of a few hundred KiB between them is worth 2-4 % of bandwidth
- * (bf16 8 -> 1 at 256 MiB: 6.5 -> 6.8 TB/s).  The best stagger depends on the buffer size; this is
- * an option for callers that measure, not something pccl_hip_alloc does on its own.
+ * and a stagger between them is worth 2-8 % of bandwidth (bf16 8 -> 1 at 256 MiB 6.5 -> 6.8 TB/s,
+ * 8 -> 2 at 128 MiB 6.55 -> 6.9, 2 -> 2 at 64 MiB 6.2 -> 6.75; the one loss measured: 2 -> 1 at
+ * 256 MiB 7.2 -> 7.0).  The built-in stagger is 580 KiB from 96 MiB per buffer and 20 KiB below;
+ * the effect is not monotonic in the stagger, so this is an option for callers that measure, not
+ * something pccl_hip_alloc does on its own.
  * Free the whole group with pccl_hip_free(ptrs[0]).  No counterpart in the reference. */
 int pccl_hip_alloc_group(void **ptrs, int n, long nbytes_each, long pad_bytes);
 

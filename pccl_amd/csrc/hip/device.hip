@@ -62,6 +62,10 @@ Tuning tuning() {
 // 7.1 -> 7.1.  Pads of 4-68 KiB help the 256 MiB case as much but cost the 128 MiB cases 10 %,
 // and 1028 KiB does the opposite, so the effect is not monotonic in the pad.
 constexpr long kDefaultGroupPad = (576l << 10) + 4096;
+// Below about 96 MiB per buffer that pad costs (8 -> 1 at 64 MiB: 6.8 -> 5.6-6.3) where a small one
+// is neutral or helps (8 -> 1 at 64 MiB 6.8 -> 6.85, 2 -> 2 at 64 MiB 6.2 -> 6.9).
+constexpr long kSmallBufferGroupPad = 20l << 10;
+constexpr long kSmallBufferBytes = 96l << 20;
 
 static std::mutex g_mem_mutex;
 static std::unordered_map<void *, long> &mem_map() {
@@ -127,7 +131,7 @@ int pccl_hip_alloc_group(void **ptrs, int n, long nbytes_each, long pad_bytes) {
   if (!ptrs || n < 1) return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_alloc_group: ptrs is null or n %d < 1", n);
   for (int k = 0; k < n; ++k) ptrs[k] = nullptr;
   if (nbytes_each <= 0) return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_alloc_group: nbytes_each %ld <= 0", nbytes_each);
-  if (pad_bytes < 0) pad_bytes = kDefaultGroupPad;
+  if (pad_bytes < 0) pad_bytes = nbytes_each < kSmallBufferBytes ? kSmallBufferGroupPad : kDefaultGroupPad;
   pad_bytes = (pad_bytes + 255) / 256 * 256;
   const long stride = (nbytes_each + 255) / 256 * 256 + pad_bytes;
   const long gran = 2l << 20;
