@@ -14,15 +14,14 @@
 //     XCDs, so the ticket counter of a queue is hammered from one XCD only -- and
 //     moves on to the other queues when its own is exhausted;
 //   * a workgroup claims an entry by taking a ticket from RingBuffer::head_,
-//     reads the entry, and waits until the op's dependencies are met (its ready word
-//     holds the number of this run; written by whoever takes pre_dependencies_ to 0).  Every
+//     reads the entry, and waits until the op's dependencies have arrived (its arrivals
+//     word equals pre_dependencies_, which itself stays constant).  Every
 //     dependency of a claimed entry lies earlier in the global order; each queue
 //     keeps at least one workgroup until it is exhausted; hence the unfinished
 //     claimed entry that comes first in the global order can always run, and the
 //     drain cannot deadlock whatever the number of resident workgroups;
-//   * the workgroup finishing the last part of an op decrements
-//     pre_dependencies_ of each successor (32-bit atomic on the word at offset
-//     12; the count is the low byte and never borrows);
+//   * the workgroup finishing the last part of an op adds one to the arrivals word of
+//     each successor (an atomic whose result nobody waits for) and clears its own;
 //   * data moves between workgroups (possibly on different XCDs, whose L2s are not
 //     coherent with each other) through device-coherent accesses: parts load and
 //     store with sc1, wait for their stores, and only then touch the counters with

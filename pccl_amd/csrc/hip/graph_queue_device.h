@@ -40,7 +40,7 @@ struct GraphControl {
   HotWord *hot;                           // kHot* words, see below
   const int *group_base;                  // per op: first of its kPartGroups words in `groups`, or -1
   HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
-  HotWord *ready;                         // per op: number of the run in which its dependencies were last met
+  HotWord *ready;                         // per op: dependencies that have arrived in this run
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
   int queue_count[kQueues];
@@ -233,8 +233,7 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // Thread 0, after a part of op `h` is complete: count it; the op's last part re-arms
 // the op's counters for the next run and releases its successors.
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const PayloadSlot *slot, int uid, int part, int home,
-                                            unsigned int run_no) {
+                                            const PayloadSlot *slot, int uid, int part, int home) {
   const int parts = slot->parts;
   int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
   if (parts > kGroupThreshold) {
@@ -250,17 +249,19 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   if (old != 1) return;
   if (counted > 1) __hip_atomic_store(&h->remaining_executors_, counted, __ATOMIC_RELAXED, AGENT);
   const unsigned int w12 = slot->payload.initial_word12_;
-  if (w12 & 0xffu) __hip_atomic_store(word12(h), w12, __ATOMIC_RELAXED, AGENT);
+  // The op is complete.  Its own arrivals word goes back to zero for the next run (every
+  // dependency of this op has arrived, or it could not have run), and it arrives at each
+  // successor: one add on the successor's arrivals word, whose result nobody waits for.  The
+  // workgroups that already hold parts of a successor poll that word until it equals the
+  // successor's pre_dependencies_ -- not the header, whose line the counting atomics of this
+  // and neighbouring ops need (with 1024 pollers on a header line a hand-over between two
+  // 32 MiB ops took 6 us longer), and without an atomic whose result decides who announces
+  // (that round trip was a third of the latency between two dependent ops).
+  if (w12 & 0xffu) __hip_atomic_store(&g.ready[uid].value, 0u, __ATOMIC_RELAXED, AGENT);
   const int n_next = (int)(w12 >> 24);
   const int *next = g.succ + slot->succ_start;
-  // Whoever takes a successor's count to zero announces it on the successor's own ready word:
-  // the workgroups that already hold parts of the successor poll that word, not the header,
-  // whose line the counting atomics of this and neighbouring ops need (with 1024 pollers on a
-  // header line a hand-over between two 32 MiB ops took 6 us longer).
-  for (int s = 0; s < n_next; ++s) {
-    const unsigned int before = __hip_atomic_fetch_sub(word12(&g.headers[next[s]]), 1u, __ATOMIC_RELAXED, AGENT);
-    if ((before & 0xffu) == 1u) __hip_atomic_store(&g.ready[next[s]].value, run_no, __ATOMIC_RELAXED, AGENT);
-  }
+  for (int s = 0; s < n_next; ++s)
+    __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
   __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
 }
 
@@ -289,16 +290,15 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   // in the kernel arguments) so that a launch recorded into a HIP graph uses a fresh one on
   // every replay; it is read at the first signal op, always before the last workgroup out of
   // this run bumps it.
-  unsigned int run_no = 0;
-  if (threadIdx.x == 0) run_no = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT);
-  const unsigned int signal_base = run_no << 16;
+  unsigned int signal_base = 0;
+  bool have_signal_base = false;
   for (;;) {
     if (threadIdx.x == 0) {
       // The part executed in the previous iteration is complete (barrier below): every
       // wavefront waited for its write-through stores before that barrier, so the data is
       // at the point of coherence and relaxed device-scope atomics are enough to hand it
       // over; no L2 write-back / invalidate is involved.
-      if (h) finish_part(g, h, slot, cur_uid, cur_part, home, run_no);
+      if (h) finish_part(g, h, slot, cur_uid, cur_part, home);
       int go = 0;
       unsigned long long e = 0;
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
@@ -323,10 +323,12 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         const int uid = (int)(e & 0xffffffffu);
         pccl_operation_layout_header *hc = &g.headers[uid];
         const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
-        // wait for the op's dependencies (none: nothing will ever write its ready word)
-        if ((sc->payload.initial_word12_ & 0xffu) != 0 &&
+        // wait until every dependency of the op has arrived (none: nothing ever writes the
+        // word); pre_dependencies_ in the header is the count to reach and stays constant
+        const unsigned int n_pred = __hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT) & 0xffu;
+        if (n_pred != 0 &&
             !bounded_wait(abort_flag, spin_limit, [&] {
-              return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == run_no;
+              return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == n_pred;
             })) {
           go = 0;
           break;
@@ -334,6 +336,10 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         const int prim = sc->payload.primitive_;
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
+        if (!have_signal_base) {
+          signal_base = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT) << 16;
+          have_signal_base = true;
+        }
         const unsigned int want = signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
         if (prim == PCCL_NOTIFY) {
           // everything this op depends on is already at the point of coherence
@@ -344,7 +350,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           go = 0;
           break;
         }
-        finish_part(g, hc, sc, uid, 0, home, run_no);
+        finish_part(g, hc, sc, uid, 0, home);
       }
       s_entry = e;
       s_go = go;
