@@ -180,6 +180,18 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
 int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,
                           void *stream);
 
+/* Per-entry timeline of the executor (no counterpart in the reference, whose headers
+ * keep only the two progress counters of operator.h:32-33).  enable != 0 allocates 32 bytes
+ * per queue entry once and makes the following runs record, per entry in queue order, four
+ * 64-bit words: { op_uid | part << 32 | workgroup << 52, ticket drawn, dependencies met,
+ * part complete }, times in ticks of the device's constant 100 MHz clock; each run
+ * overwrites the last.  enable == 0 stops recording.  Not to be switched while a run is in
+ * flight.  read_trace waits for `stream`, copies up to `capacity` records (4 words each)
+ * and reports the number of entries of the graph in *n_records. */
+int pccl_hip_graph_trace(void *graph, int enable);
+int pccl_hip_graph_read_trace(void *graph, void *stream, unsigned long long *records, long capacity,
+                              long *n_records);
+
 /* Device address of the GraphBufferLayout and launch facts, for inspection. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 

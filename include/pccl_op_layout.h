@@ -49,13 +49,11 @@ typedef struct pccl_ring_buffer {
 /* One DAG node, 32 bytes.
  *   required_executors_  workgroup-sized parts the op is split into;
  *   remaining_executors_ parts not yet finished (counts down, then restored);
- *   pre_dependencies_    predecessors not yet finished; the op is pushed on
- *                        its ready queue when this reaches 0.  It shares the
- *                        32-bit word at offset 12 with the three bytes after
- *                        it, and device code decrements it with a 32-bit atomic
- *                        subtract of 1 on that word (low byte, little endian;
- *                        never borrows because it is only decremented while
- *                        non-zero);
+ *   pre_dependencies_    number of predecessors; constant during a run.  Device
+ *                        code counts the predecessors that have finished on a
+ *                        word of its own per op (outside this struct, alone on a
+ *                        cache line) and runs the op when that count equals
+ *                        this field;
  *   op_buffer_/op_size_  payload: pccl_op_payload, at most 255 bytes;
  *   next_op_uids_head_   num_next_ops_ successor uids. */
 typedef struct pccl_operation_layout_header {
@@ -88,7 +86,7 @@ typedef struct pccl_op_payload {
   unsigned char compute_;   /* enum pccl_compute   */
   unsigned char n_in_;
   unsigned char n_out_;
-  unsigned int initial_word12_; /* pristine value of the header's word at offset 12 */
+  unsigned int initial_word12_; /* copy of the header's word at offset 12 (pre_dependencies_ .. num_next_ops_) */
   pccl_chunk_meta chunks_[10];
 } pccl_op_payload;
 

@@ -68,6 +68,7 @@ DrainKernel drain_for(int dtype, int compute) {
 
 struct Graph {
   char *dev = nullptr;          // device arena; starts with GraphControl
+  unsigned long long *trace = nullptr;  // device trace records, if tracing was switched on
   std::vector<char> image;      // pristine host copy of the arena
   size_t payload_off = 0;       // arena offset of the payload array
   int n_ops = 0;
@@ -226,7 +227,9 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     }
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
   }
-  // global order of the entries: by level, then op id, then part
+  // global order of the entries: by level, then op id, then part.  (A list schedule of the
+  // graph under a cost model, which lets short chains run ahead of long ones, was measured on
+  // the 4096-op schedule and was no faster: workgroups wait longer for dependencies there.)
   std::vector<int> by_level(n_ops);
   for (int i = 0; i < n_ops; ++i) by_level[i] = i;
   std::stable_sort(by_level.begin(), by_level.end(), [&](int a, int b) { return level[a] < level[b]; });
@@ -387,6 +390,42 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   return PCCL_OK;
 }
 
+int pccl_hip_graph_trace(void *graph, int enable) {
+  pccl_host::clear_error();
+  Graph *G = (Graph *)graph;
+  if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_trace: graph is null");
+  std::lock_guard<std::mutex> lock(G->mu);
+  GraphControl *C = (GraphControl *)G->image.data();
+  if (!enable) { C->trace = nullptr; return PCCL_OK; }  // the buffer stays until the graph is destroyed
+  const size_t bytes = sizeof(unsigned long long) * kTraceWords * (size_t)std::max(G->total_tiles, 1);
+  if (!G->trace) {
+    hipError_t e = hipMalloc((void **)&G->trace, bytes);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      G->trace = nullptr;
+      return fail(PCCL_ERR_NOMEM, "hipMalloc(%zu) for the trace records: %s", bytes, hipGetErrorString(e));
+    }
+  }
+  PCCL_HIP_CHECK(hipMemset(G->trace, 0, bytes));
+  C->trace = G->trace;
+  return PCCL_OK;
+}
+
+int pccl_hip_graph_read_trace(void *graph, void *stream, unsigned long long *records, long capacity, long *n_records) {
+  pccl_host::clear_error();
+  Graph *G = (Graph *)graph;
+  if (!G || !n_records) return fail(PCCL_ERR_INVALID_ARG, "graph_read_trace: null argument");
+  *n_records = 0;
+  if (!G->trace) return fail(PCCL_ERR_INVALID_ARG, "graph_read_trace: tracing was never switched on for this graph");
+  if (capacity < 0 || (capacity > 0 && !records)) return fail(PCCL_ERR_INVALID_ARG, "graph_read_trace: bad record buffer");
+  PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  const long n = std::min<long>(capacity, G->total_tiles);
+  if (n > 0)
+    PCCL_HIP_CHECK(hipMemcpy(records, G->trace, sizeof(unsigned long long) * kTraceWords * (size_t)n, hipMemcpyDeviceToHost));
+  *n_records = G->total_tiles;
+  return PCCL_OK;
+}
+
 int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed, unsigned int *total) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
@@ -472,6 +511,10 @@ int pccl_hip_graph_destroy(void *graph) {
   Graph *G = (Graph *)graph;
   if (!G) return PCCL_OK;
   hipError_t e = hipFree(G->dev);
+  if (G->trace) {
+    const hipError_t e2 = hipFree(G->trace);
+    if (e == hipSuccess) e = e2;
+  }
   delete G;
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "hipFree of the op graph: %s", hipGetErrorString(e));
   return PCCL_OK;

@@ -41,6 +41,7 @@ struct GraphControl {
   const int *group_base;                  // per op: first of its kPartGroups words in `groups`, or -1
   HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
   HotWord *ready;                         // per op: dependencies that have arrived in this run
+  unsigned long long *trace;              // null, or 4 words per queue entry (see kTrace*)
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
   int queue_count[kQueues];
@@ -101,7 +102,11 @@ __device__ __forceinline__ void run_part_body(const RcOperands &a, long head, lo
       if (j < a.n_out) body.out[j] = a.out[j] + head * D::kElemBytes;
     // Every access of a part is device-coherent: its inputs may have been written
     // by a workgroup on another XCD moments ago, and its outputs may be read by one.
-    constexpr int kUnroll = NIN >= 3 ? 1 : 2;
+    // Packs a lane has in flight: a part is short (8 packs per lane and stream at the built-in
+    // part size), and every batch of loads costs a full memory latency before its stores can go.
+    // (The variant for unaligned streams assembles each pack from two loads, and a pack of 8-bit
+    // floats unpacks into 16 accumulators: both stay at 1-2 to keep three wavefronts per SIMD.)
+    constexpr int kUnroll = !ALIGNED ? (NIN >= 3 ? 1 : 2) : NIN == 1 ? 4 : D::kElemBytes == 1 ? (NIN >= 3 ? 1 : 2) : NIN == 2 ? 4 : NIN <= 4 ? 2 : 1;
     body_packs<D, Op, NIN, kUnroll, ALIGNED, kMemCoherent, kMemCoherent>(body, n_packs, 0, 1);
   }
   if (threadIdx.x >= kBlock - kWave)
@@ -214,6 +219,15 @@ __device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, long lo,
 
 #define AGENT __HIP_MEMORY_SCOPE_AGENT
 
+// Trace record of a queue entry (entry t of queue q is record t * kQueues + q), times in ticks
+// of the constant 100 MHz clock: who ran what, when the ticket was drawn, when the op's
+// dependencies were met, when the part was complete.
+constexpr int kTraceWords = 4;
+constexpr int kTraceWhat = 0;     // op uid | part << 32 | workgroup << 52
+constexpr int kTraceClaimed = 1;
+constexpr int kTraceReady = 2;
+constexpr int kTraceDone = 3;
+
 // Polls `ready` until it holds.  Gives up (and raises the abort word, so that every
 // workgroup leaves) after spin_limit polls or when another workgroup has given up.
 template <class Ready>
@@ -232,20 +246,35 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 
 // Thread 0, after a part of op `h` is complete: count it; the op's last part re-arms
 // the op's counters for the next run and releases its successors.
+// `draw_ticket` requests the workgroup's next ticket; it is called exactly once, at the point
+// where its round trip costs least: right behind the first counting atomic whose result this
+// function has to wait for (the two then travel together), or, when nothing is counted
+// (single-part op), after the successors have been told, so that their release is not held up
+// behind the ticket (memory operations of a wavefront return in order).
+template <class DrawTicket>
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const PayloadSlot *slot, int uid, int part, int home) {
+                                            const PayloadSlot *slot, int uid, int part, int home,
+                                            DrawTicket draw_ticket) {
   const int parts = slot->parts;
   int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
+  bool drawn = false;
   if (parts > kGroupThreshold) {
     const int group = part % kPartGroups;
     unsigned int *word = &g.groups[g.group_base[uid] + group].value;
-    if (__hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, AGENT) != 1u) return;
+    const unsigned int before = __hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, AGENT);
+    draw_ticket();
+    drawn = true;
+    if (before != 1u) return;
     // this group is done: re-arm it (parts p < parts with p % kPartGroups == group)
     __hip_atomic_store(word, (unsigned int)((parts - group + kPartGroups - 1) / kPartGroups), __ATOMIC_RELAXED, AGENT);
     counted = kPartGroups;
   }
   int old = 1;
-  if (counted > 1) old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
+  if (counted > 1) {
+    old = __hip_atomic_fetch_sub(&h->remaining_executors_, 1, __ATOMIC_RELAXED, AGENT);
+    if (!drawn) draw_ticket();
+    drawn = true;
+  }
   if (old != 1) return;
   if (counted > 1) __hip_atomic_store(&h->remaining_executors_, counted, __ATOMIC_RELAXED, AGENT);
   const unsigned int w12 = slot->payload.initial_word12_;
@@ -263,6 +292,7 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   for (int s = 0; s < n_next; ++s)
     __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
   __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
+  if (!drawn) draw_ticket();
 }
 
 template <int DT, class Op>
@@ -285,6 +315,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   pccl_operation_layout_header *h = nullptr;
   const PayloadSlot *slot = nullptr;
   int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
+  unsigned long long *cur_trace = nullptr;  // its trace record (thread 0 only)
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   // Signal values are offset by (run number << 16).  The run number lives on the device (not
   // in the kernel arguments) so that a launch recorded into a HIP graph uses a fresh one on
@@ -298,22 +329,50 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
       // wavefront waited for its write-through stores before that barrier, so the data is
       // at the point of coherence and relaxed device-scope atomics are enough to hand it
       // over; no L2 write-back / invalidate is involved.
-      if (h) finish_part(g, h, slot, cur_uid, cur_part, home);
+      // The next ticket is requested while the finished part is being counted, so that the
+      // two round trips overlap instead of following each other (see finish_part).
+      int first_q = -1, first_t = 0;
+      unsigned int aborted = 0;
+      auto draw_ticket = [&] {
+        for (int i = 0; i < kQueues && first_q < 0; ++i) {
+          const int q = (home + i) % kQueues;
+          if (!(exhausted & (1u << q)) && g.queue_count[q] > 0) first_q = q;
+        }
+        if (first_q >= 0) first_t = __hip_atomic_fetch_add(g.queue_head[first_q], 1, __ATOMIC_RELAXED, AGENT);
+        aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
+      };
+      if (h) {
+        if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
+        finish_part(g, h, slot, cur_uid, cur_part, home, draw_ticket);
+      } else {
+        draw_ticket();
+      }
       int go = 0;
       unsigned long long e = 0;
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
       // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
       for (;;) {
         go = 0;
-        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0) break;
+        if (aborted) break;
         for (int i = 0; i < kQueues && !go; ++i) {
           const int q = (home + i) % kQueues;
           if (exhausted & (1u << q)) continue;
           const int n = g.queue_count[q];
-          const int t = n > 0 ? __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT) : n;
+          int t = n;
+          if (q == first_q) {  // the ticket requested above
+            t = first_t;
+            first_q = -1;
+          } else if (n > 0) {
+            t = __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT);
+          }
           if (t < n) {
             e = g.queue_entries[q][t];
             go = 1;
+            if (g.trace) {
+              cur_trace = g.trace + ((size_t)t * kQueues + q) * kTraceWords;
+              cur_trace[kTraceWhat] = e | ((unsigned long long)blockIdx.x << 52);
+              cur_trace[kTraceClaimed] = wall_clock64();
+            }
             if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
           } else {
             exhausted |= 1u << q;
@@ -324,16 +383,20 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         pccl_operation_layout_header *hc = &g.headers[uid];
         const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
         // wait until every dependency of the op has arrived (none: nothing ever writes the
-        // word); pre_dependencies_ in the header is the count to reach and stays constant
-        const unsigned int n_pred = __hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT) & 0xffu;
-        if (n_pred != 0 &&
+        // word); pre_dependencies_ in the header is the count to reach and stays constant.
+        // The count, the first look at the arrivals and the primitive go out together.
+        const unsigned int w12 = __hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT);
+        const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
+        const int prim = sc->payload.primitive_;
+        const unsigned int n_pred = w12 & 0xffu;
+        if (n_pred != 0 && arrived != n_pred &&
             !bounded_wait(abort_flag, spin_limit, [&] {
               return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == n_pred;
             })) {
           go = 0;
           break;
         }
-        const int prim = sc->payload.primitive_;
+        if (cur_trace) cur_trace[kTraceReady] = wall_clock64();
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
         if (!have_signal_base) {
@@ -350,7 +413,9 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           go = 0;
           break;
         }
-        finish_part(g, hc, sc, uid, 0, home);
+        if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
+        finish_part(g, hc, sc, uid, 0, home, [] {});
+        aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
       s_go = go;

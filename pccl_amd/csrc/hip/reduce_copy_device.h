@@ -410,7 +410,9 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
         for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
           if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + chunk, off, r);
       }
-    } else {  // last, partial chunk: same shape, every pack guarded
+    } else if constexpr (D::kElemBytes == 1 && NIN > 1) {
+      // last, partial chunk, 8-bit floats: pack by pack (the batched form below costs them a
+      // wavefront per SIMD in registers)
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const unsigned int off = (threadIdx.x + (unsigned)u * kBlock) * 16u;
@@ -423,6 +425,27 @@ __device__ __forceinline__ void body_packs(const RcOperands &a, long n_packs, lo
 #pragma unroll
           for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
             if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + chunk, off, r);
+        }
+      }
+    } else {  // last, partial chunk: same shape; a lane without a pack u re-reads the chunk's
+      // last pack (so that all loads still go out together) and stores nothing for it
+      const unsigned int last = (unsigned int)(n_packs - base - 1);
+      u32x4 v[UNROLL][NIN];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const unsigned int p = threadIdx.x + (unsigned)u * kBlock;
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) v[u][k] = load_pack<D, ALIGNED, LD>(a.in[k] + chunk, (p < last ? p : last) * 16u);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const unsigned int p = threadIdx.x + (unsigned)u * kBlock;
+        if (p <= last) {
+          const u32x4 r = fold_pack<D, Op, NIN>(v[u]);
+          store_pack<D, true, ST>(a.out[0] + chunk, p * 16u, r);
+#pragma unroll
+          for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
+            if (j < a.n_out) store_pack<D, ALIGNED, ST>(a.out[j] + chunk, p * 16u, r);
         }
       }
     }

@@ -78,6 +78,8 @@ def lib():
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.pccl_hip_graph_trace.argtypes = [vp, ci]
+        L.pccl_hip_graph_read_trace.argtypes = [vp, vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_next_signal_base.argtypes = [vp, ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_set_spin_limit.argtypes = [vp, ctypes.c_uint]
         L.pccl_hip_graph_destroy.argtypes = [vp]
@@ -226,6 +228,23 @@ class Graph:
         lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)
         _check(lib().pccl_hip_graph_info(self._h, ctypes.byref(lay), ctypes.byref(nt), ctypes.byref(nw)))
         return {"device_layout": lay.value, "n_tiles": nt.value, "n_workgroups": nw.value}
+
+    def trace(self, enable=True):
+        """Switches the per-entry timeline on or off for the following runs."""
+        _check(lib().pccl_hip_graph_trace(self._h, 1 if enable else 0))
+
+    def read_trace(self, stream=None):
+        """Timeline of the last run: uint64 array (entries, 4) in queue order; columns: what
+        (op_uid | part << 32 | workgroup << 52), ticket drawn, dependencies met, part complete,
+        in ticks of the device's 100 MHz clock."""
+        import numpy as np
+        n = ctypes.c_long(0)
+        _check(lib().pccl_hip_graph_read_trace(self._h, ctypes.c_void_p(_addr(stream)), None, 0, ctypes.byref(n)))
+        out = np.zeros((n.value, 4), dtype=np.uint64)
+        if n.value:
+            _check(lib().pccl_hip_graph_read_trace(self._h, ctypes.c_void_p(_addr(stream)), out.ctypes.data_as(ctypes.c_void_p),
+                                                   n.value, ctypes.byref(n)))
+        return out
 
     def destroy(self):
         if self._h:

@@ -417,3 +417,44 @@ def test_mixed_dtypes_and_computes_in_one_graph(hip, oracle):
     assert np.isinf(oracle.widen("f16", checks[2][3])).any() and np.isinf(oracle.widen("f16", checks[8][3])).any()
     assert (checks[3][3] & 0x7f == 0x7e).any() and (checks[7][3] & 0x7f == 0x7b).any()
     g.destroy()
+
+
+# ---- per-entry timeline -------------------------------------------------------------------
+
+def test_trace_records_every_entry_once_and_in_dependency_order(hip, oracle):
+    """The timeline of a run names every (op, part) exactly once, its three times are ordered,
+    and no part of an op starts before the last part of each of its dependencies is done."""
+    import torch
+    count = 100000  # 200 KB of bf16: several parts per op
+    a, b, c = (H.gen("bf16", count, 91, k) for k in range(3))
+    da, db, dc = (H.DevBuf(torch, "bf16", count, 0, src=x) for x in (a, b, c))
+    dt, du, dv = (H.DevBuf(torch, "bf16", count, 0) for _ in range(3))
+    ops = [dict(dtype="bf16", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+           dict(dtype="bf16", compute="max", ins=[db.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[]),
+           dict(dtype="bf16", compute="sum", ins=[dt.ptr, du.ptr], outs=[dv.ptr], count=count, deps=[0, 1])]
+    g = hip.Graph(ops)
+    with pytest.raises(hip.PcclError):
+        g.read_trace(_stream(torch))  # never switched on
+    g.trace(True)
+    for _ in range(2):  # each run overwrites the last
+        _run_and_check(torch, hip, g, 3)
+    tr = g.read_trace(_stream(torch))
+    info = g.info()
+    assert tr.shape == (info["n_tiles"], 4)
+    uid = (tr[:, 0] & np.uint64(0xffffffff)).astype(np.int64)
+    part = ((tr[:, 0] >> np.uint64(32)) & np.uint64(0xfffff)).astype(np.int64)
+    wg = (tr[:, 0] >> np.uint64(52)).astype(np.int64)
+    assert wg.min() >= 0 and wg.max() < info["n_workgroups"]
+    for u in range(3):
+        assert sorted(part[uid == u].tolist()) == list(range(int((uid == u).sum()))) and (uid == u).sum() > 1
+    claimed, ready, done = (tr[:, k].astype(np.int64) for k in (1, 2, 3))
+    assert (claimed > 0).all() and (claimed <= ready).all() and (ready <= done).all()
+    assert ready[uid == 2].min() >= max(done[uid == 0].max(), done[uid == 1].max())
+    assert done.max() - claimed.min() < 100 * 1000 * 100  # under 100 ms of the 100 MHz clock
+    want = oracle.reduce("bf16", "sum", [oracle.reduce("bf16", "sum", [a, b]), oracle.reduce("bf16", "max", [b, c])])
+    H.assert_bits_equal(dv.download(), want, "traced run")
+    # switched off: runs still work and leave the records alone
+    g.trace(False)
+    _run_and_check(torch, hip, g, 3)
+    assert np.array_equal(g.read_trace(_stream(torch)), tr)
+    g.destroy()
