@@ -86,11 +86,24 @@ typedef struct pccl_op_payload {
   unsigned char compute_;   /* enum pccl_compute   */
   unsigned char n_in_;
   unsigned char n_out_;
-  unsigned int initial_word12_; /* copy of the header's word at offset 12 (pre_dependencies_ .. num_next_ops_) */
+  unsigned char pre_dependencies_; /* copy of the header's field */
+  unsigned char part_preds_;       /* of those, dependencies that are met part by part (see below) */
+  unsigned char part_nexts_;       /* successors that this op releases part by part; they come
+                                      first in next_op_uids_head_ */
+  unsigned char num_next_ops_;     /* copy of the header's field */
   pccl_chunk_meta chunks_[10];
 } pccl_op_payload;
 
 #define PCCL_MAX_OP_CHUNKS 10
+
+/* Part-by-part dependencies.  When op B depends on op A, both are cut into the same number of
+ * parts over the same number of bytes, and every operand of A that B's operands overlap
+ * (with a write on either side) starts at the same address as the operand of B it overlaps,
+ * then part p of B needs only part p of A, not all of A; the executor then lets B's part p
+ * start as soon as A's part p is complete (and all of B's other dependencies are), which is
+ * what lets a chain of large ops stream instead of draining between ops.  The same must hold
+ * for every op still possibly in flight behind A through such edges; otherwise the
+ * dependency stays whole-op.  The observable result is that of whole-op dependencies. */
 
 /* Ready-queue entry: which op, which of its required_executors_ parts. */
 typedef struct pccl_queue_entry {

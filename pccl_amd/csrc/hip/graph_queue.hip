@@ -66,9 +66,15 @@ DrainKernel drain_for(int dtype, int compute) {
 
 // ---- host side ----------------------------------------------------------------
 
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+int elem_bytes(int dtype) { return pccl_host::pccl_dtype_bytes(dtype); }
+
 struct Graph {
   char *dev = nullptr;          // device arena; starts with GraphControl
   unsigned long long *trace = nullptr;  // device trace records, if tracing was switched on
+  bool trace_on = false;
+  unsigned int spin_limit = kDefaultSpinLimit;
   std::vector<char> image;      // pristine host copy of the arena
   size_t payload_off = 0;       // arena offset of the payload array
   int n_ops = 0;
@@ -78,22 +84,93 @@ struct Graph {
   unsigned int runs = 0;        // launches so far; run r uses signal values (r << 16) + value
   DrainKernel kernel = nullptr;
   std::mutex mu;
+  // what the arena was built from (graph_rebind may have to build it again)
+  std::vector<pccl_op_desc> descs;   // deps point into deps_store
+  std::vector<int> deps_store;
+  long tile_bytes = 0;               // as passed to graph_create
+  std::vector<int> parts;            // per op
+  std::vector<int> topo;             // a topological order of the ops
+  std::vector<unsigned char> part_edge;  // per dependency, in descs order: met part by part
 };
 
-size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+// ---- which dependencies can be met part by part -------------------------------
+// B depends on A.  Part p of B needs only part p of A when both ops are cut alike (same
+// number of parts, same bytes per part and in all) and every pair of operands through which
+// they conflict (A writes what B reads or writes, or A reads what B writes) starts at the
+// same address: then part p of either op touches the same bytes of that pair.  A pair that
+// overlaps at different addresses makes some other part of A matter, and no conflicting pair
+// at all means that the dependency orders something this code cannot see; both keep the
+// dependency whole-op.
+enum Conflict { kNoConflict, kSameAddress, kOtherAddress };
 
-int elem_bytes(int dtype) { return pccl_host::pccl_dtype_bytes(dtype); }
+Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t bytes) {
+  bool any = false, other = false;
+  auto pair = [&](const void *x, const void *y) {
+    const uintptr_t p = (uintptr_t)x, q = (uintptr_t)y;
+    if (p < q + bytes && q < p + bytes) {
+      any = true;
+      if (p != q) other = true;
+    }
+  };
+  for (int j = 0; j < a.n_out; ++j) {
+    for (int k = 0; k < b.n_in; ++k) pair(a.outs[j], b.ins[k]);
+    for (int k = 0; k < b.n_out; ++k) pair(a.outs[j], b.outs[k]);
+  }
+  for (int j = 0; j < a.n_in; ++j)
+    for (int k = 0; k < b.n_out; ++k) pair(a.ins[j], b.outs[k]);
+  return other ? kOtherAddress : any ? kSameAddress : kNoConflict;
+}
 
-}  // namespace
+// Flags per dependency (ops in index order, dependencies in list order).  behind[b] lists the
+// ops that may still be running when a part of b starts: its part-by-part predecessors and
+// theirs.  Whole-op semantics promise b that ALL its ancestors are complete, so b must not
+// conflict with any op of behind[b] at differing addresses either; when it would, or when the
+// list grows long, the dependency stays whole-op (which also empties what lies behind it).
+std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
+                                                 const std::vector<int> &topo) {
+  constexpr size_t kMaxBehind = 32;
+  const int n_ops = (int)ops.size();
+  std::vector<size_t> dep_start(n_ops + 1, 0);
+  for (int i = 0; i < n_ops; ++i) dep_start[i + 1] = dep_start[i] + (size_t)ops[i].n_deps;
+  std::vector<unsigned char> flags(dep_start[n_ops], 0);
+  if (const char *env = getenv("PCCL_HIP_PART_DEPS"))
+    if (env[0] == '0') return flags;  // every dependency whole-op
+  std::vector<std::vector<int>> behind(n_ops);
+  auto is_data = [&](const pccl_op_desc &o) { return o.primitive != PCCL_NOTIFY && o.primitive != PCCL_GET_NOTIFIED; };
+  auto bytes_of = [&](const pccl_op_desc &o) { return (uintptr_t)o.count * (uintptr_t)elem_bytes(o.dtype); };
+  for (int b : topo) {
+    const pccl_op_desc &B = ops[b];
+    if (!is_data(B) || parts[b] < 2) continue;
+    const uintptr_t bytes = bytes_of(B);
+    const uintptr_t per = (uintptr_t)part_elems(B.count, parts[b]) * (uintptr_t)elem_bytes(B.dtype);
+    for (int d = 0; d < B.n_deps; ++d) {
+      const int a = B.deps[d];
+      const pccl_op_desc &A = ops[a];
+      if (!is_data(A) || parts[a] != parts[b] || bytes_of(A) != bytes ||
+          (uintptr_t)part_elems(A.count, parts[a]) * (uintptr_t)elem_bytes(A.dtype) != per)
+        continue;
+      if (conflict_of(A, B, bytes) != kSameAddress) continue;
+      bool ok = behind[a].size() + behind[b].size() + 1 <= kMaxBehind;
+      for (size_t k = 0; ok && k < behind[a].size(); ++k)
+        ok = conflict_of(ops[behind[a][k]], B, bytes) != kOtherAddress;
+      if (!ok) continue;
+      flags[dep_start[b] + d] = 1;
+      auto add = [&](int x) {
+        if (std::find(behind[b].begin(), behind[b].end(), x) == behind[b].end()) behind[b].push_back(x);
+      };
+      add(a);
+      for (int x : behind[a]) add(x);
+    }
+  }
+  return flags;
+}
 
-extern "C" {
-
-int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph) {
-  pccl_host::clear_error();
-  if (!graph) return fail(PCCL_ERR_INVALID_ARG, "graph_create: graph is null");
-  *graph = nullptr;
-  if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_create: bad op array");
-  if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
+// Validates G->descs and builds the device arena and its host image from them.  On failure
+// nothing is left allocated.  `run_number`: what the device's run word starts at.
+int build_graph(Graph *G, unsigned int run_number) {
+  const pccl_op_desc *ops = G->descs.data();
+  const int n_ops = (int)G->descs.size();
+  long tile_bytes = G->tile_bytes;
   // With the built-in part size the parts of a large op grow with it instead of multiplying
   // (see the part count below).
   const bool default_tile = tile_bytes == 0;
@@ -209,6 +286,8 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   std::vector<int> level(n_ops, 0);
   {
     std::vector<int> indeg(n_ops), stack;
+    G->topo.clear();
+    G->topo.reserve(n_ops);
     for (int i = 0; i < n_ops; ++i) {
       indeg[i] = n_pred[i] + order_pred[i];
       if (!indeg[i]) stack.push_back(i);
@@ -221,6 +300,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     while (!stack.empty()) {
       const int u = stack.back();
       stack.pop_back();
+      G->topo.push_back(u);
       ++seen;
       for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) relax(u, succ[e]);
       for (int v : order_succ[u]) relax(u, v);
@@ -234,33 +314,73 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   for (int i = 0; i < n_ops; ++i) by_level[i] = i;
   std::stable_sort(by_level.begin(), by_level.end(), [&](int a, int b) { return level[a] < level[b]; });
 
+  // first entry of each op in that order
+  std::vector<int> first_entry(n_ops, 0);
+  {
+    long long t = 0;
+    for (int idx = 0; idx < n_ops; ++idx) {
+      first_entry[by_level[idx]] = (int)t;
+      t += parts[by_level[idx]];
+    }
+  }
+
+  // ---- dependencies met part by part ---------------------------------------
+  // Successor lists again, this time with the successors that are released part by part
+  // first, and beside each of those the entry index of its part 0.
+  G->parts = parts;
+  G->part_edge = classify_dependencies(G->descs, parts, G->topo);
+  std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
+  bool any_part_edge = false;
+  {
+    size_t at = 0;
+    for (int i = 0; i < n_ops; ++i)
+      for (int d = 0; d < ops[i].n_deps; ++d, ++at)
+        if (G->part_edge[at]) {
+          ++n_part_next[ops[i].deps[d]];
+          ++n_part_pred[i];
+          any_part_edge = true;
+        }
+    std::vector<int> fill_part(n_ops, 0), fill_whole(n_ops, 0);
+    at = 0;
+    for (int i = 0; i < n_ops; ++i)
+      for (int d = 0; d < ops[i].n_deps; ++d, ++at) {
+        const int u = ops[i].deps[d];
+        const int pos = succ_start[u] + (G->part_edge[at] ? fill_part[u]++ : n_part_next[u] + fill_whole[u]++);
+        succ[pos] = i;
+        succ_part_base[pos] = G->part_edge[at] ? first_entry[i] : -1;
+      }
+  }
+
   // ---- arena layout ----------------------------------------------------------
   size_t off = align_up(sizeof(GraphControl), 256);
   const size_t off_opptr = off;   off = align_up(off + sizeof(void *) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_hdr = off;     off = align_up(off + sizeof(pccl_operation_layout_header) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_payload = off; off = align_up(off + kPayloadStride * (size_t)std::max(n_ops, 1), 256);
   const size_t off_succ = off;    off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
+  const size_t off_succ_part = off; off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_hot = off;     off = align_up(off + sizeof(HotWord) * kHotWords, 256);
   int n_grouped = 0;  // ops that count their parts in groups
   for (int i = 0; i < n_ops; ++i) n_grouped += parts[i] > kGroupThreshold;
   const size_t off_ready = off;   off = align_up(off + sizeof(HotWord) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_gbase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_groups = off;  off = align_up(off + sizeof(HotWord) * (size_t)kPartGroups * (size_t)std::max(n_grouped, 1), 256);
+  const size_t off_part_arrivals = off;
+  if (any_part_edge) off = align_up(off + sizeof(unsigned int) * (size_t)(tiles + kQueues), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
   const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
   const size_t arena_bytes = off;
 
-  Graph *G = new Graph();
   G->n_ops = n_ops;
   G->total_tiles = (int)tiles;
   G->payload_off = off_payload;
   G->kernel = kernel;
-  if (hipGetDevice(&G->device) != hipSuccess) { delete G; return fail(PCCL_ERR_NO_DEVICE, "no current device"); }
+  if (hipGetDevice(&G->device) != hipSuccess) return fail(PCCL_ERR_NO_DEVICE, "no current device");
+  G->dev = nullptr;
   hipError_t e = hipMalloc((void **)&G->dev, arena_bytes);
   if (e != hipSuccess) {
     (void)hipGetLastError();
-    delete G;
+    G->dev = nullptr;
     return fail(PCCL_ERR_NOMEM, "hipMalloc(%zu) for the op graph: %s", arena_bytes, hipGetErrorString(e));
   }
   G->image.assign(arena_bytes, 0);
@@ -279,6 +399,9 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   C->headers = (pccl_operation_layout_header *)(dev + off_hdr);
   C->slots = dev + off_payload;
   C->succ = (const int *)(dev + off_succ);
+  C->succ_part_base = (const int *)(dev + off_succ_part);
+  C->part_arrivals = any_part_edge ? (unsigned int *)(dev + off_part_arrivals) : nullptr;
+  C->trace = G->trace_on ? G->trace : nullptr;
   C->group_base = (const int *)(dev + off_gbase);
   C->groups = (HotWord *)(dev + off_groups);
   C->ready = (HotWord *)(dev + off_ready);
@@ -294,11 +417,11 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
       next += kPartGroups;
     }
   }
-  C->spin_limit = kDefaultSpinLimit;
+  C->spin_limit = G->spin_limit;
   C->total_tiles = (int)tiles;
   hot[kHotCompleted].value = 0;
   hot[kHotTotal].value = (unsigned int)n_ops;
-  hot[kHotRun].value = 1;
+  hot[kHotRun].value = run_number;
 
   // deal the entries round-robin onto the queues, in global order
   std::vector<std::vector<unsigned long long>> qe(kQueues);
@@ -354,20 +477,57 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     pl->compute_ = o.compute;
     pl->n_in_ = o.n_in;
     pl->n_out_ = o.n_out;
-    memcpy(&pl->initial_word12_, (char *)h + 12, 4);
+    pl->pre_dependencies_ = h->pre_dependencies_;
+    pl->part_preds_ = (unsigned char)n_part_pred[i];
+    pl->part_nexts_ = (unsigned char)n_part_next[i];
+    pl->num_next_ops_ = h->num_next_ops_;
     // signal ops: the only operand is the signal word, num_elems_ carries the value
     for (int k = 0; k < o.n_in; ++k) pl->chunks_[k] = pccl_chunk_meta{o.dtype, (void *)o.ins[k], o.count};
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
   }
   if (n_edges) memcpy(img + off_succ, succ.data(), sizeof(int) * n_edges);
+  if (n_edges) memcpy(img + off_succ_part, succ_part_base.data(), sizeof(int) * n_edges);
   // never more workgroups than entries
   G->n_wg = (int)std::max<long long>(1, std::min<long long>(tiles, cap));
 
   e = hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     (void)hipFree(dev);
-    delete G;
+    G->dev = nullptr;
     return fail(PCCL_ERR_HIP, "uploading the op graph: %s", hipGetErrorString(e));
+  }
+  return PCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph) {
+  pccl_host::clear_error();
+  if (!graph) return fail(PCCL_ERR_INVALID_ARG, "graph_create: graph is null");
+  *graph = nullptr;
+  if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_create: bad op array");
+  if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
+  // own copy of the ops and their dependency lists
+  Graph *G = new Graph();
+  G->tile_bytes = tile_bytes;
+  G->descs.assign(ops, ops + n_ops);
+  size_t n_deps = 0;
+  for (int i = 0; i < n_ops; ++i) {
+    if (ops[i].n_deps < 0 || (ops[i].n_deps > 0 && !ops[i].deps)) {
+      delete G;
+      return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
+    }
+    n_deps += (size_t)ops[i].n_deps;
+  }
+  G->deps_store.reserve(n_deps);
+  for (int i = 0; i < n_ops; ++i) G->deps_store.insert(G->deps_store.end(), ops[i].deps, ops[i].deps + ops[i].n_deps);
+  for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) G->descs[i].deps = G->deps_store.data() + at;
+  const int rc = build_graph(G, 1);
+  if (rc != PCCL_OK) {
+    delete G;
+    return rc;
   }
   *graph = G;
   return PCCL_OK;
@@ -396,6 +556,7 @@ int pccl_hip_graph_trace(void *graph, int enable) {
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_trace: graph is null");
   std::lock_guard<std::mutex> lock(G->mu);
   GraphControl *C = (GraphControl *)G->image.data();
+  G->trace_on = enable != 0;
   if (!enable) { C->trace = nullptr; return PCCL_OK; }  // the buffer stays until the graph is destroyed
   const size_t bytes = sizeof(unsigned long long) * kTraceWords * (size_t)std::max(G->total_tiles, 1);
   if (!G->trace) {
@@ -460,14 +621,33 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   if (G->n_ops == 0 || nbytes == 0 || old_base == new_base) return PCCL_OK;
   std::lock_guard<std::mutex> lock(G->mu);
   const uintptr_t lo = (uintptr_t)old_base, hi = lo + (uintptr_t)nbytes;
+  auto moved = [&](const void *p) {
+    const uintptr_t a = (uintptr_t)p;
+    return a >= lo && a < hi ? (void *)((uintptr_t)new_base + (a - lo)) : (void *)p;
+  };
+  for (pccl_op_desc &o : G->descs) {
+    for (int k = 0; k < o.n_in; ++k) o.ins[k] = moved(o.ins[k]);
+    for (int k = 0; k < o.n_out; ++k) o.outs[k] = moved(o.outs[k]);
+  }
+  // Which dependencies may be met part by part depends on which operands share addresses
+  // (an output tensor that now is the input tensor, say).  If that changed, the arena is
+  // built again from the moved ops; earlier runs on `stream` finish first.
+  if (classify_dependencies(G->descs, G->parts, G->topo) != G->part_edge) {
+    PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    char *old_dev = G->dev;
+    const int rc = build_graph(G, G->runs + 1u);
+    if (rc != PCCL_OK) {
+      G->dev = old_dev;  // the old arena still describes the old addresses: the graph is unusable
+      return rc;
+    }
+    PCCL_HIP_CHECK(hipFree(old_dev));
+    return PCCL_OK;
+  }
   char *payloads = G->image.data() + G->payload_off;
   for (int i = 0; i < G->n_ops; ++i) {
     pccl_op_payload *pl = (pccl_op_payload *)(payloads + kPayloadStride * (size_t)i);
     const int nc = pl->n_in_ + pl->n_out_;
-    for (int k = 0; k < nc; ++k) {
-      const uintptr_t a = (uintptr_t)pl->chunks_[k].addr_;
-      if (a >= lo && a < hi) pl->chunks_[k].addr_ = (void *)((uintptr_t)new_base + (a - lo));
-    }
+    for (int k = 0; k < nc; ++k) pl->chunks_[k].addr_ = moved(pl->chunks_[k].addr_);
   }
   // ordered after earlier runs on `stream`; the source is pageable host memory,
   // so the call returns once the bytes are staged
@@ -501,6 +681,7 @@ int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls) {
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_set_spin_limit: graph is null");
   if (polls < 64) polls = 64;
   std::lock_guard<std::mutex> lock(G->mu);
+  G->spin_limit = polls;
   ((GraphControl *)G->image.data())->spin_limit = polls;
   PCCL_HIP_CHECK(hipMemcpy(G->dev + offsetof(GraphControl, spin_limit), &polls, sizeof(polls), hipMemcpyHostToDevice));
   return PCCL_OK;

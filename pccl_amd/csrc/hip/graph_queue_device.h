@@ -42,6 +42,8 @@ struct GraphControl {
   HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
   HotWord *ready;                         // per op: dependencies that have arrived in this run
   unsigned long long *trace;              // null, or 4 words per queue entry (see kTrace*)
+  unsigned int *part_arrivals;            // per queue entry (t * kQueues + q): part-by-part dependencies that have arrived
+  const int *succ_part_base;              // beside succ: entry index of part 0 of a successor released part by part
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
   int queue_count[kQueues];
@@ -77,6 +79,26 @@ struct PayloadSlot {
   int succ_start;           // successors at GraphControl::succ + succ_start
 };
 static_assert(sizeof(PayloadSlot) == kPayloadStride, "payload slot stride");
+
+// What the bookkeeping of a finished part needs from the op's slot.  The workgroup reads it
+// together with the payload when the part starts (uniform loads), so that no load stands
+// between the end of the part and the atomics that hand it over.
+struct OpFacts {
+  int parts;
+  int succ_start;
+  unsigned int counts;  // payload bytes 4..7: pre_dependencies_, part_preds_, part_nexts_, num_next_ops_
+  __device__ __forceinline__ static OpFacts of(const PayloadSlot *slot) {
+    OpFacts f;
+    f.parts = slot->parts;
+    f.succ_start = slot->succ_start;
+    f.counts = *(const unsigned int *)&slot->payload.pre_dependencies_;
+    return f;
+  }
+  __device__ __forceinline__ int pre_dependencies() const { return (int)(counts & 0xffu); }
+  __device__ __forceinline__ int part_preds() const { return (int)((counts >> 8) & 0xffu); }
+  __device__ __forceinline__ int part_nexts() const { return (int)((counts >> 16) & 0xffu); }
+  __device__ __forceinline__ int num_next_ops() const { return (int)(counts >> 24); }
+};
 
 __device__ __forceinline__ unsigned int *word12(pccl_operation_layout_header *h) {
   return (unsigned int *)((char *)h + 12);
@@ -253,9 +275,17 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // behind the ticket (memory operations of a wavefront return in order).
 template <class DrawTicket>
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const PayloadSlot *slot, int uid, int part, int home,
+                                            const OpFacts &op, int uid, int part, int home,
                                             DrawTicket draw_ticket) {
-  const int parts = slot->parts;
+  const int parts = op.parts;
+  // successors that need only this part of the op (they come first in the successor list):
+  // part `part` of each is told right away
+  const int n_part_next = op.part_nexts();
+  if (n_part_next) {
+    const int *first_entry = g.succ_part_base + op.succ_start;
+    for (int s = 0; s < n_part_next; ++s)
+      __hip_atomic_fetch_add(&g.part_arrivals[first_entry[s] + part], 1u, __ATOMIC_RELAXED, AGENT);
+  }
   int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
   bool drawn = false;
   if (parts > kGroupThreshold) {
@@ -277,7 +307,6 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   }
   if (old != 1) return;
   if (counted > 1) __hip_atomic_store(&h->remaining_executors_, counted, __ATOMIC_RELAXED, AGENT);
-  const unsigned int w12 = slot->payload.initial_word12_;
   // The op is complete.  Its own arrivals word goes back to zero for the next run (every
   // dependency of this op has arrived, or it could not have run), and it arrives at each
   // successor: one add on the successor's arrivals word, whose result nobody waits for.  The
@@ -286,10 +315,11 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   // and neighbouring ops need (with 1024 pollers on a header line a hand-over between two
   // 32 MiB ops took 6 us longer), and without an atomic whose result decides who announces
   // (that round trip was a third of the latency between two dependent ops).
-  if (w12 & 0xffu) __hip_atomic_store(&g.ready[uid].value, 0u, __ATOMIC_RELAXED, AGENT);
-  const int n_next = (int)(w12 >> 24);
-  const int *next = g.succ + slot->succ_start;
-  for (int s = 0; s < n_next; ++s)
+  if (op.pre_dependencies() > op.part_preds())
+    __hip_atomic_store(&g.ready[uid].value, 0u, __ATOMIC_RELAXED, AGENT);
+  const int n_next = op.num_next_ops();
+  const int *next = g.succ + op.succ_start;
+  for (int s = n_part_next; s < n_next; ++s)
     __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
   __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
   if (!drawn) draw_ticket();
@@ -315,6 +345,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   pccl_operation_layout_header *h = nullptr;
   const PayloadSlot *slot = nullptr;
   int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
+  OpFacts cur_op = {1, 0, 0};     // ... and its op's facts (uniform)
   unsigned long long *cur_trace = nullptr;  // its trace record (thread 0 only)
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   // Signal values are offset by (run number << 16).  The run number lives on the device (not
@@ -343,12 +374,13 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
       };
       if (h) {
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, h, slot, cur_uid, cur_part, home, draw_ticket);
+        finish_part(g, h, cur_op, cur_uid, cur_part, home, draw_ticket);
       } else {
         draw_ticket();
       }
       int go = 0;
       unsigned long long e = 0;
+      size_t entry_index = 0;  // of e in the global order
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
       // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
       for (;;) {
@@ -367,9 +399,10 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           }
           if (t < n) {
             e = g.queue_entries[q][t];
+            entry_index = (size_t)t * kQueues + q;
             go = 1;
             if (g.trace) {
-              cur_trace = g.trace + ((size_t)t * kQueues + q) * kTraceWords;
+              cur_trace = g.trace + entry_index * kTraceWords;
               cur_trace[kTraceWhat] = e | ((unsigned long long)blockIdx.x << 52);
               cur_trace[kTraceClaimed] = wall_clock64();
             }
@@ -385,16 +418,31 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         // wait until every dependency of the op has arrived (none: nothing ever writes the
         // word); pre_dependencies_ in the header is the count to reach and stays constant.
         // The count, the first look at the arrivals and the primitive go out together.
+        // Dependencies met part by part arrive on the entry's own word instead; the entry is
+        // that word's only reader and clears it for the next run.
         const unsigned int w12 = __hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
+        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + entry_index : nullptr;
+        const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
-        const unsigned int n_pred = w12 & 0xffu;
+        const unsigned int part_preds = sc->payload.part_preds_;
+        const unsigned int n_pred = (w12 & 0xffu) - part_preds;  // whole-op dependencies
         if (n_pred != 0 && arrived != n_pred &&
             !bounded_wait(abort_flag, spin_limit, [&] {
               return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == n_pred;
             })) {
           go = 0;
           break;
+        }
+        if (part_preds != 0) {
+          if (part_arrived != part_preds &&
+              !bounded_wait(abort_flag, spin_limit, [&] {
+                return __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) == part_preds;
+              })) {
+            go = 0;
+            break;
+          }
+          __hip_atomic_store(part_word, 0u, __ATOMIC_RELAXED, AGENT);
         }
         if (cur_trace) cur_trace[kTraceReady] = wall_clock64();
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
@@ -414,7 +462,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, hc, sc, uid, 0, home, [] {});
+        finish_part(g, hc, OpFacts::of(sc), uid, 0, home, [] {});
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
@@ -429,8 +477,9 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
     h = &g.headers[uid];
     slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
     const pccl_op_payload *pl = &slot->payload;
+    cur_op = OpFacts::of(slot);
     const long count = pl->chunks_[0].num_elems_;
-    const long per = part_elems(count, slot->parts);
+    const long per = part_elems(count, cur_op.parts);
     const long lo = (long)part * per;
     long n = count - lo;
     if (n > per) n = per;

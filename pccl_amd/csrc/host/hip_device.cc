@@ -59,6 +59,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_LDS_BYTES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_UNROLL");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_TILE_BYTES");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_PART_DEPS");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;

@@ -423,7 +423,7 @@ def test_mixed_dtypes_and_computes_in_one_graph(hip, oracle):
 
 def test_trace_records_every_entry_once_and_in_dependency_order(hip, oracle):
     """The timeline of a run names every (op, part) exactly once, its three times are ordered,
-    and no part of an op starts before the last part of each of its dependencies is done."""
+    and no part of an op starts before the parts it needs of its dependencies are done."""
     import torch
     count = 100000  # 200 KB of bf16: several parts per op
     a, b, c = (H.gen("bf16", count, 91, k) for k in range(3))
@@ -449,7 +449,11 @@ def test_trace_records_every_entry_once_and_in_dependency_order(hip, oracle):
         assert sorted(part[uid == u].tolist()) == list(range(int((uid == u).sum()))) and (uid == u).sum() > 1
     claimed, ready, done = (tr[:, k].astype(np.int64) for k in (1, 2, 3))
     assert (claimed > 0).all() and (claimed <= ready).all() and (ready <= done).all()
-    assert ready[uid == 2].min() >= max(done[uid == 0].max(), done[uid == 1].max())
+    # op 2 reads what ops 0 and 1 wrote, at the same addresses and cut alike: its part p needs
+    # their parts p (not the whole ops)
+    for p in range(int((uid == 2).sum())):
+        mine = ready[(uid == 2) & (part == p)][0]
+        assert mine >= done[(uid == 0) & (part == p)][0] and mine >= done[(uid == 1) & (part == p)][0]
     assert done.max() - claimed.min() < 100 * 1000 * 100  # under 100 ms of the 100 MHz clock
     want = oracle.reduce("bf16", "sum", [oracle.reduce("bf16", "sum", [a, b]), oracle.reduce("bf16", "max", [b, c])])
     H.assert_bits_equal(dv.download(), want, "traced run")
@@ -457,4 +461,142 @@ def test_trace_records_every_entry_once_and_in_dependency_order(hip, oracle):
     g.trace(False)
     _run_and_check(torch, hip, g, 3)
     assert np.array_equal(g.read_trace(_stream(torch)), tr)
+    g.destroy()
+
+
+# ---- dependencies met part by part ---------------------------------------------------------
+
+def _timeline(torch, g):
+    tr = g.read_trace(_stream(torch))
+    uid = (tr[:, 0] & np.uint64(0xffffffff)).astype(np.int64)
+    part = ((tr[:, 0] >> np.uint64(32)) & np.uint64(0xfffff)).astype(np.int64)
+    return uid, part, tr[:, 2].astype(np.int64), tr[:, 3].astype(np.int64)
+
+
+def test_chain_of_large_in_place_ops_streams_part_by_part(hip, oracle):
+    """t = a + b; t = t * c (in place); u = max(t, a); t = u + t: every op has many parts and
+    reads or overwrites its predecessor's output at the same addresses, so part p follows
+    part p.  Bits must equal the ops executed one after the other."""
+    import torch
+    count = 3 * 1000 * 1000 + 17
+    a, b, c = (H.gen("f32", count, 97, k) for k in range(3))
+    da, db, dc = (H.DevBuf(torch, "f32", count, 0, src=x) for x in (a, b, c))
+    dt, du = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+           dict(dtype="f32", compute="prod", ins=[dt.ptr, dc.ptr], outs=[dt.ptr], count=count, deps=[0]),
+           dict(dtype="f32", compute="max", ins=[dt.ptr, da.ptr], outs=[du.ptr], count=count, deps=[1]),
+           dict(dtype="f32", compute="sum", ins=[du.ptr, dt.ptr], outs=[dt.ptr], count=count, deps=[2, 1])]
+    g = hip.Graph(ops)
+    g.trace(True)
+    t1 = oracle.reduce("f32", "prod", [oracle.reduce("f32", "sum", [a, b]), c])
+    u = oracle.reduce("f32", "max", [t1, a])
+    want = oracle.reduce("f32", "sum", [u, t1])
+    for _ in range(3):
+        _run_and_check(torch, hip, g, 4)
+        H.assert_bits_equal(dt.download(), want, "chain t")
+        H.assert_bits_equal(du.download(), u, "chain u")
+    uid, part, ready, done = _timeline(torch, g)
+    n_parts = int((uid == 0).sum())
+    assert n_parts > 16 and all(int((uid == k).sum()) == n_parts for k in range(4))
+    for k in (1, 2, 3):  # part p never before part p of the op before
+        for p in range(n_parts):
+            assert ready[(uid == k) & (part == p)][0] >= done[(uid == k - 1) & (part == p)][0]
+    # ... and the chain did overlap: some part of op 1 was ready before op 0 was complete
+    assert ready[uid == 1].min() < done[uid == 0].max()
+    assert dt.guards_intact() and du.guards_intact()
+    g.destroy()
+
+
+def test_shifted_overlap_keeps_the_dependency_whole(hip, oracle):
+    """B reads A's output 64 elements further on (and, behind A, X's output likewise): part p
+    of B needs other parts of A, so B must wait for all of A.  Checked on the timeline and on
+    the bits."""
+    import torch
+    count, shift = 2 * 1000 * 1000, 64
+    a, b = H.gen("bf16", count, 98, 0), H.gen("bf16", count, 98, 1)
+    tail = H.gen("bf16", shift, 98, 2)
+    da, db = H.DevBuf(torch, "bf16", count, 0, src=a), H.DevBuf(torch, "bf16", count, 0, src=b)
+    dT = H.DevBuf(torch, "bf16", count + shift, 0, src=np.concatenate([np.zeros(count, dtype=tail.dtype), tail]))
+    dU, dV, dW = (H.DevBuf(torch, "bf16", count, 0) for _ in range(3))
+    es = 2
+    ops = [  # X: T[0:n] = a + b
+           dict(dtype="bf16", compute="sum", ins=[da.ptr, db.ptr], outs=[dT.ptr], count=count, deps=[]),
+           # A: U = T[0:n] + a           (same addresses as X's output: part by part)
+           dict(dtype="bf16", compute="sum", ins=[dT.ptr, da.ptr], outs=[dU.ptr], count=count, deps=[0]),
+           # B: V = U + T[64:n+64]       (U at A's addresses, but T shifted against X, which lies behind A)
+           dict(dtype="bf16", compute="sum", ins=[dU.ptr, dT.ptr + shift * es], outs=[dV.ptr], count=count, deps=[1]),
+           # C: W = T[64:n+64] + b       (shifted against X directly)
+           dict(dtype="bf16", compute="sum", ins=[dT.ptr + shift * es, db.ptr], outs=[dW.ptr], count=count, deps=[0])]
+    g = hip.Graph(ops)
+    g.trace(True)
+    T = np.concatenate([oracle.reduce("bf16", "sum", [a, b]), tail])
+    U = oracle.reduce("bf16", "sum", [T[:count], a])
+    for _ in range(3):
+        _run_and_check(torch, hip, g, 4)
+        H.assert_bits_equal(dU.download(), U, "U")
+        H.assert_bits_equal(dV.download(), oracle.reduce("bf16", "sum", [U, T[shift:]]), "V")
+        H.assert_bits_equal(dW.download(), oracle.reduce("bf16", "sum", [T[shift:], b]), "W")
+    uid, part, ready, done = _timeline(torch, g)
+    assert ready[uid == 2].min() >= done[uid == 1].max()  # B after all of A (hence all of X)
+    assert ready[uid == 3].min() >= done[uid == 0].max()  # C after all of X
+    g.destroy()
+
+
+def test_rebind_that_changes_aliasing_rebuilds_the_graph(hip, oracle):
+    """A: t = a + b; B: u = t + c.  Rebinding u onto a's buffer, shifted, makes B overwrite what
+    A reads: the dependency turns whole-op (graph rebuilt inside rebind); rebinding it back
+    restores the part-by-part form.  Results must match sequential execution each time."""
+    import torch
+    count, shift = 1500 * 1000, 64
+    a_full = H.gen("f32", count + shift, 99, 0)
+    b, c = H.gen("f32", count, 99, 1), H.gen("f32", count, 99, 2)
+    dA = H.DevBuf(torch, "f32", count + shift, 0, src=a_full)
+    db, dc = H.DevBuf(torch, "f32", count, 0, src=b), H.DevBuf(torch, "f32", count, 0, src=c)
+    dt, du = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    ops = [dict(dtype="f32", compute="sum", ins=[dA.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0])]
+    g = hip.Graph(ops)
+    g.trace(True)
+    t = oracle.reduce("f32", "sum", [a_full[:count], b])
+    u = oracle.reduce("f32", "sum", [t, c])
+    _run_and_check(torch, hip, g, 2)
+    H.assert_bits_equal(du.download(), u, "before rebind")
+    uid, part, ready, done = _timeline(torch, g)
+    assert all(ready[(uid == 1) & (part == p)][0] >= done[(uid == 0) & (part == p)][0] for p in range(int((uid == 1).sum())))
+    # u -> a's buffer + 64 elements
+    g.rebind(du.ptr, dA.ptr + 4 * shift, 4 * count, _stream(torch))
+    g.trace(True)
+    for _ in range(2):
+        dA.upload(a_full)
+        _run_and_check(torch, hip, g, 2)
+        H.assert_bits_equal(dt.download(), t, "t after rebind")
+        got = dA.download()
+        H.assert_bits_equal(got[shift:], u, "u inside a's buffer")
+        H.assert_bits_equal(got[:shift], a_full[:shift], "a's first elements")
+        uid, part, ready, done = _timeline(torch, g)
+        assert ready[uid == 1].min() >= done[uid == 0].max()
+    # and back
+    g.rebind(dA.ptr + 4 * shift, du.ptr, 4 * count, _stream(torch))
+    dA.upload(a_full)
+    du.upload(np.zeros(count, dtype=np.float32).view(u.dtype))
+    _run_and_check(torch, hip, g, 2)
+    H.assert_bits_equal(du.download(), u, "after rebinding back")
+    assert dA.guards_intact() and du.guards_intact() and dt.guards_intact()
+    g.destroy()
+
+
+def test_part_dependencies_can_be_switched_off(hip, oracle, monkeypatch):
+    import torch
+    monkeypatch.setenv("PCCL_HIP_PART_DEPS", "0")
+    count = 1000 * 1000
+    a, b = H.gen("bf16", count, 100, 0), H.gen("bf16", count, 100, 1)
+    da, db = H.DevBuf(torch, "bf16", count, 0, src=a), H.DevBuf(torch, "bf16", count, 0, src=b)
+    dt, du = H.DevBuf(torch, "bf16", count, 0), H.DevBuf(torch, "bf16", count, 0)
+    g = hip.Graph([dict(dtype="bf16", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+                   dict(dtype="bf16", compute="sum", ins=[dt.ptr, db.ptr], outs=[du.ptr], count=count, deps=[0])])
+    g.trace(True)
+    _run_and_check(torch, hip, g, 2)
+    uid, part, ready, done = _timeline(torch, g)
+    assert ready[uid == 1].min() >= done[uid == 0].max()
+    H.assert_bits_equal(du.download(), oracle.reduce("bf16", "sum", [oracle.reduce("bf16", "sum", [a, b]), b]), "whole-op")
     g.destroy()
