@@ -192,6 +192,20 @@ int pccl_hip_graph_trace(void *graph, int enable);
 int pccl_hip_graph_read_trace(void *graph, void *stream, unsigned long long *records, long capacity,
                               long *n_records);
 
+/* How the executor treats each dependency of the graph (no counterpart in the reference):
+ * one byte per dependency, ops in uid order and each op's dependencies in list order;
+ * 1 = met part by part (part p of the op waits only for part p of that predecessor, see
+ * pccl_op_layout.h), 0 = the op waits for the whole predecessor.  Copies up to `capacity`
+ * bytes and reports the number of dependencies in *n_deps.  graph_rebind may change it. */
+int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capacity, long *n_deps);
+
+/* The rule behind that, on its own: given the ops and the number of parts each is cut into
+ * (part p of an op covers elements [p * per, min((p + 1) * per, count)) of every operand,
+ * per = ceil(count / parts) rounded up to 64), writes one byte per dependency as above.
+ * Touches no device; it exists so that the rule can be checked against every order of
+ * execution it allows. */
+int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int *parts, unsigned char *kinds);
+
 /* Device address of the GraphBufferLayout and launch facts, for inspection. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 

@@ -666,6 +666,49 @@ int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_
   return PCCL_OK;
 }
 
+int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int *parts, unsigned char *kinds) {
+  pccl_host::clear_error();
+  if (n_ops < 0 || (n_ops > 0 && (!ops || !parts))) return fail(PCCL_ERR_INVALID_ARG, "classify_dependencies: bad arguments");
+  std::vector<pccl_op_desc> descs(ops, ops + n_ops);
+  std::vector<int> part_counts(parts, parts + n_ops), indeg(n_ops, 0), topo;
+  std::vector<std::vector<int>> succ(n_ops);
+  size_t n_deps = 0;
+  for (int i = 0; i < n_ops; ++i) {
+    const pccl_op_desc &o = ops[i];
+    if (o.n_deps < 0 || (o.n_deps > 0 && !o.deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
+    if (parts[i] < 1 || o.count < 0 || o.dtype >= PCCL_NUM_DTYPES || o.n_in > PCCL_MAX_INPUTS || o.n_out > PCCL_MAX_OUTPUTS)
+      return fail(PCCL_ERR_INVALID_ARG, "op %d: bad part count, count, dtype or operand count", i);
+    for (int d = 0; d < o.n_deps; ++d) {
+      if (o.deps[d] < 0 || o.deps[d] >= n_ops || o.deps[d] == i) return fail(PCCL_ERR_GRAPH, "op %d: dependency %d is not another op", i, o.deps[d]);
+      succ[o.deps[d]].push_back(i);
+      ++indeg[i];
+    }
+    n_deps += (size_t)o.n_deps;
+  }
+  for (int i = 0; i < n_ops; ++i)
+    if (!indeg[i]) topo.push_back(i);
+  for (size_t k = 0; k < topo.size(); ++k)
+    for (int v : succ[topo[k]])
+      if (--indeg[v] == 0) topo.push_back(v);
+  if ((int)topo.size() != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle");
+  const std::vector<unsigned char> flags = classify_dependencies(descs, part_counts, topo);
+  if (n_deps && !kinds) return fail(PCCL_ERR_INVALID_ARG, "classify_dependencies: kinds is null");
+  if (n_deps) memcpy(kinds, flags.data(), n_deps);
+  return PCCL_OK;
+}
+
+int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capacity, long *n_deps) {
+  pccl_host::clear_error();
+  Graph *G = (Graph *)graph;
+  if (!G || !n_deps) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: null argument");
+  if (capacity < 0 || (capacity > 0 && !kinds)) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: bad buffer");
+  std::lock_guard<std::mutex> lock(G->mu);
+  *n_deps = (long)G->part_edge.size();
+  const long n = std::min<long>(capacity, *n_deps);
+  if (n > 0) memcpy(kinds, G->part_edge.data(), (size_t)n);
+  return PCCL_OK;
+}
+
 int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;

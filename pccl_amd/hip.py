@@ -78,6 +78,8 @@ def lib():
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.pccl_hip_classify_dependencies.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), vp]
+        L.pccl_hip_graph_dependency_kinds.argtypes = [vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_trace.argtypes = [vp, ci]
         L.pccl_hip_graph_read_trace.argtypes = [vp, vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_next_signal_base.argtypes = [vp, ctypes.POINTER(ctypes.c_uint)]
@@ -167,42 +169,66 @@ def accumulate(dtype, compute, src, outs, count, stream=None):
                                      len(outs), count, ctypes.c_void_p(_addr(stream))))
 
 
+def _op_descs(ops):
+    """list of op dicts -> (OpDesc array, objects to keep alive while it is in use)."""
+    n = len(ops)
+    arr = (OpDesc * max(n, 1))()
+    keep = []
+    for i, o in enumerate(ops):
+        d = arr[i]
+        d.op_uid = i
+        prim = o.get("primitive")
+        if prim in (NOTIFY, GET_NOTIFIED):
+            # signal op: "signal" = address of the 32-bit word, "value" = 0..65535
+            d.primitive = prim
+            d.n_in, d.n_out = (0, 1) if prim == NOTIFY else (1, 0)
+            (d.outs if prim == NOTIFY else d.ins)[0] = _addr(o["signal"])
+            d.count = o["value"]
+        else:
+            n_in, n_out = len(o["ins"]), len(o["outs"])
+            d.primitive = prim if prim is not None else (COPY if n_in == 1 else REDUCE)
+            d.dtype = _code(DTYPES, o["dtype"])
+            d.compute = _code(COMPUTES, o.get("compute", "sum"))
+            d.n_in, d.n_out = n_in, n_out
+            for k in range(min(n_in, MAX_INPUTS)):
+                d.ins[k] = _addr(o["ins"][k])
+            for k in range(min(n_out, MAX_OUTPUTS)):
+                d.outs[k] = _addr(o["outs"][k])
+            d.count = o["count"]
+        deps = list(o.get("deps", ()))
+        d.n_deps = len(deps)
+        buf = (ctypes.c_int * max(len(deps), 1))(*deps)
+        keep.append(buf)
+        d.deps = ctypes.cast(buf, ctypes.POINTER(ctypes.c_int))
+    return arr, keep
+
+
+def part_elems(count, parts):
+    """Elements per part of an op cut into `parts` parts (the last part may be shorter)."""
+    per = (count + parts - 1) // parts
+    return (per + 63) // 64 * 64
+
+
+def classify_dependencies(ops, parts):
+    """The executor's rule for which dependencies are met part by part, without a device:
+    ops as for Graph, parts[i] = number of parts of op i.  Returns one flag per dependency
+    (ops in order, dependencies in list order)."""
+    arr, keep = _op_descs(ops)
+    n_deps = sum(len(o.get("deps", ())) for o in ops)
+    kinds = (ctypes.c_ubyte * max(n_deps, 1))()
+    pa = (ctypes.c_int * max(len(ops), 1))(*parts)
+    _check(lib().pccl_hip_classify_dependencies(arr, len(ops), pa, kinds))
+    return list(kinds)[:n_deps]
+
+
 class Graph:
     """A DAG of COPY / REDUCE ops resident on the device, drained by one launch."""
 
     def __init__(self, ops, tile_bytes=0):
         """ops: list of dicts with keys dtype, compute, ins, outs, count, deps (op index list)."""
-        n = len(ops)
-        arr = (OpDesc * max(n, 1))()
-        self._keep = []
-        for i, o in enumerate(ops):
-            d = arr[i]
-            d.op_uid = i
-            prim = o.get("primitive")
-            if prim in (NOTIFY, GET_NOTIFIED):
-                # signal op: "signal" = address of the 32-bit word, "value" = 0..65535
-                d.primitive = prim
-                d.n_in, d.n_out = (0, 1) if prim == NOTIFY else (1, 0)
-                (d.outs if prim == NOTIFY else d.ins)[0] = _addr(o["signal"])
-                d.count = o["value"]
-            else:
-                n_in, n_out = len(o["ins"]), len(o["outs"])
-                d.primitive = prim if prim is not None else (COPY if n_in == 1 else REDUCE)
-                d.dtype = _code(DTYPES, o["dtype"])
-                d.compute = _code(COMPUTES, o.get("compute", "sum"))
-                d.n_in, d.n_out = n_in, n_out
-                for k in range(min(n_in, MAX_INPUTS)):
-                    d.ins[k] = _addr(o["ins"][k])
-                for k in range(min(n_out, MAX_OUTPUTS)):
-                    d.outs[k] = _addr(o["outs"][k])
-                d.count = o["count"]
-            deps = list(o.get("deps", ()))
-            d.n_deps = len(deps)
-            buf = (ctypes.c_int * max(len(deps), 1))(*deps)
-            self._keep.append(buf)
-            d.deps = ctypes.cast(buf, ctypes.POINTER(ctypes.c_int))
+        arr, self._keep = _op_descs(ops)
         self._h = ctypes.c_void_p(None)
-        _check(lib().pccl_hip_graph_create(arr, n, tile_bytes, ctypes.byref(self._h)))
+        _check(lib().pccl_hip_graph_create(arr, len(ops), tile_bytes, ctypes.byref(self._h)))
 
     def run(self, stream=None):
         _check(lib().pccl_hip_graph_run(self._h, ctypes.c_void_p(_addr(stream))))
@@ -228,6 +254,15 @@ class Graph:
         lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)
         _check(lib().pccl_hip_graph_info(self._h, ctypes.byref(lay), ctypes.byref(nt), ctypes.byref(nw)))
         return {"device_layout": lay.value, "n_tiles": nt.value, "n_workgroups": nw.value}
+
+    def dependency_kinds(self):
+        """One flag per dependency (ops in uid order, dependencies in list order): 1 = met part
+        by part, 0 = waits for the whole predecessor."""
+        n = ctypes.c_long(0)
+        _check(lib().pccl_hip_graph_dependency_kinds(self._h, None, 0, ctypes.byref(n)))
+        buf = (ctypes.c_ubyte * max(n.value, 1))()
+        _check(lib().pccl_hip_graph_dependency_kinds(self._h, buf, n.value, ctypes.byref(n)))
+        return list(buf)[:n.value]
 
     def trace(self, enable=True):
         """Switches the per-entry timeline on or off for the following runs."""

@@ -124,3 +124,50 @@ def replay_with_signals(oracle, ops, order, resolve):
             oracle.reduce_copy(o["dtype"], o["compute"], [resolve(*x, o["count"]) for x in o["ins"]],
                                [resolve(*x, o["count"]) for x in o["outs"]])
     return slots
+
+
+def random_pool_program(rng, pool_elems, n_ops):
+    """Ops in program order over regions of one f32 pool.  Regions of equal length start at
+    multiples of that length, sometimes pushed on by a few hundred elements, so that later ops
+    meet earlier results at the same address, at a shifted address, or not at all.  Inside an
+    op an output may be one of the inputs exactly; otherwise its operands are disjoint.
+    Dependencies: every earlier op with a conflicting operand (RAW, WAW, WAR), transitively
+    reduced, so that the program means what running the ops one after the other means and
+    leans on whole-op dependencies being transitive."""
+    lengths = [40_000, 40_000, 65_536, 100_000]
+    ops = []
+    for i in range(n_ops):
+        n = lengths[rng.integers(len(lengths))]
+        def region():
+            base = int(rng.integers(0, (pool_elems - n - 1024) // n)) * n
+            if rng.random() < 0.25:
+                base += int(rng.integers(1, 8)) * 64
+            return base
+        def disjoint(a, b):
+            return a + n <= b or b + n <= a
+        n_in, n_out = int(rng.integers(1, 4)), int(rng.integers(1, 3))
+        ins, outs = [], []
+        while len(ins) < n_in:
+            r = region()
+            if all(disjoint(r, x) for x in ins):
+                ins.append(r)
+        while len(outs) < n_out:
+            r = ins[0] if (not outs and rng.random() < 0.3) else region()
+            if all(disjoint(r, x) for x in outs) and all(disjoint(r, x) or r == x for x in ins):
+                outs.append(r)
+        ops.append(dict(count=n, ins=ins, outs=outs, compute=["sum", "max", "min"][rng.integers(3)] if n_in > 1 else "sum"))
+    def overlap(a, na, b, nb):
+        return a < b + nb and b < a + na
+    reach = []  # reach[i]: ops that op i transitively depends on
+    for i, o in enumerate(ops):
+        direct = []
+        for j in range(i):
+            p = ops[j]
+            conflict = any(overlap(x, p["count"], y, o["count"]) for x in p["outs"] for y in o["ins"] + o["outs"]) or \
+                any(overlap(x, p["count"], y, o["count"]) for x in p["ins"] for y in o["outs"])
+            if conflict:
+                direct.append(j)
+        kept = [j for j in direct if not any(j in reach[k] for k in direct if k != j)]
+        o["deps"] = kept
+        reach.append(set(direct).union(*[reach[j] for j in direct]) if direct else set())
+    return ops
