@@ -398,8 +398,13 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
             t = __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT);
           }
           if (t < n) {
-            e = g.queue_entries[q][t];
-            entry_index = (size_t)t * kQueues + q;
+            // Only lane 0 is here, so "the first lane's value" is the value: with the index
+            // uniform, this load and those of the op's slot and header below are scalar loads,
+            // which do not queue behind the vector memory traffic of the parts in flight on
+            // this compute unit.  What they read is constant during a run.
+            const int qs = __builtin_amdgcn_readfirstlane(q), ts = __builtin_amdgcn_readfirstlane(t);
+            e = g.queue_entries[qs][ts];
+            entry_index = (size_t)ts * kQueues + qs;
             go = 1;
             if (g.trace) {
               cur_trace = g.trace + entry_index * kTraceWords;
@@ -412,7 +417,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           }
         }
         if (!go) break;
-        const int uid = (int)(e & 0xffffffffu);
+        const int uid = __builtin_amdgcn_readfirstlane((int)(e & 0xffffffffu));
         pccl_operation_layout_header *hc = &g.headers[uid];
         const PayloadSlot *sc = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
         // wait until every dependency of the op has arrived (none: nothing ever writes the
@@ -420,7 +425,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         // The count, the first look at the arrivals and the primitive go out together.
         // Dependencies met part by part arrive on the entry's own word instead; the entry is
         // that word's only reader and clears it for the next run.
-        const unsigned int w12 = __hip_atomic_load(word12(hc), __ATOMIC_RELAXED, AGENT);
+        const unsigned int w12 = *word12(hc);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
         unsigned int *part_word = g.part_arrivals ? g.part_arrivals + entry_index : nullptr;
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
