@@ -170,14 +170,27 @@ template <> struct Dtype<PCCL_F16> {
       acc.x = Op::f(acc.x, x.x);
       acc.y = Op::f(acc.y, x.y);
     }
+    float lo = acc.x, hi = acc.y;
+    rounded_to_f32(lo);
+    rounded_to_f32(hi);
+    acc.x = lo;
+    acc.y = hi;
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(acc, f16x2));
   }
   template <class Op, int N> static __device__ __forceinline__ elem_t elem(const elem_t (&e)[N]) {
     float acc = (float)__builtin_bit_cast(_Float16, e[0]);
 #pragma unroll
     for (int k = 1; k < N; ++k) acc = Op::f(acc, (float)__builtin_bit_cast(_Float16, e[k]));
+    rounded_to_f32(acc);
     return __builtin_bit_cast(unsigned short, (_Float16)acc);
   }
+  // The fold's last step must round to binary32 before the result is narrowed.  Left alone,
+  // the compiler folds "multiply a float by a widened half, narrow to half" into one
+  // v_fma_mixlo_f16, which rounds the exact product once; where the binary32 product lies
+  // exactly between two binary16 values that is one unit away from rounding twice (seen on
+  // 1 of ~10^4 head / tail elements of an 8-input product).  The empty asm makes the value
+  // opaque to that pattern and costs no instruction.
+  static __device__ __forceinline__ void rounded_to_f32(float &x) { asm volatile("" : "+v"(x)); }
 };
 
 // 8-bit floats (OCP E4M3FN and E5M2), four per word.  Widening is the hardware's exact

@@ -224,3 +224,58 @@ def test_group_allocation(hip, oracle):
     hip.free(d[0])
     with pytest.raises(hip.PcclError):
         hip.alloc_group(0, 16)
+
+
+# ---- the fold rounds to binary32 at every step, then once to the element type ----------------
+
+def _tie_tuples(oracle, dtype, compute, n_in, want, seed):
+    """Tuples of n_in elements whose binary32 left fold lies EXACTLY between two values of the
+    element type.  There, rounding the last step's exact result straight to the element type
+    (what a fused multiply-and-narrow instruction does) differs from rounding it to binary32
+    first in about half the cases, so these are the inputs that tell the two apart."""
+    rng = np.random.default_rng(seed)
+    low_bits = 13 if dtype == "f16" else 16
+    found = []
+    while sum(len(f) for f in found) < want:
+        vals = rng.uniform(0.5, 2.0, (1 << 20, n_in)).astype(np.float32)
+        if compute == "sum":
+            vals *= rng.choice(np.float32([1, -1, 0.25, 8]), vals.shape)
+        bits = oracle.narrow(dtype, vals)
+        x = oracle.widen(dtype, bits)
+        acc = x[:, 0].copy()
+        for k in range(1, n_in):
+            acc = (acc * x[:, k] if compute == "prod" else acc + x[:, k]).astype(np.float32)
+        tie = (acc.view(np.uint32) & np.uint32((1 << low_bits) - 1)) == np.uint32(1 << (low_bits - 1))
+        found.append(bits[tie])
+    return np.concatenate(found)[:want]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_fold_rounds_to_binary32_before_narrowing(hip, oracle, dtype):
+    """Every path an element can take (16-byte packs, the element-wise head and tail of an
+    unaligned buffer, parts of the queue executor) must round like the CPU checker on inputs
+    whose binary32 fold is a tie of the element type."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    for compute, n_in in (("prod", 8), ("prod", 3), ("sum", 4), ("sum", 8)):
+        ties = _tie_tuples(oracle, dtype, compute, n_in, 7 * 40, 4242 + n_in)
+        ins = [np.ascontiguousarray(ties[:, k]) for k in range(n_in)]
+        want = oracle.reduce(dtype, compute, ins)
+        what = "%s %s %d inputs" % (dtype, compute, n_in)
+        # all through packs (aligned), and with an element-wise head and tail (offset buffers)
+        H.assert_bits_equal(H.hip_reduce(torch, hip, dtype, compute, ins)[0], want, what + ", aligned")
+        got = H.hip_reduce(torch, hip, dtype, compute, ins, in_offsets=[2 * (k + 1) for k in range(n_in)], out_offsets=[6])[0]
+        H.assert_bits_equal(got, want, what + ", offset buffers")
+        # seven elements at a time: every element goes the element-wise way
+        for lo in range(0, len(want), 7):
+            got = H.hip_reduce(torch, hip, dtype, compute, [a[lo:lo + 7] for a in ins], out_offsets=[2])[0]
+            H.assert_bits_equal(got, want[lo:lo + 7], what + ", elements %d.." % lo)
+        # the queue executor, parts of 1 KiB starting off 16 bytes
+        d_in = [H.DevBuf(torch, dtype, len(want), 2 * (k % 5), src=a) for k, a in enumerate(ins)]
+        d_out = H.DevBuf(torch, dtype, len(want), 10)
+        g = hip.Graph([dict(dtype=dtype, compute=compute, ins=[b.ptr for b in d_in], outs=[d_out.ptr], count=len(want))],
+                      tile_bytes=1024)
+        g.run(stream)
+        assert g.status(stream) == (1, 1)
+        H.assert_bits_equal(d_out.download(), want, what + ", queue")
+        g.destroy()
