@@ -625,24 +625,51 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     const uintptr_t a = (uintptr_t)p;
     return a >= lo && a < hi ? (void *)((uintptr_t)new_base + (a - lo)) : (void *)p;
   };
-  for (pccl_op_desc &o : G->descs) {
-    for (int k = 0; k < o.n_in; ++k) o.ins[k] = moved(o.ins[k]);
-    for (int k = 0; k < o.n_out; ++k) o.outs[k] = moved(o.outs[k]);
+  // the ops with their operands moved; nothing of the graph changes until this has been checked
+  std::vector<pccl_op_desc> next = G->descs;  // (dependency lists stay where they are, in deps_store)
+  for (size_t i = 0; i < next.size(); ++i) {
+    pccl_op_desc &o = next[i];
+    // a signal word moves like an operand; it is 4 bytes whatever the op's dtype field says
+    const bool is_signal = o.primitive == PCCL_NOTIFY || o.primitive == PCCL_GET_NOTIFIED;
+    const uintptr_t es = is_signal ? 4 : (uintptr_t)elem_bytes(o.dtype);
+    for (int k = 0; k < o.n_in + o.n_out; ++k) {
+      void *p = moved(k < o.n_in ? o.ins[k] : o.outs[k - o.n_in]);
+      if ((uintptr_t)p % es)
+        return fail(PCCL_ERR_MISALIGNED, "graph_rebind: op %zu operand %d would not be %d-byte aligned", i, k, (int)es);
+      if (k < o.n_in) o.ins[k] = p;
+      else o.outs[k - o.n_in] = p;
+    }
   }
   // Which dependencies may be met part by part depends on which operands share addresses
   // (an output tensor that now is the input tensor, say).  If that changed, the arena is
-  // built again from the moved ops; earlier runs on `stream` finish first.
-  if (classify_dependencies(G->descs, G->parts, G->topo) != G->part_edge) {
+  // built again from the moved ops, beside the old one, which is given up only when the new
+  // one stands; earlier runs on `stream` finish first.
+  if (classify_dependencies(next, G->parts, G->topo) != G->part_edge) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    Graph fresh;
+    fresh.descs.swap(next);
+    fresh.tile_bytes = G->tile_bytes;
+    fresh.trace = G->trace;
+    fresh.trace_on = G->trace_on;
+    fresh.spin_limit = G->spin_limit;
+    const int rc = build_graph(&fresh, G->runs + 1u);
+    if (rc != PCCL_OK) return rc;
     char *old_dev = G->dev;
-    const int rc = build_graph(G, G->runs + 1u);
-    if (rc != PCCL_OK) {
-      G->dev = old_dev;  // the old arena still describes the old addresses: the graph is unusable
-      return rc;
-    }
+    G->dev = fresh.dev;
+    G->image.swap(fresh.image);
+    G->payload_off = fresh.payload_off;
+    G->total_tiles = fresh.total_tiles;
+    G->n_wg = fresh.n_wg;
+    G->device = fresh.device;
+    G->kernel = fresh.kernel;
+    G->descs.swap(fresh.descs);
+    G->parts.swap(fresh.parts);
+    G->topo.swap(fresh.topo);
+    G->part_edge.swap(fresh.part_edge);
     PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
+  G->descs.swap(next);
   char *payloads = G->image.data() + G->payload_off;
   for (int i = 0; i < G->n_ops; ++i) {
     pccl_op_payload *pl = (pccl_op_payload *)(payloads + kPayloadStride * (size_t)i);

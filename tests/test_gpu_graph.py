@@ -600,3 +600,23 @@ def test_part_dependencies_can_be_switched_off(hip, oracle, monkeypatch):
     assert ready[uid == 1].min() >= done[uid == 0].max()
     H.assert_bits_equal(du.download(), oracle.reduce("bf16", "sum", [oracle.reduce("bf16", "sum", [a, b]), b]), "whole-op")
     g.destroy()
+
+
+def test_rebind_refuses_a_move_that_breaks_element_alignment(hip, oracle):
+    """f64 operands moved by 4 bytes: refused, and the graph keeps working where it was."""
+    import torch
+    count = 5000
+    a, b = H.gen("f64", count, 101, 0), H.gen("f64", count, 101, 1)
+    da, db = H.DevBuf(torch, "f64", count, 0, src=a), H.DevBuf(torch, "f64", count, 0, src=b)
+    do, spare = H.DevBuf(torch, "f64", count, 0), H.DevBuf(torch, "f64", count + 1, 0)
+    g = hip.Graph([dict(dtype="f64", compute="sum", ins=[da.ptr, db.ptr], outs=[do.ptr], count=count)])
+    with pytest.raises(hip.PcclError) as e:
+        g.rebind(do.ptr, spare.ptr + 4, 8 * count, _stream(torch))
+    assert e.value.code == hip.ERR_MISALIGNED
+    _run_and_check(torch, hip, g, 1)
+    H.assert_bits_equal(do.download(), oracle.reduce("f64", "sum", [a, b]), "after the refused rebind")
+    g.rebind(do.ptr, spare.ptr + 8, 8 * count, _stream(torch))
+    _run_and_check(torch, hip, g, 1)
+    H.assert_bits_equal(spare.download()[1:], oracle.reduce("f64", "sum", [a, b]), "after the good rebind")
+    assert spare.guards_intact()
+    g.destroy()
