@@ -265,6 +265,29 @@ def main():
                         "the 14-step figure walks 1.3 GiB of distinct data"}
             del grad, peers, result, send
 
+            # the whole collective over 8 virtual ranks as ONE launch of the queue executor:
+            # 112 ops (8 ranks x 14 steps), every dependency a read of what the step before wrote
+            full = {}
+            for per_rank_mib in (1, 8, 32):
+                ir, per_rank = lang.ring_allreduce(8, (per_rank_mib << 20) // 2 // 8, dtype="bf16")
+                low = ir.lower()
+                rb = {"in": [randn(torch, per_rank, "bf16", 1e-2) for _ in range(8)],
+                      "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
+                g = hip.Graph(lang.bind(low, lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+                tf = event_times_us(torch, lambda: g.run(stream), 20, 3)
+                done, total = g.status(stream)
+                assert done == total == len(low)
+                for r in range(1, 8):
+                    assert torch.equal(rb["out"][r], rb["out"][0])
+                moved = sum((len(o["ins"]) + len(o["outs"])) * o["count"] * 2 for o in low)
+                kinds = g.dependency_kinds()
+                full["8_ranks_x_%d_MiB" % per_rank_mib] = dict(stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low),
+                                                              algorithmic_bytes=moved, queue_entries=g.info()["n_tiles"],
+                                                              dependencies_part_by_part="%d of %d" % (sum(kinds), len(kinds)))
+                g.destroy()
+                del rb
+            extras["ring_allreduce_one_launch"] = full
+
         # ---- plumbing config: f32 2 -> 1, 4 MiB ---------------------------------------------
         if want("plumbing"):
             a, b = randn(torch, 1 << 20, "f32"), randn(torch, 1 << 20, "f32")

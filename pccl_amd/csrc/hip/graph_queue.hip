@@ -91,6 +91,7 @@ struct Graph {
   std::vector<int> parts;            // per op
   std::vector<int> topo;             // a topological order of the ops
   std::vector<unsigned char> part_edge;  // per dependency, in descs order: met part by part
+  std::vector<unsigned char> part_eligible;  // per op: its dependencies may be met part by part
 };
 
 // ---- which dependencies can be met part by part -------------------------------
@@ -102,6 +103,7 @@ struct Graph {
 // at all means that the dependency orders something this code cannot see; both keep the
 // dependency whole-op.
 enum Conflict { kNoConflict, kSameAddress, kOtherAddress };
+constexpr long long kMaxPartWordEntries = 1ll << 22;
 
 Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t bytes) {
   bool any = false, other = false;
@@ -126,8 +128,11 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // theirs.  Whole-op semantics promise b that ALL its ancestors are complete, so b must not
 // conflict with any op of behind[b] at differing addresses either; when it would, or when the
 // list grows long, the dependency stays whole-op (which also empties what lies behind it).
+// `eligible` (optional, per op): 0 keeps every dependency OF that op whole-op whatever the rule
+// would allow (the caller's judgement of whether it pays, see build_graph).
 std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
-                                                 const std::vector<int> &topo) {
+                                                 const std::vector<int> &topo,
+                                                 const std::vector<unsigned char> *eligible = nullptr) {
   constexpr size_t kMaxBehind = 32;
   const int n_ops = (int)ops.size();
   std::vector<size_t> dep_start(n_ops + 1, 0);
@@ -140,7 +145,7 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
   auto bytes_of = [&](const pccl_op_desc &o) { return (uintptr_t)o.count * (uintptr_t)elem_bytes(o.dtype); };
   for (int b : topo) {
     const pccl_op_desc &B = ops[b];
-    if (!is_data(B) || parts[b] < 2) continue;
+    if (!is_data(B) || parts[b] < 2 || (eligible && !(*eligible)[b])) continue;
     const uintptr_t bytes = bytes_of(B);
     const uintptr_t per = (uintptr_t)part_elems(B.count, parts[b]) * (uintptr_t)elem_bytes(B.dtype);
     for (int d = 0; d < B.n_deps; ++d) {
@@ -327,8 +332,11 @@ int build_graph(Graph *G, unsigned int run_number) {
   // ---- dependencies met part by part ---------------------------------------
   // Successor lists again, this time with the successors that are released part by part
   // first, and beside each of those the entry index of its part 0.
+  // Each entry then needs a word of its own, 64 bytes from the next (see the arena layout);
+  // graphs of more than 4 Mi entries (a 256 MiB array) keep every dependency whole-op.
   G->parts = parts;
-  G->part_edge = classify_dependencies(G->descs, parts, G->topo);
+  G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
+  G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
   std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
   bool any_part_edge = false;
   {
@@ -364,8 +372,13 @@ int build_graph(Graph *G, unsigned int run_number) {
   const size_t off_ready = off;   off = align_up(off + sizeof(HotWord) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_gbase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_groups = off;  off = align_up(off + sizeof(HotWord) * (size_t)kPartGroups * (size_t)std::max(n_grouped, 1), 256);
+  // One word per entry, 64 bytes apart: a word is polled by the workgroup that holds its entry
+  // and bumped by others.  Packed 32 to a 128-byte line they cost more than the part-by-part
+  // hand-over saves (ring all-reduce of 8 x 1 MiB: 82 us against 76 us with whole-op waits;
+  // 64 bytes apart: 66 us; 8 x 8 MiB: 114 -> 94 us against 123; the 4096-op schedule 181 -> 171 us).
   const size_t off_part_arrivals = off;
-  if (any_part_edge) off = align_up(off + sizeof(unsigned int) * (size_t)(tiles + kQueues), 256);
+  const int part_shift = 4;
+  if (any_part_edge) off = align_up(off + (sizeof(unsigned int) << part_shift) * (size_t)(tiles + kQueues), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
   const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
@@ -401,6 +414,7 @@ int build_graph(Graph *G, unsigned int run_number) {
   C->succ = (const int *)(dev + off_succ);
   C->succ_part_base = (const int *)(dev + off_succ_part);
   C->part_arrivals = any_part_edge ? (unsigned int *)(dev + off_part_arrivals) : nullptr;
+  C->part_shift = part_shift;
   C->trace = G->trace_on ? G->trace : nullptr;
   C->group_base = (const int *)(dev + off_gbase);
   C->groups = (HotWord *)(dev + off_groups);
@@ -644,7 +658,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // (an output tensor that now is the input tensor, say).  If that changed, the arena is
   // built again from the moved ops, beside the old one, which is given up only when the new
   // one stands; earlier runs on `stream` finish first.
-  if (classify_dependencies(next, G->parts, G->topo) != G->part_edge) {
+  if (classify_dependencies(next, G->parts, G->topo, &G->part_eligible) != G->part_edge) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
     fresh.descs.swap(next);
@@ -666,6 +680,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->parts.swap(fresh.parts);
     G->topo.swap(fresh.topo);
     G->part_edge.swap(fresh.part_edge);
+    G->part_eligible.swap(fresh.part_eligible);
     PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }

@@ -42,7 +42,9 @@ struct GraphControl {
   HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
   HotWord *ready;                         // per op: dependencies that have arrived in this run
   unsigned long long *trace;              // null, or 4 words per queue entry (see kTrace*)
-  unsigned int *part_arrivals;            // per queue entry (t * kQueues + q): part-by-part dependencies that have arrived
+  unsigned int *part_arrivals;            // per queue entry (t * kQueues + q), 1 << part_shift words apart:
+                                          // part-by-part dependencies that have arrived
+  int part_shift;
   const int *succ_part_base;              // beside succ: entry index of part 0 of a successor released part by part
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
@@ -284,7 +286,7 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   if (n_part_next) {
     const int *first_entry = g.succ_part_base + op.succ_start;
     for (int s = 0; s < n_part_next; ++s)
-      __hip_atomic_fetch_add(&g.part_arrivals[first_entry[s] + part], 1u, __ATOMIC_RELAXED, AGENT);
+      __hip_atomic_fetch_add(&g.part_arrivals[(size_t)(first_entry[s] + part) << g.part_shift], 1u, __ATOMIC_RELAXED, AGENT);
   }
   int counted = parts;  // what remaining_executors_ counts: parts, or groups of parts
   bool drawn = false;
@@ -427,7 +429,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         // that word's only reader and clears it for the next run.
         const unsigned int w12 = *word12(hc);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
-        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + entry_index : nullptr;
+        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + (entry_index << g.part_shift) : nullptr;
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;
