@@ -254,16 +254,6 @@ int build_graph(Graph *G, unsigned int run_number) {
   }
   occ = std::min(occ, 8);
   const long long cap = (long long)pccl_host::compute_units() * occ;
-  // parts: with the built-in part size an op is cut into at most one part per resident
-  // workgroup, so that one large op alone fills the chip in a single round of parts
-  for (int i = 0; i < n_ops; ++i) {
-    long p = (op_bytes[i] + tile_bytes - 1) / tile_bytes;
-    if (default_tile) p = std::min<long>(p, (long)cap);
-    parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
-    tiles += parts[i];
-  }
-  if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
-
   // ---- acyclicity (Kahn) -----------------------------------------------------
   std::vector<int> succ_start(n_ops + 1, 0);
   for (int i = 0; i < n_ops; ++i) succ_start[i + 1] = succ_start[i] + n_succ[i];
@@ -312,6 +302,34 @@ int build_graph(Graph *G, unsigned int run_number) {
     }
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
   }
+  // ---- parts ------------------------------------------------------------------
+  // A given tile_bytes cuts every op into parts of that size.  The built-in choice works per
+  // dependency level: the parts of one level should be about 0.8 of a round for the resident
+  // workgroups (part = 1.25 x level bytes / workgroups, within 8 KiB .. 128 KiB), so that with
+  // dependencies met part by part every workgroup draws about one part of each level in
+  // turn.  Measured on ring all-reduces of 8 x 1 / 8 / 32 / 64 MiB and on the 4096-op schedule
+  // with fixed part sizes of 16 .. 256 KiB: each has its best time where a level holds 0.7 to
+  // 1.3 rounds (8 x 64 MiB: 32 KiB parts = 2.7 rounds 385 us, 64 KiB = 1.3 rounds 339 us,
+  // 128 KiB = 0.7 rounds 355 us; the schedule: 16 KiB = 2 rounds 222 us, 32 KiB = 1.1 rounds
+  // 172 us, 64 KiB = 0.7 rounds 190 us), and one large op alone in its level fills the chip in
+  // a single round.
+  {
+    std::vector<long long> level_bytes(n_ops + 1, 0);
+    for (int i = 0; i < n_ops; ++i) level_bytes[level[i]] += op_bytes[i];
+    for (int i = 0; i < n_ops; ++i) {
+      long part_bytes = tile_bytes;
+      if (default_tile) {
+        const long long want = level_bytes[level[i]] * 5 / (cap * 4);
+        part_bytes = (long)std::min<long long>(std::max<long long>((want + 4095) / 4096 * 4096, 8 << 10), 128 << 10);
+      }
+      long p = (op_bytes[i] + part_bytes - 1) / part_bytes;
+      if (default_tile) p = std::min<long>(p, (long)cap);
+      parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
+      tiles += parts[i];
+    }
+    if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
+  }
+
   // global order of the entries: by level, then op id, then part.  (A list schedule of the
   // graph under a cost model, which lets short chains run ahead of long ones, was measured on
   // the 4096-op schedule and was no faster: workgroups wait longer for dependencies there.)
