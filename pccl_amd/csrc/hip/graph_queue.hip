@@ -5,7 +5,8 @@
 // Protocol (the reference declares the structs, operator.h:7-38, but no code
 // reads or writes them, so the protocol is defined here):
 //   * an op is split into required_executors_ parts of about tile_bytes of
-//     output; a queue entry names (op_uid, part);
+//     output (built-in choice: sized per dependency level, see "parts" below);
+//     a queue entry names (op_uid, part);
 //   * the entries of all ops are laid out once, at graph creation, in a
 //     topological order (dependency level, then op id, then part) and dealt
 //     round-robin onto kQueues ready queues (GraphBufferLayout::ready_queues /
@@ -22,6 +23,9 @@
 //     drain cannot deadlock whatever the number of resident workgroups;
 //   * the workgroup finishing the last part of an op adds one to the arrivals word of
 //     each successor (an atomic whose result nobody waits for) and clears its own;
+//   * where a successor is cut like the op and touches the same bytes part for part,
+//     its part p waits only for the op's part p (classify_dependencies below): every
+//     part of the op bumps the word of the successor's entry p when it is complete;
 //   * data moves between workgroups (possibly on different XCDs, whose L2s are not
 //     coherent with each other) through device-coherent accesses: parts load and
 //     store with sc1, wait for their stores, and only then touch the counters with
@@ -176,11 +180,8 @@ int build_graph(Graph *G, unsigned int run_number) {
   const pccl_op_desc *ops = G->descs.data();
   const int n_ops = (int)G->descs.size();
   long tile_bytes = G->tile_bytes;
-  // With the built-in part size the parts of a large op grow with it instead of multiplying
-  // (see the part count below).
-  const bool default_tile = tile_bytes == 0;
-  if (default_tile) tile_bytes = kDefaultTileBytes;
-  tile_bytes = std::max<long>(tile_bytes, 1024);
+  const bool default_tile = tile_bytes == 0;  // parts are then sized per dependency level, below
+  if (!default_tile) tile_bytes = std::max<long>(tile_bytes, 1024);
 
   // ---- validate; one (dtype, compute) pair for all REDUCE ops --------------
   int g_dtype = -1, g_compute = -1;  // the (dtype, compute) pair of the REDUCE ops, if they share one

@@ -13,7 +13,6 @@ namespace pccl_queue {
 using namespace pccl_dev;
 
 constexpr int kQueues = 8;  // one per XCD of an MI355X
-constexpr long kDefaultTileBytes = 32 << 10;
 constexpr unsigned int kDefaultSpinLimit = 1u << 21;  // a few seconds of polling
 
 // Words that many workgroups update or poll, each alone on its 256-byte line.
