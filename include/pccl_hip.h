@@ -178,7 +178,12 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
 
 /* Replaces operand addresses: every operand that lies in [old_base,
  * old_base+nbytes) moves to new_base + the same offset.  Lets exeOp bind a
- * new input / output tensor without rebuilding the graph. */
+ * new input / output tensor without rebuilding the graph: the new addresses are
+ * uploaded behind earlier work on `stream`.  If the move changes which operands
+ * share addresses (and with that which dependencies can be met part by part),
+ * the call waits for `stream` and builds the device arena again.  A move that
+ * would leave an operand unaligned for its element type returns
+ * PCCL_ERR_MISALIGNED and changes nothing. */
 int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,
                           void *stream);
 
