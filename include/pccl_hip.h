@@ -181,7 +181,8 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
  * new input / output tensor without rebuilding the graph: the new addresses are
  * uploaded behind earlier work on `stream`.  If the move changes which operands
  * share addresses (and with that which dependencies can be met part by part),
- * the call waits for `stream` and builds the device arena again.  A move that
+ * the call waits for `stream` and rewrites the graph's device arena in place
+ * (launches recorded by stream capture stay valid).  A move that
  * would leave an operand unaligned for its element type returns
  * PCCL_ERR_MISALIGNED and changes nothing. */
 int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,

@@ -76,6 +76,7 @@ int elem_bytes(int dtype) { return pccl_host::pccl_dtype_bytes(dtype); }
 
 struct Graph {
   char *dev = nullptr;          // device arena; starts with GraphControl
+  size_t arena_bytes = 0;
   unsigned long long *trace = nullptr;  // device trace records, if tracing was switched on
   bool trace_on = false;
   unsigned int spin_limit = kDefaultSpinLimit;
@@ -176,7 +177,11 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
 
 // Validates G->descs and builds the device arena and its host image from them.  On failure
 // nothing is left allocated.  `run_number`: what the device's run word starts at.
-int build_graph(Graph *G, unsigned int run_number) {
+// `reuse`: an arena of `reuse_bytes` to build into instead of allocating one (the arena's
+// layout depends on the ops and their parts only, not on their addresses, so the arena of the
+// same ops at other addresses fits exactly; a launch recorded by stream capture keeps
+// pointing at it).
+int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t reuse_bytes = 0) {
   const pccl_op_desc *ops = G->descs.data();
   const int n_ops = (int)G->descs.size();
   long tile_bytes = G->tile_bytes;
@@ -378,7 +383,6 @@ int build_graph(Graph *G, unsigned int run_number) {
   G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
   G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
   std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
-  bool any_part_edge = false;
   {
     size_t at = 0;
     for (int i = 0; i < n_ops; ++i)
@@ -386,7 +390,6 @@ int build_graph(Graph *G, unsigned int run_number) {
         if (G->part_edge[at]) {
           ++n_part_next[ops[i].deps[d]];
           ++n_part_pred[i];
-          any_part_edge = true;
         }
     std::vector<int> fill_part(n_ops, 0), fill_whole(n_ops, 0);
     at = 0;
@@ -416,9 +419,12 @@ int build_graph(Graph *G, unsigned int run_number) {
   // and bumped by others.  Packed 32 to a 128-byte line they cost more than the part-by-part
   // hand-over saves (ring all-reduce of 8 x 1 MiB: 82 us against 76 us with whole-op waits;
   // 64 bytes apart: 66 us; 8 x 8 MiB: 114 -> 94 us against 123; the 4096-op schedule 181 -> 171 us).
+  // The words are there whether or not a dependency uses them now: graph_rebind can change
+  // that, and must not change the arena's layout.
   const size_t off_part_arrivals = off;
   const int part_shift = 4;
-  if (any_part_edge) off = align_up(off + (sizeof(unsigned int) << part_shift) * (size_t)(tiles + kQueues), 256);
+  const bool part_words = tiles <= kMaxPartWordEntries;
+  if (part_words) off = align_up(off + (sizeof(unsigned int) << part_shift) * (size_t)(tiles + kQueues), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
   const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
@@ -430,7 +436,10 @@ int build_graph(Graph *G, unsigned int run_number) {
   G->kernel = kernel;
   if (hipGetDevice(&G->device) != hipSuccess) return fail(PCCL_ERR_NO_DEVICE, "no current device");
   G->dev = nullptr;
-  hipError_t e = hipMalloc((void **)&G->dev, arena_bytes);
+  G->arena_bytes = arena_bytes;
+  hipError_t e = hipSuccess;
+  if (reuse && reuse_bytes == arena_bytes) G->dev = reuse;
+  else e = hipMalloc((void **)&G->dev, arena_bytes);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     G->dev = nullptr;
@@ -453,7 +462,7 @@ int build_graph(Graph *G, unsigned int run_number) {
   C->slots = dev + off_payload;
   C->succ = (const int *)(dev + off_succ);
   C->succ_part_base = (const int *)(dev + off_succ_part);
-  C->part_arrivals = any_part_edge ? (unsigned int *)(dev + off_part_arrivals) : nullptr;
+  C->part_arrivals = part_words ? (unsigned int *)(dev + off_part_arrivals) : nullptr;
   C->part_shift = part_shift;
   C->trace = G->trace_on ? G->trace : nullptr;
   C->group_base = (const int *)(dev + off_gbase);
@@ -546,7 +555,7 @@ int build_graph(Graph *G, unsigned int run_number) {
 
   e = hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) {
-    (void)hipFree(dev);
+    if (dev != reuse) (void)hipFree(dev);
     G->dev = nullptr;
     return fail(PCCL_ERR_HIP, "uploading the op graph: %s", hipGetErrorString(e));
   }
@@ -695,9 +704,10 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     }
   }
   // Which dependencies may be met part by part depends on which operands share addresses
-  // (an output tensor that now is the input tensor, say).  If that changed, the arena is
-  // built again from the moved ops, beside the old one, which is given up only when the new
-  // one stands; earlier runs on `stream` finish first.
+  // (an output tensor that now is the input tensor, say).  If that changed, the arena's
+  // contents are built again from the moved ops, in place (its layout does not depend on
+  // addresses, and launches recorded by stream capture point at it); earlier runs on `stream`
+  // finish first.  Only a failed upload can leave the graph unusable.
   if (classify_dependencies(next, G->parts, G->topo, &G->part_eligible) != G->part_edge) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
@@ -706,10 +716,11 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.trace = G->trace;
     fresh.trace_on = G->trace_on;
     fresh.spin_limit = G->spin_limit;
-    const int rc = build_graph(&fresh, G->runs + 1u);
-    if (rc != PCCL_OK) return rc;
     char *old_dev = G->dev;
+    const int rc = build_graph(&fresh, G->runs + 1u, G->dev, G->arena_bytes);
+    if (rc != PCCL_OK) return rc;
     G->dev = fresh.dev;
+    G->arena_bytes = fresh.arena_bytes;
     G->image.swap(fresh.image);
     G->payload_off = fresh.payload_off;
     G->total_tiles = fresh.total_tiles;
@@ -721,7 +732,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->topo.swap(fresh.topo);
     G->part_edge.swap(fresh.part_edge);
     G->part_eligible.swap(fresh.part_eligible);
-    PCCL_HIP_CHECK(hipFree(old_dev));
+    if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
   G->descs.swap(next);

@@ -89,3 +89,39 @@ def test_queue_run_with_signal_ops_replay(hip, oracle):
     # consecutive replays used consecutive run numbers
     assert [b - a for a, b in zip(seen, seen[1:])] == [1 << 16, 1 << 16]
     g.destroy()
+
+
+def test_recorded_queue_run_survives_a_rebind_that_changes_aliasing(hip, oracle):
+    """A: t = a + b; B: u = t + c, recorded once.  Rebinding u onto a's buffer (shifted) turns
+    the dependency from part-by-part to whole-op, which rebuilds the graph's contents; the
+    recording made before must still be valid (same arena) and give sequential results."""
+    import torch
+    count, shift = 1500 * 1000, 64
+    a_full = H.gen("f32", count + shift, 401, 0)
+    b, c = H.gen("f32", count, 401, 1), H.gen("f32", count, 401, 2)
+    dA = H.DevBuf(torch, "f32", count + shift, 0, src=a_full)
+    db, dc = H.DevBuf(torch, "f32", count, 0, src=b), H.DevBuf(torch, "f32", count, 0, src=c)
+    dt, du = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    g = hip.Graph([dict(dtype="f32", compute="sum", ins=[dA.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+                   dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0])])
+    assert g.dependency_kinds() == [1]
+    arena = g.info()["device_layout"]
+    graph = _capture(torch, lambda stream: g.run(stream))
+    t = oracle.reduce("f32", "sum", [a_full[:count], b])
+    u = oracle.reduce("f32", "sum", [t, c])
+    du.view().fill_(0xFF)
+    graph.replay()
+    torch.cuda.synchronize()
+    H.assert_bits_equal(du.download(), u, "replay before the rebind")
+    g.rebind(du.ptr, dA.ptr + 4 * shift, 4 * count, torch.cuda.current_stream().cuda_stream)
+    assert g.dependency_kinds() == [0] and g.info()["device_layout"] == arena
+    for it in range(2):
+        dA.upload(a_full)
+        dt.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        H.assert_bits_equal(dt.download(), t, "t, replay %d after the rebind" % it)
+        H.assert_bits_equal(dA.download()[shift:], u, "u inside a's buffer, replay %d" % it)
+    assert g.status(torch.cuda.current_stream().cuda_stream) == (2, 2)
+    g.destroy()
