@@ -194,7 +194,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
  * 64-bit words: { op_uid | part << 32 | workgroup << 52, ticket drawn, dependencies met,
  * part complete }, times in ticks of the device's constant 100 MHz clock; each run
  * overwrites the last.  enable == 0 stops recording.  Not to be switched while a run is in
- * flight.  read_trace waits for `stream`, copies up to `capacity` records (4 words each)
+ * flight; a run recorded by stream capture keeps the setting it was recorded with.  read_trace waits for `stream`, copies up to `capacity` records (4 words each)
  * and reports the number of entries of the graph in *n_records. */
 int pccl_hip_graph_trace(void *graph, int enable);
 int pccl_hip_graph_read_trace(void *graph, void *stream, unsigned long long *records, long capacity,
@@ -228,7 +228,9 @@ int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
 /* Bounds every wait inside the drain kernel to `polls` polls of a queue slot
  * (default about 2 million, a few seconds).  When a wait gives up the kernel
  * raises its abort flag, every workgroup leaves, and pccl_hip_graph_status
- * returns PCCL_ERR_GRAPH after restoring the graph's pristine state. */
+ * returns PCCL_ERR_GRAPH after restoring the graph's pristine state.  Takes effect
+ * with the next pccl_hip_graph_run (a run recorded by stream capture keeps the limit it
+ * was recorded with). */
 int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls);
 
 int pccl_hip_graph_destroy(void *graph);
