@@ -134,7 +134,7 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // conflict with any op of behind[b] at differing addresses either; when it would, or when the
 // list grows long, the dependency stays whole-op (which also empties what lies behind it).
 // `eligible` (optional, per op): 0 keeps every dependency OF that op whole-op whatever the rule
-// would allow (the caller's judgement of whether it pays, see build_graph).
+// would allow (build_graph: graphs with too many entries for a part-arrival word each).
 std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
                                                  const std::vector<int> &topo,
                                                  const std::vector<unsigned char> *eligible = nullptr) {
