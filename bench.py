@@ -197,8 +197,8 @@ def main():
             del full
 
         # ---- 128 MiB variants: bf16 8->1 and fp16 8->2 ------------------------------------
+        c3 = 1 << 26
         if want("nvls"):
-            c3 = 1 << 26
             t = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [x[:c3] for x in ins], [out[:c3]], c3, stream), 30, 5)
             extras["nvls_bf16_8in_1out_128MiB"] = dict(stats(t), GBps_median=gbps(9 * c3 * 2, t[len(t) // 2]))
             ins16 = [randn(torch, c3, "f16") for _ in range(8)]

@@ -26,6 +26,65 @@ struct AccLaunch {
   long count;
 };
 
+// One pack per lane with a compile-time number of destinations: 1 + NOUT loads in flight per
+// lane, then the folds and stores (the destinations are distinct buffers by contract, so
+// nothing written here is read here).  With the count a run-time bound on loops over an array
+// of packs the compiler carried the whole array through every branch for f32 and f64 (240
+// VGPRs, two wavefronts per SIMD: f32 1 -> 7 at 4.6 TB/s where bf16 reached 6.35).
+// How the stores leave matters once the streams are many, and differently for few and for many
+// destinations (128 MiB operands, medians over fresh allocations, all dtypes):
+//   3-4 destinations: every fold first, then the stores in one burst   6.4-6.5 TB/s
+//                     (folds and stores interleaved: 5.9-6.4, by the fold's length)
+//   5-8 destinations: fold and store one destination after the other, with a pause of 128
+//                     clocks (8 destinations: 320) between the stores   6.2-6.5 TB/s
+//                     (no pause: 5.6-5.7 for the short folds of i32 / f32 / f64, 6.1-6.5 for
+//                     the longer ones of bf16 / f16 / f8, whose arithmetic paces them anyway;
+//                     one burst: 5.5-5.8)
+template <class D, class Op, bool ALIGNED, int LD, int ST, int NOUT>
+__device__ __forceinline__ void accumulate_pack(const AccLaunch &p, size_t wg, unsigned int off) {
+  const u32x4 x = load_pack<D, ALIGNED, LD>(p.in + wg, off);
+  u32x4 d[NOUT];
+#pragma unroll
+  for (int j = 0; j < NOUT; ++j)  // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
+    d[j] = j == 0 ? load_pack<D, true, LD>(p.out[0] + wg, off) : load_pack<D, ALIGNED, LD>(p.out[j] + wg, off);
+  if constexpr (NOUT <= 2) {
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) {
+      const u32x4 v[2] = {d[j], x};
+      const u32x4 r = fold_pack<D, Op, 2>(v);
+      if (j == 0) store_pack<D, true, ST>(p.out[0] + wg, off, r);
+      else store_pack<D, ALIGNED, ST>(p.out[j] + wg, off, r);
+    }
+  } else if constexpr (NOUT <= 4) {
+    // every load back, every fold done, then the stores in one burst
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) {
+      const u32x4 v[2] = {d[j], x};
+      d[j] = fold_pack<D, Op, 2>(v);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) {
+      if (j == 0) store_pack<D, true, ST>(p.out[0] + wg, off, d[0]);
+      else store_pack<D, ALIGNED, ST>(p.out[j] + wg, off, d[j]);
+    }
+  } else {
+    // every load back, then fold and store destination after destination, the stores spaced
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) {
+      const u32x4 v[2] = {d[j], x};
+      const u32x4 r = fold_pack<D, Op, 2>(v);
+      if (j == 0) store_pack<D, true, ST>(p.out[0] + wg, off, r);
+      else store_pack<D, ALIGNED, ST>(p.out[j] + wg, off, r);
+      if (j + 1 < NOUT) __builtin_amdgcn_s_sleep(NOUT == 8 ? 5 : 2);
+    }
+  }
+}
+
 // ALIGNED: input and every output 16-byte aligned after the head peel.
 // MEM: cache treatment as for reduce_copy (0 cacheable, 1 streaming, 2 streaming loads and
 // write-through stores).
@@ -41,23 +100,16 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
     // (wave-uniform base, lane offset) addressing: the workgroup's 4 KiB of every stream
     const size_t wg = (size_t)p.head * D::kElemBytes + (size_t)blockIdx.x * (kBlock * 16);
     const unsigned int off = threadIdx.x * 16u;
-    // All loads first, then the stores: the destinations are distinct buffers (checked by the
-    // host; partial overlap is outside the contract), so nothing written here is read here,
-    // and a lane keeps 1 + n_out loads in flight instead of two.
-    const u32x4 x = load_pack<D, ALIGNED, kLd>(p.in + wg, off);
-    u32x4 d[PCCL_MAX_OUTPUTS];
-#pragma unroll
-    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
-      if (j < p.n_out)  // output 0 is 16-byte aligned by the peel; the others only if ALIGNED
-        d[j] = j == 0 ? load_pack<D, true, kLd>(p.out[0] + wg, off) : load_pack<D, ALIGNED, kLd>(p.out[j] + wg, off);
-#pragma unroll
-    for (int j = 0; j < PCCL_MAX_OUTPUTS; ++j)
-      if (j < p.n_out) {
-        const u32x4 v[2] = {d[j], x};
-        const u32x4 r = fold_pack<D, Op, 2>(v);
-        if (j == 0) store_pack<D, true, kSt>(p.out[0] + wg, off, r);
-        else store_pack<D, ALIGNED, kSt>(p.out[j] + wg, off, r);
-      }
+    switch (p.n_out) {
+      case 1: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 1>(p, wg, off); break;
+      case 2: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 2>(p, wg, off); break;
+      case 3: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 3>(p, wg, off); break;
+      case 4: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 4>(p, wg, off); break;
+      case 5: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 5>(p, wg, off); break;
+      case 6: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 6>(p, wg, off); break;
+      case 7: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 7>(p, wg, off); break;
+      default: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 8>(p, wg, off); break;
+    }
   }
   // head and tail elements: the last wavefront of the last workgroup
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x >= kBlock - kWave) {
