@@ -36,7 +36,8 @@ struct AccLaunch {
 //   3-4 destinations: every fold first, then the stores in one burst   6.4-6.5 TB/s
 //                     (folds and stores interleaved: 5.9-6.4, by the fold's length)
 //   5-8 destinations: fold and store one destination after the other, with a pause of 128
-//                     clocks (8 destinations: 320) between the stores   6.2-6.5 TB/s
+//                     clocks (8 destinations: 320; 5-6 destinations of a 1- or 2-byte type,
+//                     whose folds are long: 64) between the stores      6.2-6.5 TB/s
 //                     (no pause: 5.6-5.7 for the short folds of i32 / f32 / f64, 6.1-6.5 for
 //                     the longer ones of bf16 / f16 / f8, whose arithmetic paces them anyway;
 //                     one burst: 5.5-5.8)
@@ -80,7 +81,7 @@ __device__ __forceinline__ void accumulate_pack(const AccLaunch &p, size_t wg, u
       const u32x4 r = fold_pack<D, Op, 2>(v);
       if (j == 0) store_pack<D, true, ST>(p.out[0] + wg, off, r);
       else store_pack<D, ALIGNED, ST>(p.out[j] + wg, off, r);
-      if (j + 1 < NOUT) __builtin_amdgcn_s_sleep(NOUT == 8 ? 5 : 2);
+      if (j + 1 < NOUT) __builtin_amdgcn_s_sleep(NOUT == 8 ? 5 : (D::kElemBytes < 4 && NOUT <= 6) ? 1 : 2);
     }
   }
 }
