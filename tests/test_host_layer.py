@@ -377,3 +377,14 @@ def test_tensor_overload_header_compiles_against_torch(tmp_path):
     for inc in cpp_extension.include_paths():
         cmd += ["-I", inc]
     subprocess.run(cmd + [str(src)], check=True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits with status 2 before
+    touching torch or the GPU."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=60)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
