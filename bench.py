@@ -288,6 +288,40 @@ def main():
                 del rb
             extras["ring_allreduce_one_launch"] = full
 
+            # the same all-reduce as the one-exchange ("direct") schedule a fully connected node
+            # prefers: rank d folds slice d of all 8 inputs in rank order (8 -> 1), then a copy
+            # stores it into the 7 other ranks' outputs; 16 ops, one queue launch.  Beside it the
+            # whole thing as ONE reduce-copy launch with 8 inputs and 8 outputs.
+            direct = {}
+            for per_rank_mib in (1, 8, 32):
+                ir, per_rank = lang.direct_allreduce(8, (per_rank_mib << 20) // 2 // 8, dtype="bf16")
+                low = ir.lower()
+                rb = {"in": [randn(torch, per_rank, "bf16", 1e-2) for _ in range(8)],
+                      "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
+                g = hip.Graph(lang.bind(low, lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+                tf = event_times_us(torch, lambda: g.run(stream), 20, 3)
+                done, total = g.status(stream)
+                assert done == total == len(low)
+                want_sum = rb["in"][0].float()
+                for r in range(1, 8):
+                    want_sum = want_sum + rb["in"][r].float()
+                want_sum = want_sum.to(torch.bfloat16)
+                for r in range(8):
+                    assert torch.equal(rb["out"][r], want_sum), "direct all-reduce differs from the fp32 fold in rank order"
+                    rb["out"][r].zero_()
+                moved = sum((len(o["ins"]) + len(o["outs"])) * o["count"] * 2 for o in low)
+                dkinds = g.dependency_kinds()
+                t1 = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", rb["in"], rb["out"], per_rank, stream), 20, 3)
+                for r in range(8):
+                    assert torch.equal(rb["out"][r], want_sum)
+                direct["8_ranks_x_%d_MiB" % per_rank_mib] = dict(
+                    stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low), algorithmic_bytes=moved,
+                    queue_entries=g.info()["n_tiles"], dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
+                    as_one_launch_8in_8out=dict(stats(t1), GBps_median=gbps(16 * per_rank * 2, t1[len(t1) // 2])))
+                g.destroy()
+                del rb, want_sum
+            extras["direct_allreduce_one_launch"] = direct
+
         # ---- plumbing config: f32 2 -> 1, 4 MiB ---------------------------------------------
         if want("plumbing"):
             a, b = randn(torch, 1 << 20, "f32"), randn(torch, 1 << 20, "f32")
