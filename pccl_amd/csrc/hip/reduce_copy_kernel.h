@@ -21,7 +21,8 @@ struct RcLaunch {
 // the Infinity Cache one pack per lane and one workgroup per 4 KiB of every stream
 // (the hardware dispatcher then walks memory in address order) beats every
 // persistent / grid-stride shape for all n_in; only cache-resident copies and
-// 2-input reductions gain (about 5 %) from 4 packs per lane.
+// 2-input reductions gain (about 5 %) from 4 packs per lane in this, the general kernel
+// (the lean kernel, taken wherever it applies, has one pack per lane throughout).
 __host__ __device__ constexpr int small_unroll_for(int n_in) { return n_in <= 2 ? 4 : 1; }
 
 // MEM: how the launch treats the caches (host-side choice by operand size and shape).
