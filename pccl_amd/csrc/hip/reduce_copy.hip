@@ -125,7 +125,10 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   unsigned lds = 0;
   if (t.lds_bytes >= 0) {
     lds = (unsigned)t.lds_bytes;
-  } else if (big) {
+  } else if (big || (n_in == 2 && n_out == 2 && total_bytes >= (64l << 20))) {
+    // (a ring reduce step, 2 -> 2, gains from its cap of 5 already at 16 MiB per buffer: 7 steps
+    // over distinct 32 MiB chunks 150 -> 146 us, the same buffers again and again at 16 MiB per
+    // buffer 6.5 -> 6.9 TB/s; 2 -> 1, 3 -> 1, 4 -> 1 and 8 -> 1 of that size lose 1-4 % under theirs)
     const int streams = n_in + n_out;
     int wgs = (20 + streams / 2) / streams;
     wgs = std::max(2, std::min(8, wgs));
