@@ -135,6 +135,20 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // list grows long, the dependency stays whole-op (which also empties what lies behind it).
 // `eligible` (optional, per op): 0 keeps every dependency OF that op whole-op whatever the rule
 // would allow (build_graph: graphs with too many entries for a part-arrival word each).
+// Parts of one op that stand together in the order of the entries before the next op of the
+// same dependency level takes its turn (PCCL_HIP_ORDER_BLOCK; 0 = all of them, i.e. op after
+// op).  With op after op the workgroups in flight cover two or three large ops at a time; in
+// blocks they work on every op of the level at once, each through a narrow window.  Measured on
+// 14 independent 32 MiB ring steps (7 reductions 2 -> 2, 7 copies; 256 parts each): op after op
+// 208-210 us, blocks of 8 .. 64 parts 197-198 us (7.1 TB/s), blocks of 128 214 us; ring and direct
+// all-reduces over 8 ranks x 1 .. 64 MiB and the 4096-op schedule (at most 3 parts per op) are
+// unchanged within 1 %.
+int order_block() {
+  int block = 32;
+  if (const char *env = getenv("PCCL_HIP_ORDER_BLOCK")) block = atoi(env);
+  return block > 0 ? block : 1 << 30;
+}
+
 std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
                                                  const std::vector<int> &topo,
                                                  const std::vector<unsigned char> *eligible = nullptr) {
@@ -336,9 +350,9 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
   }
 
-  // global order of the entries: by level; inside a level by where the op's predecessors stand
-  // in the order (the op whose last predecessor comes first comes first), then op id; parts of
-  // an op in sequence.  Workgroups draw tickets in this order and finish their parts at about
+  // global order of the entries: by level; inside a level the ops by where their predecessors
+  // stand in the order (the op whose last predecessor comes first comes first), then op id; the
+  // ops of a level take turns with blocks of order_block() consecutive parts.  Workgroups draw tickets in this order and finish their parts at about
   // the pace at which they drew them, so the entry a workgroup draws next should depend on
   // entries that were drawn early.  With op id alone a ring step of rank 0 (which waits for
   // rank 7's previous step, the LAST op of the level before) stood first in its level: ring
@@ -414,6 +428,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   for (int i = 0; i < n_ops; ++i) n_grouped += parts[i] > kGroupThreshold;
   const size_t off_ready = off;   off = align_up(off + sizeof(HotWord) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_gbase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
+  const size_t off_ebase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_groups = off;  off = align_up(off + sizeof(HotWord) * (size_t)kPartGroups * (size_t)std::max(n_grouped, 1), 256);
   // One word per entry, 64 bytes apart: a word is polled by the workgroup that holds its entry
   // and bumped by others.  Packed 32 to a 128-byte line they cost more than the part-by-part
@@ -466,6 +481,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   C->part_shift = part_shift;
   C->trace = G->trace_on ? G->trace : nullptr;
   C->group_base = (const int *)(dev + off_gbase);
+  C->entry_base = (const int *)(dev + off_ebase);
+  for (int i = 0; i < n_ops; ++i) ((int *)(img + off_ebase))[i] = first_entry[i];
   C->groups = (HotWord *)(dev + off_groups);
   C->ready = (HotWord *)(dev + off_ready);
   {
@@ -490,10 +507,17 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   std::vector<std::vector<unsigned long long>> qe(kQueues);
   {
     long long t = 0;
-    for (int idx = 0; idx < n_ops; ++idx) {
-      const int i = by_level[idx];
-      for (int p = 0; p < parts[i]; ++p, ++t)
-        qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32));
+    const int block = order_block();
+    for (int lo = 0; lo < n_ops;) {
+      int hi = lo, most = 0;
+      while (hi < n_ops && level[by_level[hi]] == level[by_level[lo]]) most = std::max(most, parts[by_level[hi++]]);
+      for (int first = 0; first < most; first += block)
+        for (int idx = lo; idx < hi; ++idx) {
+          const int i = by_level[idx];
+          for (int p = first; p < std::min(first + block, parts[i]); ++p, ++t)
+            qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32));
+        }
+      lo = hi;
     }
   }
   {

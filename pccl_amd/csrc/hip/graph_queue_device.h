@@ -38,6 +38,7 @@ struct GraphControl {
   const int *succ;                        // all successor uid lists, back to back
   HotWord *hot;                           // kHot* words, see below
   const int *group_base;                  // per op: first of its kPartGroups words in `groups`, or -1
+  const int *entry_base;                  // per op: number of its part 0 (parts of an op are numbered in sequence)
   HotWord *groups;                        // part counters of the ops that count in groups, see finish_part
   HotWord *ready;                         // per op: dependencies that have arrived in this run
   unsigned long long *trace;              // null, or 4 words per queue entry (see kTrace*)
@@ -428,7 +429,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         // that word's only reader and clears it for the next run.
         const unsigned int w12 = *word12(hc);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
-        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + (entry_index << g.part_shift) : nullptr;
+        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + ((size_t)(g.entry_base[uid] + (int)(e >> 32)) << g.part_shift) : nullptr;
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;

@@ -60,6 +60,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_UNROLL");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_TILE_BYTES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PART_DEPS");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_ORDER_BLOCK");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;

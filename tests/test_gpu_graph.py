@@ -620,3 +620,52 @@ def test_rebind_refuses_a_move_that_breaks_element_alignment(hip, oracle):
     H.assert_bits_equal(spare.download()[1:], oracle.reduce("f64", "sum", [a, b]), "after the good rebind")
     assert spare.guards_intact()
     g.destroy()
+
+
+@pytest.mark.parametrize("block", ["1", "3", "32", "0"])
+def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, block):
+    """Three chains of two many-part ops each (the second reads and overwrites what the first
+    wrote, part by part) plus a single-part op: whatever the number of consecutive parts an op
+    contributes to the queue order before the next op of its level takes its turn, the bits are
+    those of the ops executed one after the other, and the order recorded by the timeline is
+    the blocked one."""
+    import torch
+    monkeypatch.setenv("PCCL_HIP_ORDER_BLOCK", block)
+    counts = [700 * 1000 + 3, 300 * 1000, 1000 * 1000 + 11]
+    ops, want, outs = [], [], []
+    for c, count in enumerate(counts):
+        a, b = H.gen("bf16", count, 120 + c, 0), H.gen("bf16", count, 120 + c, 1)
+        da, db = H.DevBuf(torch, "bf16", count, 0, src=a), H.DevBuf(torch, "bf16", count, 0, src=b)
+        dt = H.DevBuf(torch, "bf16", count, 0)
+        outs.append((da, db, dt))
+        ops.append(dict(dtype="bf16", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]))
+        t = oracle.reduce("bf16", "sum", [a, b])
+        want.append(oracle.reduce("bf16", "max", [t, b]))
+    for c, count in enumerate(counts):
+        da, db, dt = outs[c]
+        ops.append(dict(dtype="bf16", compute="max", ins=[dt.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[c]))
+    small = H.gen("bf16", 100, 130, 0)
+    ds, dso = H.DevBuf(torch, "bf16", 100, 0, src=small), H.DevBuf(torch, "bf16", 100, 0)
+    ops.append(dict(dtype="bf16", compute="sum", ins=[ds.ptr], outs=[dso.ptr], count=100, deps=[]))
+    g = hip.Graph(ops, tile_bytes=16 << 10)
+    g.trace(True)
+    for _ in range(3):  # the graph re-arms itself, part words included
+        _run_and_check(torch, hip, g, len(ops))
+        for c in range(len(counts)):
+            H.assert_bits_equal(outs[c][2].download(), want[c], "chain %d, block %s" % (c, block))
+        H.assert_bits_equal(dso.download(), small, "single-part op")
+    uid, part, ready, done = _timeline(torch, g)
+    # level 0 holds ops 0, 1, 2 and 6, level 1 ops 3, 4, 5; inside a level the ops take turns
+    # with `block` consecutive parts each
+    n_parts = {u: int(part[uid == u].max()) + 1 for u in range(len(ops))}
+    assert all(n_parts[c] == n_parts[3 + c] and n_parts[c] > 8 for c in range(3)) and n_parts[6] == 1
+    b = int(block) or 1 << 30
+    expect = []
+    for level_ops in ((0, 1, 2, 6), (3, 4, 5)):
+        most = max(n_parts[u] for u in level_ops)
+        for first in range(0, most, b):
+            for u in level_ops:
+                expect += [(u, p) for p in range(first, min(first + b, n_parts[u]))]
+    assert list(zip(uid.tolist(), part.tolist())) == expect
+    assert all(d.guards_intact() for trio in outs for d in trio)
+    g.destroy()
