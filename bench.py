@@ -79,6 +79,7 @@ def cpu_baseline(count_sample):
     import numpy as np
     import pccl_oracle as orc
     cores = min(16, os.cpu_count() or 1)
+    t_begin = time.perf_counter()
     ins = [np.random.default_rng(k).integers(0x3c00, 0x4000, size=count_sample, dtype=np.uint16) for k in range(8)]
     out = np.empty(count_sample, dtype=np.uint16)
     nbytes = 9 * count_sample * 2
@@ -110,8 +111,10 @@ def cpu_baseline(count_sample):
             r["GBps_%d_thread%s" % (threads, "" if threads == 1 else "s")] = round(nb / min(ts) / 1e9, 2)
         other[name] = r
     return {"value": round(best[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "bf16 8->1 sum, %d elements per buffer (1/%d of the headline buffers), best of 5; "
-                      "single thread: %.2f GB/s" % (count_sample, (1 << 27) // count_sample, best[1]),
+            "sample": "bf16 8->1 sum, %d elements per buffer (%s), best of 5 (this leg took %.0f s); "
+                      "single thread: %.2f GB/s" % (count_sample, "the whole headline step" if count_sample == 1 << 27 else
+                                                    "1/%d of the headline buffers" % ((1 << 27) // count_sample),
+                                                    time.perf_counter() - t_begin, best[1]),
             "other_shapes": other, "host_cpus_visible": os.cpu_count()}
 
 
@@ -399,7 +402,7 @@ def main():
         "device": info,
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(1 << 24)
+        result["cpu_baseline"] = cpu_baseline(1 << 27)
     if extras:
         result["extras"] = extras
     print(json.dumps(result))
