@@ -381,6 +381,26 @@ def main():
                 "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med)),
                 "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
                 "algorithmic_bytes": sched_bytes}
+            # the same schedule the way the reference's host code would drive it: written to a
+            # schedule file, registered by name, executed on an input / output tensor pair
+            # (Engine::regOp / exeOp; every exeOp binds the tensors and launches once)
+            import tempfile
+            from pccl_amd import engine
+            with tempfile.TemporaryDirectory() as tmp:
+                path = os.path.join(tmp, "small_message.sched")
+                ir.save(path, per_rank)
+                eng = engine.Engine(0, 1)
+                eng.initEngine()
+                eng.regOp("small_message", path)
+                x = torch.cat(bufs["in"])
+                y = torch.zeros(8 * per_rank, dtype=torch.bfloat16, device="cuda")
+                te = event_times_us(torch, lambda: eng.exeOp("small_message", x, y, stream), 30, 5)
+                eng.waitOp("small_message", stream)
+                for r in range(8):
+                    assert torch.equal(y[r * per_rank:(r + 1) * per_rank], bufs["out"][r]), "engine result differs from the bound graph's"
+                extras["schedule_4096_ops"]["via_engine_exeOp"] = dict(stats(te), us_per_op=round(te[len(te) // 2] / len(low), 4))
+                eng.close()
+                del x, y
             if want("schedule_launches"):  # the same ops as one launch each ("all" includes it)
                 t2 = event_times_us(torch, individually, 5, 1)
                 extras["schedule_4096_ops"]["as_4096_launches"] = dict(stats(t2), us_per_op=round(t2[len(t2) // 2] / len(low), 4))
