@@ -629,11 +629,15 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   {
     std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
     memcpy(&control, G->image.data(), sizeof(control));
-    ++G->runs;
   }
   hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run launch failed: %s", hipGetErrorString(e));
+  {
+    // counted only once the launch is in: the device's run word moves on per executed launch
+    std::lock_guard<std::mutex> lock(G->mu);
+    ++G->runs;
+  }
   return PCCL_OK;
 }
 
@@ -741,8 +745,19 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.trace_on = G->trace_on;
     fresh.spin_limit = G->spin_limit;
     char *old_dev = G->dev;
-    const int rc = build_graph(&fresh, G->runs + 1u, G->dev, G->arena_bytes);
+    // The run number goes on from where the DEVICE stands, not from the count of graph_run
+    // calls: every replay of a recorded launch has moved the device's word on as well, and a
+    // word set back would let the signal values that earlier replays left behind satisfy the
+    // waits of the next run before its data exists.
+    unsigned int run_word = G->runs + 1u;
+    {
+      const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
+      PCCL_HIP_CHECK(hipMemcpy(&run_word, G->dev + off_hot + sizeof(HotWord) * kHotRun, sizeof(run_word),
+                               hipMemcpyDeviceToHost));
+    }
+    const int rc = build_graph(&fresh, run_word, G->dev, G->arena_bytes);
     if (rc != PCCL_OK) return rc;
+    G->runs = run_word - 1u;  // pccl_hip_graph_next_signal_base follows the device from here
     G->dev = fresh.dev;
     G->arena_bytes = fresh.arena_bytes;
     G->image.swap(fresh.image);

@@ -125,3 +125,58 @@ def test_recorded_queue_run_survives_a_rebind_that_changes_aliasing(hip, oracle)
         H.assert_bits_equal(dA.download()[shift:], u, "u inside a's buffer, replay %d" % it)
     assert g.status(torch.cuda.current_stream().cuda_stream) == (2, 2)
     g.destroy()
+
+
+def test_run_number_survives_a_rebuilding_rebind_after_replays(hip, oracle):
+    """op0: t = a + b; NOTIFY; GET_NOTIFIED; op3: u = t + c (ordered after op0 only through the
+    signal word); op4: v = u + d.  Recorded once and replayed three times, so the device's run
+    number is ahead of the count of graph_run calls.  Moving v onto t (shifted) makes the edge
+    op3 -> op4 whole-op, which rebuilds the arena: the rebuilt arena must go on from the device's
+    run number.  Were it set back, the signal value left by an earlier replay would satisfy the
+    wait at once and op3 would read t before op0 has written it."""
+    import torch
+    count, shift = 1500 * 1000, 64
+    a, b, c, d = (H.gen("f32", count, 411, k) for k in range(4))
+    da, db, dc, dd = (H.DevBuf(torch, "f32", count, 0, src=x) for x in (a, b, c, d))
+    dT = H.DevBuf(torch, "f32", count + shift, 0)
+    du, dv = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    sig = torch.zeros(4, dtype=torch.int32, device="cuda")
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dT.ptr], count=count, deps=[]),
+           dict(primitive=2, signal=sig.data_ptr(), value=1, deps=[0]),
+           dict(primitive=3, signal=sig.data_ptr(), value=1, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[dT.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[2]),
+           dict(dtype="f32", compute="sum", ins=[du.ptr, dd.ptr], outs=[dv.ptr], count=count, deps=[3])]
+    g = hip.Graph(ops)
+    assert g.dependency_kinds() == [0, 0, 1]
+    graph = _capture(torch, lambda stream: g.run(stream))
+    stream = torch.cuda.current_stream().cuda_stream
+    t = oracle.reduce("f32", "sum", [a, b])
+    u = oracle.reduce("f32", "sum", [t, c])
+    v = oracle.reduce("f32", "sum", [u, d])
+    words = []
+    for it in range(3):
+        for buf in (dT, du, dv):
+            buf.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        H.assert_bits_equal(dv.download(), v, "replay %d before the rebind" % it)
+        words.append(int(sig[0].item()) & 0xffffffff)
+    assert [y - x for x, y in zip(words, words[1:])] == [1 << 16, 1 << 16]
+    g.rebind(dv.ptr, dT.ptr + 4 * shift, 4 * count, stream)   # v now overwrites what op3 reads, shifted
+    assert g.dependency_kinds() == [0, 0, 0]
+    # the host's idea of the next base follows the device from here (it counts graph_run calls, not replays)
+    assert g.next_signal_base() == words[-1] - 1 + (1 << 16)
+    for it in range(2):
+        dT.view().fill_(0xFF)
+        du.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert g.status(stream) == (5, 5)
+        H.assert_bits_equal(du.download(), u, "u, replay %d after the rebind" % it)
+        H.assert_bits_equal(dT.download()[shift:], v, "v inside t's buffer, replay %d after the rebind" % it)
+        words.append(int(sig[0].item()) & 0xffffffff)
+    # the run number went on from where the device stood
+    assert [y - x for x, y in zip(words, words[1:])] == [1 << 16] * 4
+    g.destroy()
