@@ -1,5 +1,6 @@
 #include "engine.h"
 
+#include <algorithm>
 #include <stdexcept>
 
 #include "device_plugin.h"
@@ -86,13 +87,26 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
     const DataType dt = TypeRegistry::getTypeId(s.dtype);
     const ComputeType compute = TypeRegistry::getTypeId(s.compute);
     const PrimitiveType copy = TypeRegistry::getTypeId("copy"), reduce = TypeRegistry::getTypeId("reduce");
-    auto resolve = [&](const ScheduleOperand &x, long count) -> void * {
-      if (x.buffer == "ws") {
-        const long per_device = ws_bytes / s.devices / es;
-        if (!ws || x.offset + count > per_device)
-          throw std::runtime_error("Engine::exeOp(): workspace operand does not fit the device workspace");
-        return ws + ((long)x.device * per_device + x.offset) * es;
+    // "ws" operands live in per-device regions of the workspace, each as large as the schedule needs,
+    // laid out by the executor (the hip executor places them by the memory-channel rule of its allocator)
+    long ws_need = 0;
+    for (const ScheduleOp &o : s.ops) {
+      if (o.isSignal()) continue;
+      for (const auto &x : o.srcs) if (x.buffer == "ws") ws_need = std::max(ws_need, (x.offset + o.count) * es);
+      for (const auto &x : o.dsts) if (x.buffer == "ws") ws_need = std::max(ws_need, (x.offset + o.count) * es);
+    }
+    std::vector<long> ws_region;
+    if (ws_need > 0) {
+      if (!ws) throw std::runtime_error("Engine::exeOp(): the schedule uses the workspace, but no device has one");
+      try {
+        ws_region = op->executor->carveWorkspace(ws, ws_bytes, s.devices, ws_need);
+      } catch (const std::exception &e) {
+        throw std::runtime_error(std::string("Engine::exeOp(): workspace operand does not fit the device workspace: ") + e.what());
       }
+    }
+    auto resolve = [&](const ScheduleOperand &x, long count) -> void * {
+      (void)count;
+      if (x.buffer == "ws") return ws + ws_region[(size_t)x.device] + x.offset * es;
       const char *base = x.buffer == "in" ? static_cast<const char *>(input) : static_cast<char *>(output);
       return const_cast<char *>(base) + ((long)x.device * s.elems_per_device + x.offset) * es;
     };

@@ -41,6 +41,12 @@ public:
   virtual void rebindGraph(void *graph, const void *old_base, const void *new_base, long nbytes, void *stream) = 0;
   virtual const GraphBufferLayout *deviceLayout(void *graph) = 0;
   virtual void destroyGraph(void *graph) = 0;
+
+  // Byte offsets of n regions of nbytes_each inside [base, base + capacity): how the executor wants a
+  // workspace divided among the devices of a schedule (the role of BufferManager::assignBuffer,
+  // include/base/chunk.h:48-53).  Throws std::runtime_error when they do not fit.
+  // Default: back to back.
+  virtual std::vector<long> carveWorkspace(const void *base, long capacity, int n, long nbytes_each);
 };
 
 std::shared_ptr<ExecutorBase> getExecutor(ExecutorType type);

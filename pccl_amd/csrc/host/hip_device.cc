@@ -92,6 +92,15 @@ std::shared_ptr<ExecutorBase> getExecutor(ExecutorType type) {
   return it->second;
 }
 
+std::vector<long> ExecutorBase::carveWorkspace(const void *, long capacity, int n, long nbytes_each) {
+  if (n < 1 || nbytes_each <= 0 || (long)n * nbytes_each > capacity)
+    throw std::runtime_error("carveWorkspace(): " + std::to_string(n) + " regions of " + std::to_string(nbytes_each) +
+                             " bytes do not fit " + std::to_string(capacity) + " bytes");
+  std::vector<long> offsets((size_t)n);
+  for (int k = 0; k < n; ++k) offsets[(size_t)k] = (long)k * nbytes_each;
+  return offsets;
+}
+
 void regExecutor(ExecutorType type, std::shared_ptr<ExecutorBase> executor) {
   ExecTable &t = exec_table();
   std::lock_guard<std::mutex> lock(t.mu);
@@ -206,6 +215,13 @@ const GraphBufferLayout *HipExecutor::deviceLayout(void *graph) {
   const int rc = pccl_hip_graph_info(graph, &lay, nullptr, nullptr);
   if (rc != PCCL_OK) raise("pccl_hip_graph_info", rc);
   return static_cast<const GraphBufferLayout *>(lay);
+}
+
+std::vector<long> HipExecutor::carveWorkspace(const void *base, long capacity, int n, long nbytes_each) {
+  std::vector<long> offsets((size_t)std::max(n, 0));
+  const int rc = pccl_hip_carve(base, capacity, n, nbytes_each, offsets.data());
+  if (rc != PCCL_OK) raise("pccl_hip_carve", rc);
+  return offsets;
 }
 
 void HipExecutor::destroyGraph(void *graph) {

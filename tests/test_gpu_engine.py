@@ -213,3 +213,39 @@ def test_python_emitted_collectives(E, eng, oracle, tmp_path, which):
     eng.exeOp(which, d_in, d_out)
     eng.waitOp(which)
     H.assert_bits_equal(d_out.cpu().numpy().view(np.uint16), want, which)
+
+
+def test_schedule_staging_through_the_workspace(E, eng, oracle, tmp_path):
+    """Operands named "ws" live in per-device regions of the engine's workspace, laid out by the
+    executor (placed by the allocator's memory-channel rule): ws[r] = in[r] + in[r+1]; out[r] = ws[r]."""
+    import torch
+    W, n = 4, 3 * 1000 * 1000 + 7      # 12 MB per region: large enough for the regions to be placed
+    lines = ["pccl-schedule 1", "name staged", "dtype f32", "compute sum", "devices %d" % W,
+             "elems_per_device %d" % n, "ops %d" % (2 * W)]
+    for r in range(W):
+        lines.append("op %d REDUCE %d deps 0 src 2 in %d 0 in %d 0 dst 1 ws %d 0" % (r, n, r, (r + 1) % W, r))
+    for r in range(W):
+        lines.append("op %d COPY %d deps 1 %d src 1 ws %d 0 dst 1 out %d 0" % (W + r, n, r, r, r))
+    p = tmp_path / "staged.sched"
+    p.write_text("\n".join(lines) + "\n")
+    eng.regOp("staged", str(p))
+    host_in = H.gen("f32", W * n, 75, 0)
+    d_in, d_out = _to_dev(torch, host_in), torch.zeros(W * n * 4, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    eng.exeOp("staged", d_in, d_out, stream)
+    eng.waitOp("staged", stream)
+    got = d_out.cpu().numpy().view(np.float32)
+    for r in range(W):
+        want = oracle.reduce("f32", "sum", [host_in[r * n:(r + 1) * n], host_in[((r + 1) % W) * n:((r + 1) % W + 1) * n]])
+        H.assert_bits_equal(got[r * n:(r + 1) * n], want, "device %d" % r)
+    # a region that cannot fit the 256 MiB workspace is refused
+    big = (1 << 28) // 4 // W + 4096
+    lines[5] = "elems_per_device %d" % big
+    lines[7:] = ["op %d REDUCE %d deps 0 src 2 in %d 0 in %d 0 dst 1 ws %d 0" % (r, big, r, (r + 1) % W, r) for r in range(W)] + \
+                ["op %d COPY %d deps 1 %d src 1 ws %d 0 dst 1 out %d 0" % (W + r, big, r, r, r) for r in range(W)]
+    p2 = tmp_path / "too_big.sched"
+    p2.write_text("\n".join(lines) + "\n")
+    eng.regOp("too_big", str(p2))
+    x = torch.zeros(W * big * 4, dtype=torch.uint8, device="cuda")
+    with pytest.raises(E.EngineError):
+        eng.exeOp("too_big", x, x.clone(), stream)
