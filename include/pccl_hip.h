@@ -251,6 +251,24 @@ int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
  * was recorded with). */
 int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls);
 
+/* pccl_hip_graph_create + pccl_hip_graph_run in one call that allocates NO device memory: the
+ * graph's device state (headers, payloads, counters, ready queues: what graph_create puts into a
+ * hipMalloc'ed arena) goes into a fixed array inside the library's code object, of which every GPU
+ * holds one copy of PCCL_HIP_STATIC_ARENA_BYTES until the process ends.  No counterpart in the
+ * reference; it is for callers that cannot allocate: tight serving loops and harnesses that forbid
+ * hipMalloc.  The call uploads the state behind earlier work on `stream` and launches the drain kernel
+ * there.  A call with the very same ops as the last one on this GPU skips the upload (the state re-arms
+ * itself).  A graph that needs more than the array holds (about 4,500 ops of three parts each) is
+ * refused with PCCL_ERR_NOMEM and nothing is launched.  completed / total both NULL: returns without
+ * waiting.  Otherwise waits for `stream` and reports the two counters of operator.h:32-33
+ * (PCCL_ERR_GRAPH if the drain gave up).  All calls on one GPU share the one array: a call waits for
+ * the previous one's stream before it rewrites the state, and calls issued at the same time from
+ * several threads or onto streams that overlap race.  Not meant to be recorded by stream capture (the
+ * upload reads host memory). */
+#define PCCL_HIP_STATIC_ARENA_BYTES (8u << 20)
+int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_bytes, void *stream,
+                              unsigned int *completed, unsigned int *total);
+
 int pccl_hip_graph_destroy(void *graph);
 
 /* ---- errors ---------------------------------------------------------------- */

@@ -195,7 +195,16 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
 // layout depends on the ops and their parts only, not on their addresses, so the arena of the
 // same ops at other addresses fits exactly; a launch recorded by stream capture keeps
 // pointing at it).
-int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t reuse_bytes = 0) {
+// `fixed`: build into this memory, which the caller owns and which is not allocated here (the
+// arena must fit its capacity), and upload behind earlier work on its stream.
+struct FixedArena {
+  char *ptr;
+  size_t capacity;
+  hipStream_t stream;
+};
+
+int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t reuse_bytes = 0,
+                const FixedArena *fixed = nullptr) {
   const pccl_op_desc *ops = G->descs.data();
   const int n_ops = (int)G->descs.size();
   long tile_bytes = G->tile_bytes;
@@ -453,7 +462,12 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->dev = nullptr;
   G->arena_bytes = arena_bytes;
   hipError_t e = hipSuccess;
-  if (reuse && reuse_bytes == arena_bytes) G->dev = reuse;
+  if (fixed) {
+    if (arena_bytes > fixed->capacity)
+      return fail(PCCL_ERR_NOMEM, "the op graph needs %zu bytes of device state; the static arena holds %zu "
+                                  "(%d ops, %lld queue entries)", arena_bytes, fixed->capacity, n_ops, tiles);
+    G->dev = fixed->ptr;
+  } else if (reuse && reuse_bytes == arena_bytes) G->dev = reuse;
   else e = hipMalloc((void **)&G->dev, arena_bytes);
   if (e != hipSuccess) {
     (void)hipGetLastError();
@@ -577,16 +591,37 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // never more workgroups than entries
   G->n_wg = (int)std::max<long long>(1, std::min<long long>(tiles, cap));
 
-  e = hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
+  e = fixed ? hipMemcpyAsync(dev, img, arena_bytes, hipMemcpyHostToDevice, fixed->stream)
+            : hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) {
-    if (dev != reuse) (void)hipFree(dev);
+    if (dev != reuse && !fixed) (void)hipFree(dev);
     G->dev = nullptr;
     return fail(PCCL_ERR_HIP, "uploading the op graph: %s", hipGetErrorString(e));
   }
   return PCCL_OK;
 }
 
+// ---- the arena of pccl_hip_graph_run_static ---------------------------------------
+// Device state of ONE op graph per GPU in a file-scope device array, for callers that cannot
+// allocate device memory.  On the host the array's name is only a handle: its address on a
+// device comes from hipGetSymbolAddress (once per device, that device current) and only that
+// address is ever handed to a kernel or a copy.
+constexpr size_t kStaticArenaBytes = PCCL_HIP_STATIC_ARENA_BYTES;
+constexpr int kMaxStaticDevices = 64;
+struct StaticArena {
+  char *ptr = nullptr;          // this device's copy of g_static_arena
+  Graph *graph = nullptr;       // host side of what the array holds now
+  bool valid = false;           // ... and it is complete and was not left behind by an aborted run
+  bool used = false;
+  hipStream_t last_stream = nullptr;
+  unsigned int runs = 0;        // launches on this array so far (signal values go on from here)
+};
+std::mutex g_static_mutex;
+StaticArena g_static[kMaxStaticDevices];
+
 }  // namespace
+
+static __device__ __align__(256) unsigned char g_static_arena[PCCL_HIP_STATIC_ARENA_BYTES];
 
 extern "C" {
 
@@ -859,6 +894,86 @@ int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls) {
   G->spin_limit = polls;
   ((GraphControl *)G->image.data())->spin_limit = polls;
   PCCL_HIP_CHECK(hipMemcpy(G->dev + offsetof(GraphControl, spin_limit), &polls, sizeof(polls), hipMemcpyHostToDevice));
+  return PCCL_OK;
+}
+
+int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_bytes, void *stream,
+                              unsigned int *completed, unsigned int *total) {
+  pccl_host::clear_error();
+  if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_run_static: bad op array");
+  if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_run_static: tile_bytes %ld < 0", tile_bytes);
+  if (completed) *completed = 0;
+  if (total) *total = (unsigned int)n_ops;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(PCCL_ERR_NO_DEVICE, "no current device");
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (dev < 0 || dev >= kMaxStaticDevices) return fail(PCCL_ERR_UNSUPPORTED, "graph_run_static: device index %d", dev);
+  StaticArena &S = g_static[dev];
+  if (!S.ptr) {
+    // set-up, once per device, with that device current: where this device keeps its copy of the array
+    void *p = nullptr;
+    PCCL_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_arena)));
+    S.ptr = (char *)p;
+    S.graph = new Graph();
+  }
+  // own copy of the ops and their dependency lists
+  size_t n_deps = 0;
+  for (int i = 0; i < n_ops; ++i) {
+    if (ops[i].n_deps < 0 || (ops[i].n_deps > 0 && !ops[i].deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
+    n_deps += (size_t)ops[i].n_deps;
+  }
+  std::vector<int> deps;
+  deps.reserve(n_deps);
+  for (int i = 0; i < n_ops; ++i) deps.insert(deps.end(), ops[i].deps, ops[i].deps + ops[i].n_deps);
+  Graph *G = S.graph;
+  auto same_ops = [&] {
+    if (!S.valid || (int)G->descs.size() != n_ops || G->tile_bytes != tile_bytes || G->deps_store != deps) return false;
+    for (int i = 0; i < n_ops; ++i) {
+      const pccl_op_desc &a = G->descs[i], &b = ops[i];
+      if (a.op_uid != b.op_uid || a.primitive != b.primitive || a.dtype != b.dtype || a.compute != b.compute ||
+          a.n_in != b.n_in || a.n_out != b.n_out || a.count != b.count || a.n_deps != b.n_deps ||
+          memcmp(a.ins, b.ins, sizeof(void *) * b.n_in) || memcmp(a.outs, b.outs, sizeof(void *) * b.n_out))
+        return false;
+    }
+    return true;
+  };
+  if (!same_ops()) {
+    // The array still serves the previous call, and the host image that call was uploaded from is
+    // about to be rewritten: that call's work ends first.
+    if (S.used) PCCL_HIP_CHECK(hipStreamSynchronize(S.last_stream));
+    S.valid = false;
+    G->tile_bytes = tile_bytes;
+    G->descs.assign(ops, ops + n_ops);
+    G->deps_store.swap(deps);
+    for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) G->descs[i].deps = G->deps_store.data() + at;
+    const FixedArena fixed{S.ptr, kStaticArenaBytes, (hipStream_t)stream};
+    const int rc = build_graph(G, S.runs + 1u, nullptr, 0, &fixed);  // the whole image, zeros included, goes up: nothing of the last call's state survives
+    if (rc != PCCL_OK) return rc;
+    S.valid = true;
+  }
+  S.used = true;
+  S.last_stream = (hipStream_t)stream;
+  if (G->total_tiles > 0) {
+    GraphControl control;
+    memcpy(&control, G->image.data(), sizeof(control));
+    hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run_static launch failed: %s", hipGetErrorString(e));
+    ++S.runs;
+  }
+  if (!completed && !total) return PCCL_OK;
+  PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  if (G->total_tiles == 0) return PCCL_OK;
+  const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
+  HotWord hot[kHotWords];
+  PCCL_HIP_CHECK(hipMemcpy(hot, G->dev + off_hot, sizeof(hot), hipMemcpyDeviceToHost));
+  if (completed) *completed = hot[kHotCompleted].value;
+  if (total) *total = hot[kHotTotal].value;
+  if (hot[kHotAbort].value) {
+    S.valid = false;  // the next call uploads a fresh image
+    return fail(PCCL_ERR_GRAPH, "drain gave up: an op's dependencies were not satisfied within the spin limit "
+                                "(%u of %u ops had completed)", hot[kHotCompleted].value, hot[kHotTotal].value);
+  }
   return PCCL_OK;
 }
 

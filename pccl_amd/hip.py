@@ -78,6 +78,8 @@ def lib():
         L.pccl_hip_set_occupancy_lds.argtypes = [ci]
         L.pccl_hip_set_unroll.argtypes = [ci]
         L.pccl_hip_graph_create.argtypes = [ctypes.POINTER(OpDesc), ci, cl, ctypes.POINTER(vp)]
+        L.pccl_hip_graph_run_static.argtypes = [ctypes.POINTER(OpDesc), ci, cl, vp, ctypes.POINTER(ctypes.c_uint),
+                                                ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_run.argtypes = [vp, vp]
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
@@ -240,6 +242,24 @@ def classify_dependencies(ops, parts):
     pa = (ctypes.c_int * max(len(ops), 1))(*parts)
     _check(lib().pccl_hip_classify_dependencies(arr, len(ops), pa, kinds))
     return list(kinds)[:n_deps]
+
+
+STATIC_ARENA_BYTES = 8 << 20
+
+
+def graph_run_static(ops, stream=None, tile_bytes=0, wait=True):
+    """Runs a DAG of ops with its device state in the library's fixed per-GPU array: no device
+    allocation (pccl_hip_graph_run_static).  wait=True: waits for `stream` and returns
+    (completed, total); wait=False: returns None once the launch is enqueued."""
+    arr, keep = _op_descs(ops)
+    if not wait:
+        _check(lib().pccl_hip_graph_run_static(arr, len(ops), tile_bytes, ctypes.c_void_p(_addr(stream)), None, None))
+        return None
+    c, t = ctypes.c_uint(0), ctypes.c_uint(0)
+    _check(lib().pccl_hip_graph_run_static(arr, len(ops), tile_bytes, ctypes.c_void_p(_addr(stream)), ctypes.byref(c),
+                                           ctypes.byref(t)))
+    del keep
+    return c.value, t.value
 
 
 class Graph:
