@@ -274,25 +274,72 @@ def main():
             ring_bytes = 7 * 4 * ce * 2 + 7 * 2 * ce * 2
             tr = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[0], grad[:ce]], [result[:ce], send], ce, stream), 50, 5)
             tc = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [peers[1]], [result[ce:2 * ce]], ce, stream), 50, 5)
-            # the same 14 steps as ONE persistent launch of the queue executor: independent, and with
-            # each step depending on the one before (what arrival order imposes in a real ring)
+            # the same 14 steps as ONE persistent launch of the queue executor: ordered only by the
+            # hazards the buffers impose (every reduce step writes the one send buffer; copy step s
+            # overwrites the output chunk that reduce step s - 1 wrote), and with each step
+            # depending on the one before
             def ring_ops(chain):
                 o = []
                 for s in range(W - 1):
                     c = (W - 1 - s) % W
                     o.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]],
-                                  outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(o) - 1] if chain and o else []))
+                                  outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(o) - 1] if o else []))
                 for s in range(W - 1):
                     c = (W - s) % W
-                    o.append(dict(dtype="bf16", compute="sum", ins=[peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce,
-                                  deps=[len(o) - 1] if chain and o else []))
+                    deps = [len(o) - 1] if chain else ([s - 1] if s else [])
+                    o.append(dict(dtype="bf16", compute="sum", ins=[peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce, deps=deps))
                 return o
             tq = {}
+            ring()
+            torch.cuda.synchronize()
+            ref_result = result.clone()
             for chain in (False, True):
                 g = hip.Graph(ring_ops(chain))
+                result.zero_()
                 tq[chain] = event_times_us(torch, lambda: g.run(stream), 20, 3)
+                torch.cuda.synchronize()
+                assert torch.equal(result, ref_result), "ring walk through the queue differs from the 14 launches"
                 g.destroy()
+            # ... and gated the way a rank really is: every step waits for the arrival of its incoming
+            # chunk on a signal word (GET_NOTIFIED), and tells the next rank when its output is there
+            # (NOTIFY).  The peers are not running here, so the host marks every chunk as arrived
+            # before the launch; what orders the steps inside the launch is what would order them on
+            # a rank: the one send buffer that all seven reduce steps write (a dependency from each
+            # reduce step to the next, met part by part).
+            sig = torch.zeros(64, dtype=torch.int32, device="cuda")
+            gated = []
+            prev_reduce = None
+            for s in range(2 * (W - 1)):
+                reduce_phase = s < W - 1
+                g_i = len(gated)
+                gated.append(dict(primitive=hip.GET_NOTIFIED, signal=sig.data_ptr() + 4 * s, value=1, deps=[]))
+                if reduce_phase:
+                    c = (W - 1 - s) % W
+                    gated.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]],
+                                      outs=[result[c * ce:(c + 1) * ce], send], count=ce,
+                                      deps=[g_i] + ([prev_reduce] if prev_reduce is not None else [])))
+                    prev_reduce = len(gated) - 1
+                else:
+                    c = (W - (s - (W - 1))) % W
+                    hazard = [3 * (s - W) + 1] if s > W - 1 else []   # the reduce step that wrote this output chunk
+                    gated.append(dict(dtype="bf16", compute="sum", ins=[peers[s - (W - 1)]], outs=[result[c * ce:(c + 1) * ce]],
+                                      count=ce, deps=[g_i] + hazard))
+                gated.append(dict(primitive=hip.NOTIFY, signal=sig.data_ptr() + 4 * (32 + s), value=1, deps=[len(gated) - 1]))
+            gg = hip.Graph(gated)
+            # arrival words far enough ahead of this run's signal base to satisfy every timed run
+            sig[:32] = ((gg.next_signal_base() + (200 << 16)) & 0x7fffffff)
+            torch.cuda.synchronize()
+            result.zero_()
+            tg = event_times_us(torch, lambda: gg.run(stream), 20, 3)
+            done, total = gg.status(stream)
+            assert done == total == len(gated)
+            assert torch.equal(result, ref_result), "signal-gated ring walk differs from the 14 launches"
+            gkinds = gg.dependency_kinds()
+            gg.destroy()
             extras["ring_allreduce_rank_share"] = {
+                "all_14_steps_one_queue_launch_signal_gated": dict(
+                    stats(tg), GBps_median=gbps(ring_bytes, tg[len(tg) // 2]), ops=len(gated),
+                    dependencies_part_by_part="%d of %d" % (sum(gkinds), len(gkinds))),
                 "all_14_steps": dict(stats(t), GBps_median=gbps(ring_bytes, t[len(t) // 2])),
                 "all_14_steps_one_queue_launch": dict(stats(tq[False]), GBps_median=gbps(ring_bytes, tq[False][len(tq[False]) // 2])),
                 "all_14_steps_one_queue_launch_chained": dict(stats(tq[True]), GBps_median=gbps(ring_bytes, tq[True][len(tq[True]) // 2])),

@@ -180,8 +180,7 @@ typedef struct pccl_op_desc {
  * one ready queue (RingBuffer, :7-17).  Role: Engine::regOp,
  * csrc/engine.cc:102-104.  tile_bytes = bytes of output one workgroup handles
  * per queue entry; it fixes required_executors_.  0 = built-in choice: per dependency
- * level, about 0.8 of a round of parts for the workgroups the device holds (8 KiB to
- * 128 KiB per part). */
+ * level, 16 KiB x (bytes the level writes / 8 MiB)^(2/3), within 8 KiB to 128 KiB per part. */
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
 /* Drains the whole DAG with ONE persistent-kernel launch on `stream`; returns

@@ -43,6 +43,7 @@
 //     raises the abort flag, all workgroups leave, and the host reports
 //     PCCL_ERR_GRAPH instead of hanging.
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -333,23 +334,24 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   }
   // ---- parts ------------------------------------------------------------------
   // A given tile_bytes cuts every op into parts of that size.  The built-in choice works per
-  // dependency level: the parts of one level should be about 0.8 of a round for the resident
-  // workgroups (part = 1.25 x level bytes / workgroups, within 8 KiB .. 128 KiB), so that with
-  // dependencies met part by part every workgroup draws about one part of each level in
-  // turn.  Measured on ring all-reduces of 8 x 1 / 8 / 32 / 64 MiB and on the 4096-op schedule
-  // with fixed part sizes of 16 .. 256 KiB: each has its best time where a level holds 0.7 to
-  // 1.3 rounds (8 x 64 MiB: 32 KiB parts = 2.7 rounds 385 us, 64 KiB = 1.3 rounds 339 us,
-  // 128 KiB = 0.7 rounds 355 us; the schedule: 16 KiB = 2 rounds 222 us, 32 KiB = 1.1 rounds
-  // 172 us, 64 KiB = 0.7 rounds 190 us), and one large op alone in its level fills the chip in
-  // a single round.
+  // dependency level and grows with the bytes the level writes: part = 16 KiB x (level bytes /
+  // 8 MiB)^(2/3), within 8 KiB .. 128 KiB (for the 768 workgroups an MI355X holds of this kernel;
+  // scaled for another count), never more parts per op than workgroups.  That puts a level of 8 MiB
+  // at 0.67 rounds of the resident workgroups, 32 MiB at about one round, 64 MiB at 1.33.  Measured
+  // best part sizes it was fitted to (ring all-reduces over 8 virtual ranks of 1 / 8 / 32 / 64 MiB,
+  // the 4096-op schedule, one rank's 14 ring steps of 32 MiB ordered by their buffer hazards):
+  // levels of 8 MiB 16 KiB (12 KiB +10 %, 20 KiB +10 %), 18 MiB 32 KiB (16 KiB +29 %, 64 KiB +10 %),
+  // 32 MiB 47 KiB, 64 MiB 64-76 KiB (14 ring steps: 96 KiB +8 %, 128 KiB +19 %, 48 KiB +2 %, 32 KiB
+  // +12 %).  An earlier rule aimed every level at 0.8 rounds (parts of 104 KiB for the 14 ring steps):
+  // 227 us against 198-201 us with 64 KiB parts.
   {
     std::vector<long long> level_bytes(n_ops + 1, 0);
     for (int i = 0; i < n_ops; ++i) level_bytes[level[i]] += op_bytes[i];
     for (int i = 0; i < n_ops; ++i) {
       long part_bytes = tile_bytes;
       if (default_tile) {
-        const long long want = level_bytes[level[i]] * 5 / (cap * 4);
-        part_bytes = (long)std::min<long long>(std::max<long long>((want + 4095) / 4096 * 4096, 8 << 10), 128 << 10);
+        const double want = 16384.0 * std::pow((double)level_bytes[level[i]] / (double)(8 << 20), 2.0 / 3.0) * (768.0 / (double)cap);
+        part_bytes = (long)std::min<long long>(std::max<long long>(((long long)want + 4095) / 4096 * 4096, 8 << 10), 128 << 10);
       }
       long p = (op_bytes[i] + part_bytes - 1) / part_bytes;
       if (default_tile) p = std::min<long>(p, (long)cap);
