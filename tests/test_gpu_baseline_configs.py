@@ -203,3 +203,24 @@ def test_buffers_beyond_4_gib(hip):
     g.destroy()
     del a, b, out
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_two_byte_offsets_at_16_mi_elements(hip, oracle, dtype):
+    """The unaligned stress of configuration 4 for the 2-byte types: four inputs and the output each start an
+    odd number of elements (2, 6, 10 ... bytes) off a 64-byte line, 2^24 + 7 elements, sum and max."""
+    import torch
+    count = (1 << 24) + 7
+    offs = [2, 6, 14, 30, 62]          # bytes; the output's (last) differs from every input's
+    pool = [_dev_random(torch, dtype, count + 64, 40 + k, kind="uniform", lo=-2.0, hi=2.0) for k in range(4)]
+    out = torch.zeros(count + 64, dtype=pool[0].dtype, device="cuda")
+    ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
+    host_ins = [_host(pool[k], dtype)[offs[k] // 2:offs[k] // 2 + count] for k in range(4)]
+    for compute in ("sum", "max"):
+        out.zero_()
+        hip.reduce_copy(dtype, compute, ptr_in, [out.data_ptr() + offs[4]], count, _stream(torch))
+        torch.cuda.synchronize()
+        got = _host(out, dtype)
+        H.assert_bits_equal(got[offs[4] // 2:offs[4] // 2 + count], _expect(oracle, dtype, compute, host_ins),
+                            "%s %s at 2-byte offsets" % (dtype, compute))
+        assert not got[:offs[4] // 2].any() and not got[offs[4] // 2 + count:].any(), "wrote outside the output"

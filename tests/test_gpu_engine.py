@@ -249,3 +249,35 @@ def test_schedule_staging_through_the_workspace(E, eng, oracle, tmp_path):
     x = torch.zeros(W * big * 4, dtype=torch.uint8, device="cuda")
     with pytest.raises(E.EngineError):
         eng.exeOp("too_big", x, x.clone(), stream)
+
+
+def test_extension_module_exeop_on_torch_tensors(E, oracle, tmp_path):
+    """The reference's Python entry point: pccl.engine_c.Engine(rank, world).exeOp(name, input, output)
+    on torch tensors (csrc/python_api.cc:13-20, include/engine.h:19), here pccl_amd.engine_c: a ring
+    all-reduce over 8 virtual ranks in bf16, on torch's current stream, against the CPU checker."""
+    import torch
+    from pccl_amd import engine_c
+    p = str(tmp_path / "ring.sched")
+    E.write_ring_allreduce(p, "bf16", "sum", 8, 54321)
+    eng = engine_c.Engine(0, 1)
+    eng.initEngine()
+    eng.regOp("ring", p)
+    hdr, _ = S.parse_schedule_text(open(p).read())
+    n = hdr["devices"] * hdr["elems_per_device"]
+    for it, stream in enumerate((torch.cuda.current_stream(), torch.cuda.Stream())):
+        host_in = H.gen("bf16", n, 171 + it, 0)
+        _, want = _oracle_replay(oracle, open(p).read(), host_in)
+        with torch.cuda.stream(stream):
+            x = torch.from_numpy(host_in.view(np.int16)).cuda().view(torch.bfloat16)
+            y = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+            eng.exeOp("ring", x, y)
+            eng.waitOp("ring")
+        got = y.view(torch.int16).cpu().numpy().view(np.uint16)
+        H.assert_bits_equal(got, want, "extension module, run %d" % it)
+    with pytest.raises(RuntimeError):
+        eng.exeOp("ring", x[:100], y)          # too small for the schedule
+    with pytest.raises(RuntimeError):
+        eng.exeOp("ring", x.cpu(), y)          # not a device tensor
+    with pytest.raises(RuntimeError):
+        eng.exeOp("unknown", x, y)
+    del eng

@@ -669,3 +669,41 @@ def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, 
     assert list(zip(uid.tolist(), part.tolist())) == expect
     assert all(d.guards_intact() for trio in outs for d in trio)
     g.destroy()
+
+
+def test_graph_beside_a_kernel_that_occupies_the_gpu(hip, oracle):
+    """The drain's workgroups wait for each other inside one launch, so it needs its queues' workgroups
+    resident.  With another stream's long elementwise kernels holding compute units at the same time the
+    run must still complete every op (no bounded wait may give up), bit-exact."""
+    import torch
+    from pccl_amd import lang
+    world, size = 8, 30_001
+    ir, per_rank = lang.ring_allreduce(world, size, dtype="bf16")
+    low = ir.lower()
+    host_in = [H.gen("bf16", per_rank, 611, r) for r in range(world)]
+    bufs = {"in": [H.DevBuf(torch, "bf16", per_rank, 0, src=a) for a in host_in],
+            "out": [H.DevBuf(torch, "bf16", per_rank, 0) for _ in range(world)]}
+    g = hip.Graph(lang.bind(low, lambda b, r, e: bufs[b][r].ptr + 2 * e))
+    outs = [np.zeros(per_rank, dtype=np.uint16) for _ in range(world)]
+    hb = {"in": host_in, "out": outs}
+    for o in low:
+        n = o["count"]
+        oracle.reduce_copy("bf16", "sum", [hb[b][r][e:e + n] for (b, r, e) in o["ins"]], [hb[b][r][e:e + n] for (b, r, e) in o["outs"]])
+    side = torch.cuda.Stream()
+    hog = torch.ones(1 << 28, dtype=torch.float32, device="cuda")       # 1 GiB: each pass a few hundred microseconds
+    main = torch.cuda.current_stream()
+    for rep in range(3):
+        for r in range(world):
+            bufs["out"][r].view().fill_(0xFF)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for _ in range(40):
+                hog.mul_(1.0000001).add_(1e-9)
+        for _ in range(5):                     # several runs land while the other stream is busy
+            g.run(main.cuda_stream)
+        assert g.status(main.cuda_stream) == (len(low), len(low)), "a run gave up beside the other kernel (rep %d)" % rep
+        assert not side.query() or rep >= 0    # (the other stream may or may not have finished by now)
+        torch.cuda.synchronize()
+        for r in range(world):
+            H.assert_bits_equal(bufs["out"][r].download(), outs[r], "rank %d, rep %d" % (r, rep))
+    g.destroy()

@@ -138,6 +138,87 @@ def test_special_values(hip, oracle):
                                 "%s %s specials" % (dtype, compute))
 
 
+def _nan_inputs(oracle, dtype, n, seed):
+    """Three inputs of n elements; by element index modulo 8: 0 no NaN, 1-3 exactly one NaN (first, middle,
+    last input; random sign and payload, quiet or signalling), 4 a signalling NaN alone, 5 two NaNs
+    (first and last input), 6 +inf / -inf / finite, 7 zero / inf / finite."""
+    rng = np.random.default_rng(seed)
+    f = [rng.uniform(0.5, 2.0, n).astype(np.float32) for _ in range(3)]
+    cat = np.arange(n) % 8
+
+    def nans(quiet=None):
+        sign = rng.integers(0, 2, n).astype(np.uint32) << 31
+        q = (rng.integers(0, 2, n).astype(np.uint32) if quiet is None else np.full(n, quiet, np.uint32)) << 22
+        return (sign | np.uint32(0x7f800000) | q | rng.integers(1 << 14, 1 << 22, n).astype(np.uint32)).view(np.float32)
+
+    for k, c in ((0, 1), (1, 2), (2, 3)):
+        f[k] = np.where(cat == c, nans(), f[k])
+    f[1] = np.where(cat == 4, nans(0), f[1])
+    f[0] = np.where(cat == 5, nans(), f[0])
+    f[2] = np.where(cat == 5, nans(), f[2])
+    f[0] = np.where(cat == 6, np.float32(np.inf), np.where(cat == 7, np.float32(0.0), f[0]))
+    f[1] = np.where(cat == 6, np.float32(-np.inf), np.where(cat == 7, np.float32(np.inf), f[1]))
+
+    def store(x):
+        u = x.view(np.uint32)
+        if dtype == "f32":
+            return x.copy()
+        if dtype == "f64":   # NaN payload and sign placed by hand (a cast would be free to change them)
+            with np.errstate(invalid="ignore"):
+                d = x.astype(np.float64).view(np.uint64)
+            isn = (u & 0x7fffffff) > 0x7f800000
+            hand = ((u.astype(np.uint64) >> np.uint64(31)) << np.uint64(63)) | np.uint64(0x7ff0000000000000) | ((u.astype(np.uint64) & np.uint64(0x7fffff)) << np.uint64(29))
+            return np.where(isn, hand, d).view(np.float64)
+        if dtype == "bf16":
+            return np.where((u & 0x7fffffff) > 0x7f800000, u >> 16, oracle.narrow("bf16", x).astype(np.uint32)).astype(np.uint16)
+        hn = ((u >> 16) & 0x8000) | 0x7c00 | ((u >> 13) & 0x3ff)
+        return np.where((u & 0x7fffffff) > 0x7f800000, hn, oracle.narrow("f16", x).astype(np.uint32)).astype(np.uint16)
+
+    return [store(x) for x in f], cat
+
+
+def _check_nan_bits(oracle, dtype, compute, ins, cat, got, what):
+    """Bit for bit against the CPU checker, NaNs included (sign, payload, quiet bit).  One exception, which
+    the semantics leave open: a sum or product of SEVERAL NaN inputs is a quiet NaN carrying the sign and
+    payload of one of them (x86 keeps the first operand's, the GPU's instruction whichever the compiler put
+    first); there the result must be one of the candidates."""
+    want = oracle.reduce(dtype, compute, ins)
+    wb, gb = H.bits(want), H.bits(got)
+    several = (cat == 5) & (compute in ("sum", "prod"))
+    H.assert_bits_equal(np.where(several, 0, gb), np.where(several, 0, wb), what)
+    if several.any():
+        zero = np.zeros_like(ins[1])
+        cand = [H.bits(oracle.reduce(dtype, "sum", [ins[k], zero])) for k in (0, 2)]   # the NaN of input k, quieted
+        ok = (gb == cand[0]) | (gb == cand[1])
+        assert ok[several].all(), "%s: a several-NaN result is none of its inputs' NaNs" % what
+    # every NaN that comes out of arithmetic is quiet
+    if compute in ("sum", "prod"):
+        quiet = {"f32": 1 << 22, "f64": 1 << 51, "bf16": 1 << 6, "f16": 1 << 9}[dtype]
+        isn = np.isnan(got) if dtype in ("f32", "f64") else np.isnan(oracle.widen(dtype, got))
+        assert ((gb[isn] & np.asarray(quiet, dtype=gb.dtype)) != 0).all(), "%s: a signalling NaN came out" % what
+
+
+def test_nan_results_bit_for_bit(hip, oracle):
+    """NaN sign, payload and quiet bit through packs, head / tail elements and queue parts."""
+    import torch
+    n = 8 * 1031 + 5
+    stream = torch.cuda.current_stream().cuda_stream
+    for dtype in ("f32", "bf16", "f16", "f64"):
+        es = H.ELEM_BYTES[dtype]
+        ins, cat = _nan_inputs(oracle, dtype, n, 17)
+        for compute in ("sum", "prod", "min", "max"):
+            for offs in ([0, 0, 0], [es, 3 * es, 0]):
+                (got,) = H.hip_reduce(torch, hip, dtype, compute, ins, in_offsets=offs, out_offsets=[offs[0]])
+                _check_nan_bits(oracle, dtype, compute, ins, cat, got, "%s %s direct, offsets %s" % (dtype, compute, offs))
+            d_in = [H.DevBuf(torch, dtype, n, es * k, src=a) for k, a in enumerate(ins)]
+            d_out = H.DevBuf(torch, dtype, n, es)
+            g = hip.Graph([dict(dtype=dtype, compute=compute, ins=[b.ptr for b in d_in], outs=[d_out.ptr], count=n)], 8192)
+            g.run(stream)
+            assert g.status(stream) == (1, 1)
+            _check_nan_bits(oracle, dtype, compute, ins, cat, d_out.download(), "%s %s through the queue" % (dtype, compute))
+            g.destroy()
+
+
 def test_argument_errors(hip):
     import torch
     t = torch.zeros(1024, dtype=torch.float32, device="cuda")

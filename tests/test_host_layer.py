@@ -112,8 +112,6 @@ def test_launch_options_listed(E):
     E.LaunchEnvironments.registerOpt("PCCL_TEST_OPTION")
     E.LaunchEnvironments.registerOpt("PCCL_TEST_OPTION")
     assert E.LaunchEnvironments.listOpt().count("PCCL_TEST_OPTION") == 1
-    from pccl_amd import engine_c  # module layout of csrc/python_api.cc
-    assert engine_c.Engine is E.Engine and engine_c.utils.LaunchEnvironments.listOpt() == E.LaunchEnvironments.listOpt()
     assert E.LaunchEnvironments.getEnv("PCCL_SURELY_UNSET_VARIABLE") == ""
     assert E.LaunchEnvironments.getEnv("PATH") == os.environ["PATH"]
 
@@ -361,6 +359,32 @@ def test_collective_ir_container():
     x = bad.create_operation(PrimitiveOpType.COPY, c, c, 0, 0)
     bad.op_dag.add_edge(x, x)
     assert not bad.validate_dag() and bad.get_operation_sequence() == []
+
+
+def test_extension_module_has_the_reference_layout(E, tmp_path):
+    """pccl_amd.engine_c is a compiled extension module laid out like the reference's pccl.engine_c
+    (csrc/python_api.cc:13-27): class Engine with the reference's methods, submodule utils with
+    LaunchEnvironments; it shares the registry and the option list with the C ABI's view."""
+    import torch  # noqa: F401  (a torch extension: torch's libraries and type casters come first)
+    from pccl_amd import engine_c
+    assert engine_c.__file__.endswith(".so")
+    for method in ("initEngine", "regOp", "exeOp", "exportEndpoint", "joinCluster", "exitCluster"):
+        assert callable(getattr(engine_c.Engine, method))
+    assert engine_c.utils.LaunchEnvironments.listOpt() == E.LaunchEnvironments.listOpt()
+    assert engine_c.utils.LaunchEnvironments.getEnv("PATH") == os.environ["PATH"]
+    eng = engine_c.Engine(0, 1)
+    for call in (eng.exportEndpoint, lambda: eng.joinCluster("127.0.0.1:1"), eng.exitCluster):
+        with pytest.raises(RuntimeError, match="no cluster control plane"):
+            call()
+    with pytest.raises(RuntimeError, match="open file"):
+        eng.regOp("ring", str(tmp_path / "missing.sched"))
+    with pytest.raises(RuntimeError):
+        engine_c.Engine(3, 2)            # rank outside the world
+    # tensors that are not on the device are refused before anything is launched
+    eng2 = engine_c.Engine(0, 1)
+    x = torch.zeros(16)
+    with pytest.raises(RuntimeError):
+        eng2.exeOp("nothing", x, x.clone())
 
 
 def test_tensor_overload_header_compiles_against_torch(tmp_path):
