@@ -212,6 +212,29 @@ def main():
             for p in sep:
                 hip.free(p)
             del full, sep
+            # the headline op as a one-op schedule through Engine::regOp / exeOp (input tensor = the eight
+            # operands back to back, as exeOp's tensor layout has them)
+            import tempfile
+            from pccl_amd import engine as engine_mod
+            with tempfile.TemporaryDirectory() as tmp:
+                path = os.path.join(tmp, "fold8.sched")
+                with open(path, "w") as f:
+                    f.write("pccl-schedule 1\nname fold8\ndtype bf16\ncompute sum\ndevices 8\nelems_per_device %d\nops 1\n" % count)
+                    f.write("op 0 REDUCE %d deps 0 src 8 %s dst 1 out 0 0\n" % (count, " ".join("in %d 0" % r for r in range(8))))
+                eng = engine_mod.Engine(0, 1)
+                eng.initEngine()
+                eng.regOp("fold8", path)
+                x = torch.cat(ins)
+                y = torch.zeros(8 * count, dtype=torch.bfloat16, device="cuda")
+                te = event_times_us(torch, lambda: eng.exeOp("fold8", x, y, stream), 20, 3)
+                eng.waitOp("fold8", stream)
+                assert torch.equal(y[:count], out), "engine result differs from the headline output"
+                extras["headline_op_via_engine_exeOp"] = dict(
+                    stats(te), GBps_median=gbps(step_bytes, te[len(te) // 2]),
+                    note="one-op schedule file -> Engine::regOp / exeOp; the executor runs a graph of one op as a plain launch; "
+                         "operands are the eight 256 MiB regions of ONE input tensor (no placed starts)")
+                eng.close()
+                del x, y
 
         # ---- 128 MiB variants: bf16 8->1 and fp16 8->2, operands from separate plugin allocations ----
         c3 = 1 << 26
@@ -398,10 +421,30 @@ def main():
                 t1 = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", rb["in"], rb["out"], per_rank, stream), 20, 3)
                 for r in range(8):
                     assert torch.equal(rb["out"][r], want_sum)
+                # ... and the way the reference's host code would run it: the schedule from its file through
+                # Engine::regOp / exeOp on one input and one output tensor.  The executor folds each copy into
+                # the fold that feeds it and joins the eight slices: one 8 -> 8 launch.
+                import tempfile
+                from pccl_amd import engine as engine_mod
+                with tempfile.TemporaryDirectory() as tmp:
+                    path = os.path.join(tmp, "direct.sched")
+                    ir.save(path, per_rank)
+                    eng = engine_mod.Engine(0, 1)
+                    eng.initEngine()
+                    eng.regOp("direct", path)
+                    x = torch.cat(rb["in"])
+                    y = torch.zeros(8 * per_rank, dtype=torch.bfloat16, device="cuda")
+                    te = event_times_us(torch, lambda: eng.exeOp("direct", x, y, stream), 20, 3)
+                    eng.waitOp("direct", stream)
+                    for r in range(8):
+                        assert torch.equal(y[r * per_rank:(r + 1) * per_rank], want_sum), "engine result differs"
+                    eng.close()
+                    del x, y
                 direct["8_ranks_x_%d_MiB" % per_rank_mib] = dict(
                     stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low), algorithmic_bytes=moved,
                     queue_entries=g.info()["n_tiles"], dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
-                    as_one_launch_8in_8out=dict(stats(t1), GBps_median=gbps(16 * per_rank * 2, t1[len(t1) // 2])))
+                    as_one_launch_8in_8out=dict(stats(t1), GBps_median=gbps(16 * per_rank * 2, t1[len(t1) // 2])),
+                    via_engine_exeOp=dict(stats(te), GBps_median=gbps(16 * per_rank * 2, te[len(te) // 2])))
                 g.destroy()
                 del rb, want_sum
             extras["direct_allreduce_one_launch"] = direct

@@ -180,7 +180,18 @@ typedef struct pccl_op_desc {
  * one ready queue (RingBuffer, :7-17).  Role: Engine::regOp,
  * csrc/engine.cc:102-104.  tile_bytes = bytes of output one workgroup handles
  * per queue entry; it fixes required_executors_.  0 = built-in choice: per dependency
- * level, 16 KiB x (bytes the level writes / 8 MiB)^(2/3), within 8 KiB to 128 KiB per part. */
+ * level, 16 KiB x (bytes the level writes / 8 MiB)^(2/3), within 8 KiB to 128 KiB per part.
+ * PCCL_HIP_TILE_AUTO = the executor's choice of HOW to run the graph as well (what Engine::exeOp
+ * uses, whose caller cannot name an entry point): a graph that, after folding copies into the op that
+ * produced their input and joining ops that continue each other, is at most two ops, or at most four
+ * independent ops of 128 MiB of traffic or more each, runs as that many pccl_hip_reduce_copy launches
+ * in dependency order (one op of 256 MiB per operand: 6.8 TB/s against 5.4 through the queue; the
+ * one-exchange all-reduce over 8 ranks: one 8 -> 8 launch); every other graph goes to the queue with
+ * the built-in part sizes.  For such a graph graph_status reports all ops complete once the stream has
+ * drained, graph_info a null layout, graph_trace PCCL_ERR_UNSUPPORTED; a launch recorded by stream
+ * capture keeps the addresses it was recorded with, whatever graph_rebind does later.
+ * PCCL_HIP_PLAN_LAUNCHES=0 sends everything to the queue. */
+#define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
 /* Drains the whole DAG with ONE persistent-kernel launch on `stream`; returns

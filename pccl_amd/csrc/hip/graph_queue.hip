@@ -98,6 +98,9 @@ struct Graph {
   std::vector<int> topo;             // a topological order of the ops
   std::vector<unsigned char> part_edge;  // per dependency, in descs order: met part by part
   std::vector<unsigned char> part_eligible;  // per op: its dependencies may be met part by part
+  // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
+  bool as_launches = false;
+  std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
 };
 
 // ---- which dependencies can be met part by part -------------------------------
@@ -196,6 +199,143 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
 // layout depends on the ops and their parts only, not on their addresses, so the arena of the
 // same ops at other addresses fits exactly; a launch recorded by stream capture keeps
 // pointing at it).
+// ---- graphs that run faster as plain launches ------------------------------------------
+// The queue is built for many ops: one op alone, however large, runs slower through it than as
+// a direct launch (bf16 8 -> 1 at 256 MiB: 450 us against 354; one 64 KiB op: 13 us against 8),
+// because every workgroup streams through a window of its own instead of the whole grid walking
+// one window.  A caller of Engine::exeOp cannot choose the entry point, so graph_create may
+// (tile_bytes == PCCL_HIP_TILE_AUTO).  Two rewrites first, both of which keep every byte written
+// the same:
+//   * a COPY whose only dependency is the op that wrote its input becomes more outputs of that
+//     op (an all-reduce slice folded 8 -> 1 and then copied 1 -> 7 is one 8 -> 8 fold);
+//   * independent ops of the same shape whose operands continue each other (slice d + 1 behind
+//     slice d in every buffer) become one op.
+// What is left runs as launches in dependency order if it is at most two ops, or at most four
+// independent ops of at least 128 MiB of traffic each; anything else goes through the queue
+// unchanged (a fused op can name 16 operands, the queue's payload 10).
+bool plan_launches(const std::vector<pccl_op_desc> &ops, std::vector<pccl_op_desc> *plan) {
+  const int n = (int)ops.size();
+  if (n == 0) return false;
+  if (const char *env = getenv("PCCL_HIP_PLAN_LAUNCHES"))
+    if (env[0] == '0') return false;
+  std::vector<pccl_op_desc> w(ops);
+  std::vector<std::vector<int>> deps(n);
+  std::vector<char> alive(n, 1);
+  for (int i = 0; i < n; ++i) {
+    const pccl_op_desc &o = w[i];
+    if (o.primitive > PCCL_REDUCE || o.dtype >= PCCL_NUM_DTYPES || o.compute > PCCL_MAX || o.count < 0) return false;
+    if (o.n_in < 1 || o.n_in > PCCL_MAX_INPUTS || o.n_out < 1 || o.n_out > PCCL_MAX_OUTPUTS) return false;
+    if (o.primitive == PCCL_COPY && o.n_in != 1) return false;
+    if (o.n_deps < 0 || (o.n_deps > 0 && !o.deps)) return false;
+    for (int d = 0; d < o.n_deps; ++d) {
+      if (o.deps[d] < 0 || o.deps[d] >= n || o.deps[d] == i) return false;
+      deps[i].push_back(o.deps[d]);
+    }
+  }
+  auto bytes_of = [&](const pccl_op_desc &o) { return (uintptr_t)o.count * (uintptr_t)elem_bytes(o.dtype); };
+  // copies folded into the op that wrote their input
+  for (bool changed = true; changed;) {
+    changed = false;
+    for (int b = 0; b < n; ++b) {
+      if (!alive[b] || w[b].n_in != 1 || deps[b].size() != 1) continue;
+      const int a = deps[b][0];
+      pccl_op_desc &A = w[a], &B = w[b];
+      if (!alive[a] || bytes_of(A) != bytes_of(B) || A.n_out + B.n_out > PCCL_MAX_OUTPUTS) continue;
+      bool reads_a = false;
+      for (int j = 0; j < A.n_out; ++j) reads_a = reads_a || A.outs[j] == B.ins[0];
+      if (!reads_a) continue;
+      // B's outputs must be new buffers to A: equal to none of A's operands and overlapping none
+      bool clear = true;
+      const uintptr_t len = bytes_of(A);
+      auto overlaps = [&](const void *x, const void *y) {
+        const uintptr_t p = (uintptr_t)x, q = (uintptr_t)y;
+        return p < q + len && q < p + len;
+      };
+      for (int k = 0; k < B.n_out && clear; ++k) {
+        for (int j = 0; j < A.n_in; ++j) clear = clear && !overlaps(B.outs[k], A.ins[j]);
+        for (int j = 0; j < A.n_out; ++j) clear = clear && !overlaps(B.outs[k], A.outs[j]);
+      }
+      // nobody else may stand between them: an op that depends on A but not on B could read a buffer B
+      // overwrites only if the graph already raced, so only direct successors of B are rewired
+      if (!clear) continue;
+      for (int k = 0; k < B.n_out; ++k) A.outs[A.n_out++] = B.outs[k];
+      alive[b] = 0;
+      for (int c = 0; c < n; ++c)
+        for (int &d : deps[c])
+          if (d == b) d = a;
+      changed = true;
+    }
+  }
+  // dependency order (ops are few when this matters; quadratic is fine up to the bound below)
+  int n_alive = 0;
+  for (int i = 0; i < n; ++i) n_alive += alive[i];
+  if (n_alive > 64) return false;
+  std::vector<int> order, indeg(n, 0);
+  std::vector<char> has_succ(n, 0);
+  for (int i = 0; i < n; ++i)
+    if (alive[i]) {
+      std::sort(deps[i].begin(), deps[i].end());
+      deps[i].erase(std::unique(deps[i].begin(), deps[i].end()), deps[i].end());
+      indeg[i] = (int)deps[i].size();
+      for (int d : deps[i]) has_succ[d] = 1;
+    }
+  for (int round = 0; round < n_alive; ++round) {
+    int pick = -1;
+    for (int i = 0; i < n && pick < 0; ++i)
+      if (alive[i] && indeg[i] == 0) pick = i;
+    if (pick < 0) return false;  // a cycle: let graph_create report it
+    order.push_back(pick);
+    indeg[pick] = -1;
+    for (int c = 0; c < n; ++c)
+      if (alive[c] && indeg[c] > 0)
+        for (int d : deps[c])
+          if (d == pick) --indeg[c];
+  }
+  // independent ops of one shape whose operands continue each other become one op
+  std::vector<pccl_op_desc> out;
+  std::vector<char> free_standing;
+  for (int i : order) {
+    pccl_op_desc o = w[i];
+    std::sort(o.outs, o.outs + o.n_out);  // every output gets the same bytes: their order is free
+    const bool alone = deps[i].empty() && !has_succ[i];
+    if (alone && !out.empty() && free_standing.back()) {
+      pccl_op_desc &m = out.back();
+      const uintptr_t step = bytes_of(m);
+      bool cont = m.dtype == o.dtype && m.compute == o.compute && m.n_in == o.n_in && m.n_out == o.n_out &&
+                  m.primitive == o.primitive;
+      for (int k = 0; cont && k < o.n_in; ++k) cont = (uintptr_t)o.ins[k] == (uintptr_t)m.ins[k] + step;
+      for (int k = 0; cont && k < o.n_out; ++k) cont = (uintptr_t)o.outs[k] == (uintptr_t)m.outs[k] + step;
+      if (cont) {
+        m.count += o.count;
+        continue;
+      }
+    }
+    o.n_deps = 0;
+    o.deps = nullptr;
+    out.push_back(o);
+    free_standing.push_back(alone);
+  }
+  bool take = out.size() <= 2;
+  if (!take && out.size() <= 4) {
+    take = true;
+    for (size_t k = 0; k < out.size(); ++k)
+      take = take && free_standing[k] && (uintptr_t)(out[k].n_in + out[k].n_out) * bytes_of(out[k]) >= ((uintptr_t)128 << 20);
+  }
+  if (take) plan->swap(out);
+  return take;
+}
+
+// What pccl_hip_reduce_copy would refuse about a planned launch's operands, found at creation time.
+int check_launch(const pccl_op_desc &o) {
+  const int es = elem_bytes(o.dtype);
+  for (int k = 0; k < o.n_in + o.n_out; ++k) {
+    const void *p = k < o.n_in ? o.ins[k] : o.outs[k - o.n_in];
+    if (!p && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: operand %d is null", o.op_uid, k);
+    if ((uintptr_t)p % (uintptr_t)es) return fail(PCCL_ERR_MISALIGNED, "op %d: operand %d not %d-byte aligned", o.op_uid, k, es);
+  }
+  return PCCL_OK;
+}
+
 // `fixed`: build into this memory, which the caller owns and which is not allocated here (the
 // arena must fit its capacity), and upload behind earlier work on its stream.
 struct FixedArena {
@@ -632,7 +772,9 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   if (!graph) return fail(PCCL_ERR_INVALID_ARG, "graph_create: graph is null");
   *graph = nullptr;
   if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PCCL_ERR_INVALID_ARG, "graph_create: bad op array");
-  if (tile_bytes < 0) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
+  if (tile_bytes < 0 && tile_bytes != PCCL_HIP_TILE_AUTO) return fail(PCCL_ERR_INVALID_ARG, "graph_create: tile_bytes %ld < 0", tile_bytes);
+  const bool may_plan = tile_bytes == PCCL_HIP_TILE_AUTO;
+  if (may_plan) tile_bytes = 0;
   // own copy of the ops and their dependency lists
   Graph *G = new Graph();
   G->tile_bytes = tile_bytes;
@@ -648,6 +790,24 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   G->deps_store.reserve(n_deps);
   for (int i = 0; i < n_ops; ++i) G->deps_store.insert(G->deps_store.end(), ops[i].deps, ops[i].deps + ops[i].n_deps);
   for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) G->descs[i].deps = G->deps_store.data() + at;
+  if (may_plan && plan_launches(G->descs, &G->launches)) {
+    // the launches' operands are checked now, as graph_create checks a queue graph's
+    for (const pccl_op_desc &o : G->launches) {
+      const int rc = check_launch(o);
+      if (rc != PCCL_OK) {
+        delete G;
+        return rc;
+      }
+    }
+    G->as_launches = true;
+    G->n_ops = n_ops;
+    if (hipGetDevice(&G->device) != hipSuccess) {
+      delete G;
+      return fail(PCCL_ERR_NO_DEVICE, "no current device");
+    }
+    *graph = G;
+    return PCCL_OK;
+  }
   const int rc = build_graph(G, 1);
   if (rc != PCCL_OK) {
     delete G;
@@ -661,6 +821,20 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_run: graph is null");
+  if (G->as_launches) {
+    std::vector<pccl_op_desc> launches;
+    {
+      std::lock_guard<std::mutex> lock(G->mu);  // graph_rebind may be moving operands
+      launches = G->launches;
+    }
+    for (const pccl_op_desc &o : launches) {
+      const int rc = pccl_hip_reduce_copy(o.dtype, o.compute, o.ins, o.n_in, o.outs, o.n_out, o.count, stream);
+      if (rc != PCCL_OK) return rc;
+    }
+    std::lock_guard<std::mutex> lock(G->mu);
+    ++G->runs;
+    return PCCL_OK;
+  }
   if (G->total_tiles == 0) return PCCL_OK;
   GraphControl control;
   {
@@ -682,6 +856,7 @@ int pccl_hip_graph_trace(void *graph, int enable) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_trace: graph is null");
+  if (G->as_launches) return fail(PCCL_ERR_UNSUPPORTED, "graph_trace: this graph runs as %zu plain launches, there are no queue entries to time", G->launches.size());
   std::lock_guard<std::mutex> lock(G->mu);
   GraphControl *C = (GraphControl *)G->image.data();
   G->trace_on = enable != 0;
@@ -720,6 +895,11 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed, un
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_status: graph is null");
   PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  if (G->as_launches) {  // launches that have ended have completed their ops
+    if (completed) *completed = G->runs ? (unsigned int)G->n_ops : 0u;
+    if (total) *total = (unsigned int)G->n_ops;
+    return PCCL_OK;
+  }
   const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
   HotWord hot[kHotWords];
   PCCL_HIP_CHECK(hipMemcpy(hot, G->dev + off_hot, sizeof(hot), hipMemcpyDeviceToHost));
@@ -767,6 +947,20 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
       if (k < o.n_in) o.ins[k] = p;
       else o.outs[k - o.n_in] = p;
     }
+  }
+  if (G->as_launches) {
+    // The plan was made for the old addresses (which copies fold into their producers, which ops
+    // continue each other); it is made again for the new ones.  Nothing on the device changes.
+    std::vector<pccl_op_desc> plan;
+    if (!plan_launches(next, &plan))
+      return fail(PCCL_ERR_UNSUPPORTED, "graph_rebind: with these addresses the graph no longer runs as plain launches; create it again");
+    for (const pccl_op_desc &o : plan) {
+      const int rc = check_launch(o);
+      if (rc != PCCL_OK) return rc;
+    }
+    G->descs.swap(next);
+    G->launches.swap(plan);
+    return PCCL_OK;
   }
   // Which dependencies may be met part by part depends on which operands share addresses
   // (an output tensor that now is the input tensor, say).  If that changed, the arena's
@@ -829,9 +1023,9 @@ int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_info: graph is null");
-  if (device_layout) *device_layout = G->dev;
-  if (n_tiles) *n_tiles = G->total_tiles;
-  if (n_workgroups) *n_workgroups = G->n_wg;
+  if (device_layout) *device_layout = G->dev;  // null for a graph that runs as plain launches
+  if (n_tiles) *n_tiles = G->as_launches ? (int)G->launches.size() : G->total_tiles;
+  if (n_workgroups) *n_workgroups = G->n_wg;  // 0 for a graph that runs as plain launches
   return PCCL_OK;
 }
 
@@ -872,6 +1066,7 @@ int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capa
   if (!G || !n_deps) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: null argument");
   if (capacity < 0 || (capacity > 0 && !kinds)) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: bad buffer");
   std::lock_guard<std::mutex> lock(G->mu);
+  if (G->as_launches && G->part_edge.empty()) G->part_edge.assign(G->deps_store.size(), 0);  // stream order: whole-op
   *n_deps = (long)G->part_edge.size();
   const long n = std::min<long>(capacity, *n_deps);
   if (n > 0) memcpy(kinds, G->part_edge.data(), (size_t)n);
@@ -894,6 +1089,7 @@ int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls) {
   if (polls < 64) polls = 64;
   std::lock_guard<std::mutex> lock(G->mu);
   G->spin_limit = polls;
+  if (G->as_launches) return PCCL_OK;  // nothing waits inside plain launches
   ((GraphControl *)G->image.data())->spin_limit = polls;
   PCCL_HIP_CHECK(hipMemcpy(G->dev + offsetof(GraphControl, spin_limit), &polls, sizeof(polls), hipMemcpyHostToDevice));
   return PCCL_OK;
@@ -983,7 +1179,7 @@ int pccl_hip_graph_destroy(void *graph) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return PCCL_OK;
-  hipError_t e = hipFree(G->dev);
+  hipError_t e = G->dev ? hipFree(G->dev) : hipSuccess;
   if (G->trace) {
     const hipError_t e2 = hipFree(G->trace);
     if (e == hipSuccess) e = e2;

@@ -59,6 +59,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_LDS_BYTES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_UNROLL");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_TILE_BYTES");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_PLAN_LAUNCHES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PART_DEPS");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_ORDER_BLOCK");
   }
@@ -184,7 +185,8 @@ void *HipExecutor::createGraph(const std::vector<BoundOp> &ops) {
     d.n_deps = (int)o.deps.size();
     d.deps = o.deps.empty() ? nullptr : o.deps.data();
   }
-  long tile_bytes = 0;
+  // the executor's choice: plain launches for the few graphs that run faster that way, else the queue
+  long tile_bytes = PCCL_HIP_TILE_AUTO;
   const std::string tb = utils::LaunchEnvironments::getEnv("PCCL_HIP_TILE_BYTES");
   if (!tb.empty()) tile_bytes = std::stol(tb);
   void *graph = nullptr;

@@ -245,6 +245,7 @@ def classify_dependencies(ops, parts):
 
 
 STATIC_ARENA_BYTES = 8 << 20
+TILE_AUTO = -1   # graph_create: the executor chooses between the queue and plain launches
 
 
 def graph_run_static(ops, stream=None, tile_bytes=0, wait=True):

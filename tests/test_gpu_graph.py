@@ -707,3 +707,107 @@ def test_graph_beside_a_kernel_that_occupies_the_gpu(hip, oracle):
         for r in range(world):
             H.assert_bits_equal(bufs["out"][r].download(), outs[r], "rank %d, rep %d" % (r, rep))
     g.destroy()
+
+
+# ---- graphs the executor runs as plain launches (tile_bytes = TILE_AUTO) ----------------------------
+
+def _bound_direct_allreduce(torch, hip, oracle, world, slice_elems, dtype, seed):
+    from pccl_amd import lang
+    ir, per_rank = lang.direct_allreduce(world, slice_elems, dtype=dtype)
+    low = ir.lower()
+    host_in = [H.gen(dtype, per_rank, seed, r) for r in range(world)]
+    bufs = {"in": [H.DevBuf(torch, dtype, per_rank, 0, src=a) for a in host_in],
+            "out": [H.DevBuf(torch, dtype, per_rank, 0) for _ in range(world)]}
+    es = H.ELEM_BYTES[dtype]
+    bound = lang.bind(low, lambda b, r, e: bufs[b][r].ptr + es * e)
+    want = oracle.reduce(dtype, "sum", host_in)
+    return low, bound, bufs, want
+
+
+def test_one_exchange_allreduce_becomes_one_launch(hip, oracle):
+    """8 folds 8 -> 1 each followed by a copy 1 -> 7: the copies fold into their producers, the eight
+    8 -> 8 ops continue each other slice by slice and join: one launch.  Same bytes as the queue."""
+    import torch
+    stream = _stream(torch)
+    low, bound, bufs, want = _bound_direct_allreduce(torch, hip, oracle, 8, 20_000, "bf16", 701)
+    g = hip.Graph(bound, hip.TILE_AUTO)
+    info = g.info()
+    assert info["n_tiles"] == 1 and info["n_workgroups"] == 0 and not info["device_layout"]
+    assert g.status(stream) == (0, 16)
+    g.run(stream)
+    assert g.status(stream) == (16, 16)
+    for r in range(8):
+        H.assert_bits_equal(bufs["out"][r].download(), want, "rank %d, one launch" % r)
+        assert bufs["out"][r].guards_intact()
+        bufs["out"][r].view().fill_(0xFF)
+    assert g.dependency_kinds() == [0] * 8
+    with pytest.raises(hip.PcclError):
+        g.trace(True)
+    q = hip.Graph(bound)                       # the same ops through the queue
+    assert q.info()["n_workgroups"] > 0
+    q.run(stream)
+    assert q.status(stream) == (16, 16)
+    for r in range(8):
+        H.assert_bits_equal(bufs["out"][r].download(), want, "rank %d, queue" % r)
+    g.destroy()
+    q.destroy()
+
+
+def test_ragged_slices_and_small_graphs_as_launches(hip, oracle):
+    import torch
+    stream = _stream(torch)
+    # slices of an odd number of elements still join (the joined op is just a longer flat array)
+    low, bound, bufs, want = _bound_direct_allreduce(torch, hip, oracle, 4, 4099, "f16", 702)
+    g = hip.Graph(bound, hip.TILE_AUTO)
+    assert g.info()["n_tiles"] == 1
+    g.run(stream)
+    assert g.status(stream) == (8, 8)
+    for r in range(4):
+        H.assert_bits_equal(bufs["out"][r].download(), want, "rank %d" % r)
+    g.destroy()
+    # two dependent ops stay two launches in order: t = a + b; u = t * c (the second is no copy)
+    n = 300_007
+    a, b, c = (H.gen("f32", n, 703, k) for k in range(3))
+    da, db, dc = (H.DevBuf(torch, "f32", n, 4 * k, src=x) for k, x in enumerate((a, b, c)))
+    dt, du = H.DevBuf(torch, "f32", n, 0), H.DevBuf(torch, "f32", n, 8)
+    g = hip.Graph([dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=n, deps=[]),
+                   dict(dtype="f32", compute="prod", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=n, deps=[0])], hip.TILE_AUTO)
+    assert g.info()["n_tiles"] == 2
+    g.run(stream)
+    assert g.status(stream) == (2, 2)
+    t = oracle.reduce("f32", "sum", [a, b])
+    H.assert_bits_equal(dt.download(), t, "t")
+    H.assert_bits_equal(du.download(), oracle.reduce("f32", "prod", [t, c]), "u")
+    # rebinding moves the launches' operands
+    du2 = H.DevBuf(torch, "f32", n, 12)
+    g.rebind(du.ptr, du2.ptr, 4 * n, stream)
+    g.run(stream)
+    assert g.status(stream) == (2, 2)
+    H.assert_bits_equal(du2.download(), oracle.reduce("f32", "prod", [t, c]), "u after the rebind")
+    g.destroy()
+    # a copy onto its producer's own input is not folded in (the fold would read what it overwrites
+    # elsewhere); still two launches, still sequential semantics
+    g = hip.Graph([dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=n - 16, deps=[]),
+                   dict(dtype="f32", compute="sum", ins=[dt.ptr], outs=[da.ptr + 64], count=n - 16, deps=[0])], hip.TILE_AUTO)
+    assert g.info()["n_tiles"] == 2
+    g.run(stream)
+    assert g.status(stream) == (2, 2)
+    t2 = oracle.reduce("f32", "sum", [a[:n - 16], b[:n - 16]])
+    H.assert_bits_equal(da.download()[16:], t2, "shifted copy back onto the first input")
+    g.destroy()
+
+
+def test_many_ops_stay_in_the_queue_under_tile_auto(hip, oracle):
+    import torch
+    from pccl_amd import lang
+    ir, per_rank = lang.ring_allreduce(8, 1000, dtype="bf16")
+    low = ir.lower()
+    bufs = {"in": [H.DevBuf(torch, "bf16", per_rank, 0, src=H.gen("bf16", per_rank, 704, r)) for r in range(8)],
+            "out": [H.DevBuf(torch, "bf16", per_rank, 0) for _ in range(8)]}
+    g = hip.Graph(lang.bind(low, lambda b, r, e: bufs[b][r].ptr + 2 * e), hip.TILE_AUTO)
+    assert g.info()["n_workgroups"] > 0 and g.info()["n_tiles"] >= len(low)
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (len(low), len(low))
+    for r in range(1, 8):
+        H.assert_bits_equal(bufs["out"][r].download(), bufs["out"][0].download(), "rank %d equals rank 0" % r)
+    g.destroy()
