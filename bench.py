@@ -16,10 +16,93 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# scaled by what the same counters read for a plain copy of known size (figures and commands in
-# profiles/reduce_copy_bf16_8in_256MiB.md).
-MEASURED_TRAFFIC_BYTES = 2415753079
+# HBM bytes per launch of the headline kernel come from a committed record of two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a plain copy of known size.
+# `bench.py --traffic-record FETCH_DIR WRITE_DIR` writes the record from the two runs' output folders;
+# a normal run reads it and says whether it still belongs to this kernel and this file.
+HEADLINE_KERNEL = "pccl_dev::reduce_copy_lean_kernel<2, pccl_dev::OpSum, 8, 1, 2>"
+CALIBRATION_KERNEL = "pccl_dev::reduce_copy_lean_kernel<2, pccl_dev::OpSum, 1, 1, 2>"
+TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "reduce_copy_bf16_8in_256MiB.traffic.txt")
+PROFILE_COMMAND = "python3 bench.py --no-extras --no-cpu --steps 20 --warmup 5 --calibration-copy 10"
+
+
+def bench_sha16():
+    import hashlib
+    with open(os.path.abspath(__file__), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def _counter_means(folder, counter):
+    """Mean per-dispatch value of `counter` for the headline and the calibration kernel, from the
+    *_counter_collection.csv files rocprofv3 left under `folder`."""
+    import csv
+    import glob
+    vals = {HEADLINE_KERNEL: [], CALIBRATION_KERNEL: []}
+    files = glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+        raise SystemExit("no *_counter_collection.csv under %s" % folder)
+    for path in files:
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                name = row["Kernel_Name"].replace("void ", "").split("(")[0].strip()
+                if row["Counter_Name"] == counter and name in vals:
+                    vals[name].append(float(row["Counter_Value"]))
+    for k, v in vals.items():
+        if not v:
+            raise SystemExit("%s: no %s dispatches of %s" % (folder, counter, k))
+    return {k: (sum(v) / len(v), len(v)) for k, v in vals.items()}
+
+
+def write_traffic_record(fetch_dir, write_dir):
+    import subprocess
+    copy_kib = (1 << 28) / 1024.0   # the calibration copy reads and writes one 256 MiB buffer
+    lines, total = [], 0.0
+    for counter, folder in (("FETCH_SIZE", fetch_dir), ("WRITE_SIZE", write_dir)):
+        m = _counter_means(folder, counter)
+        (head, n_head), (cal, n_cal) = m[HEADLINE_KERNEL], m[CALIBRATION_KERNEL]
+        factor = copy_kib / cal
+        total += head * factor * 1024.0
+        lines += ["%s_copy_kernel_per_dispatch: %.1f (%d dispatches; known %d KiB)" % (counter, cal, n_cal, copy_kib),
+                  "%s_scale: %.6f" % (counter, factor),
+                  "%s_headline_kernel_per_dispatch: %.1f (%d dispatches)" % (counter, head, n_head),
+                  "%s_headline_kernel_scaled_KiB: %.0f" % (counter, head * factor)]
+    commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    text = ["# HBM traffic per launch of the headline kernel (bf16 8 -> 1, 256 MiB per buffer), rocprofv3 --pmc",
+            "kernel: %s" % HEADLINE_KERNEL,
+            "calibration_kernel: %s (plain copy of one 256 MiB buffer)" % CALIBRATION_KERNEL,
+            "command_fetch: rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir> -- %s" % PROFILE_COMMAND,
+            "command_write: rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir> -- %s" % PROFILE_COMMAND,
+            "git_commit: %s" % (commit or "unknown"),
+            "bench_py_sha16: %s" % bench_sha16()] + lines + [
+            "algorithmic_bytes: %d" % (9 << 28),
+            "traffic_bytes: %d" % round(total)]
+    with open(TRAFFIC_RECORD, "w") as f:
+        f.write("\n".join(text) + "\n")
+    print("\n".join(text))
+
+
+def read_traffic_record():
+    """(traffic bytes or None, where it comes from and whether it is stale)."""
+    if not os.path.exists(TRAFFIC_RECORD):
+        return None, {"file": None, "stale": True, "why": "no record committed"}
+    rec = {}
+    for line in open(TRAFFIC_RECORD):
+        if ":" in line and not line.startswith("#"):
+            k, v = line.split(":", 1)
+            rec[k.strip()] = v.strip()
+    why = []
+    if rec.get("kernel") != HEADLINE_KERNEL:
+        why.append("recorded for another kernel")
+    if rec.get("bench_py_sha16") != bench_sha16():
+        why.append("bench.py changed since the record was made")
+    src = {"file": os.path.relpath(TRAFFIC_RECORD, ROOT), "kernel": rec.get("kernel"), "git_commit": rec.get("git_commit"),
+           "bench_py_sha16": rec.get("bench_py_sha16"), "stale": bool(why)}
+    if why:
+        src["why"] = "; ".join(why)
+    try:
+        return int(rec["traffic_bytes"]), src
+    except (KeyError, ValueError):
+        return None, dict(src, stale=True, why="record has no traffic_bytes")
 
 
 def parse():
@@ -36,6 +119,9 @@ def parse():
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="N",
                     help="also launch N plain copies (1 input -> 1 output) of the same 256 MiB buffers: the "
                          "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--traffic-record", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="write %s from the output folders of the two rocprofv3 --pmc runs, then exit (no GPU needed)"
+                         % os.path.relpath(TRAFFIC_RECORD, ROOT))
     return ap.parse_args()
 
 
@@ -99,8 +185,10 @@ def cpu_baseline(count_sample):
     o32 = np.empty(1 << 20, dtype=np.float32)
     ring_in = [x[:1 << 24] if count_sample >= (1 << 24) else np.resize(x, 1 << 24) for x in ins[:2]]
     ring_out = [np.empty(1 << 24, dtype=np.uint16) for _ in range(2)]
+    c3 = min(count_sample, 1 << 26)
     for name, dt, i_, o_, n_, nb in (("f32_2in_1out_4MiB", "f32", a32, [o32], 1 << 20, 3 * 4 << 20),
-                                     ("bf16_2in_2out_32MiB_ring_step", "bf16", ring_in, ring_out, 1 << 24, 4 * 32 << 20)):
+                                     ("bf16_2in_2out_32MiB_ring_step", "bf16", ring_in, ring_out, 1 << 24, 4 * 32 << 20),
+                                     ("bf16_8in_1out_128MiB", "bf16", [x[:c3] for x in ins], [out[:c3]], c3, 9 * c3 * 2)):
         r = {}
         for threads in (1, cores):
             ts = []
@@ -110,6 +198,27 @@ def cpu_baseline(count_sample):
                 ts.append(time.perf_counter() - t0)
             r["GBps_%d_thread%s" % (threads, "" if threads == 1 else "s")] = round(nb / min(ts) / 1e9, 2)
         other[name] = r
+    # one rank's 14 ring steps (7 reduce steps 2 -> 2, 7 copy steps) over 32 MiB chunks
+    grad = np.resize(ins[0], 8 << 24)
+    peers = [np.resize(ins[1 + s % 7], 1 << 24) for s in range(7)]
+    result = np.empty(8 << 24, dtype=np.uint16)
+    send = np.empty(1 << 24, dtype=np.uint16)
+    ce = 1 << 24
+    r = {}
+    for threads in (1, cores):
+        ts = []
+        for _ in range(2):
+            t0 = time.perf_counter()
+            for s in range(7):
+                c = (7 - s) % 8
+                orc.reduce_copy("bf16", "sum", [peers[s], grad[c * ce:(c + 1) * ce]], [result[c * ce:(c + 1) * ce], send], ce, nthreads=threads)
+            for s in range(7):
+                c = (8 - s) % 8
+                orc.reduce_copy("bf16", "sum", [peers[s]], [result[c * ce:(c + 1) * ce]], ce, nthreads=threads)
+            ts.append(time.perf_counter() - t0)
+        r["GBps_%d_thread%s" % (threads, "" if threads == 1 else "s")] = round((7 * 4 + 7 * 2) * ce * 2 / min(ts) / 1e9, 2)
+        r["ms_%d_thread%s" % (threads, "" if threads == 1 else "s")] = round(min(ts) * 1e3, 1)
+    other["bf16_ring_rank_share_14_steps_32MiB"] = r
     return {"value": round(best[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": "bf16 8->1 sum, %d elements per buffer (%s), best of 5 (this leg took %.0f s); "
                       "single thread: %.2f GB/s" % (count_sample, "the whole headline step" if count_sample == 1 << 27 else
@@ -120,6 +229,9 @@ def cpu_baseline(count_sample):
 
 def main():
     args = parse()
+    if args.traffic_record:
+        write_traffic_record(*args.traffic_record)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (peers are HBM buffers on the "
               "same device); run with --gpus 1", file=sys.stderr)
@@ -165,9 +277,10 @@ def main():
     ts = event_times_us(torch, step, max(20, min(args.steps, 100)), 3)
     mean_us = sum(ts) / len(ts)
     achieved = step_bytes / mean_us / 1e3
+    traffic, traffic_source = read_traffic_record()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                "kernel": "reduce_copy_lean_kernel<bf16, sum, n_in=8, n_out=1>", "algorithmic_bytes_per_launch": step_bytes,
+                "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                "kernel": HEADLINE_KERNEL, "algorithmic_bytes_per_launch": step_bytes,
                 "launch_us": stats(ts)}
 
     # quick self-check of the timed buffers against torch's fp32 accumulate (same fold order)
@@ -455,7 +568,27 @@ def main():
             o = torch.empty_like(a)
             t = event_times_us(torch, lambda: hip.reduce_copy("f32", "sum", [a, b], [o], 1 << 20, stream), 100, 10)
             assert torch.equal(o, a + b)
-            extras["f32_2in_1out_4MiB"] = stats(t)
+            # where the time of one small launch goes: the host call (ctypes, argument checks, launch),
+            # launches issued back to back (what the GPU front end sustains), and one launch between two
+            # events (what `stats` reports; the kernel itself is 2.9 us by rocprofv3)
+            torch.cuda.synchronize()
+            n_calls = 2000
+            t0 = time.perf_counter()
+            for _ in range(n_calls):
+                hip.reduce_copy("f32", "sum", [a, b], [o], 1 << 20, stream)
+            host_us = (time.perf_counter() - t0) / n_calls * 1e6
+            torch.cuda.synchronize()
+            pa, pb, po = a.data_ptr(), b.data_ptr(), o.data_ptr()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n_calls):
+                hip.reduce_copy("f32", "sum", [pa, pb], [po], 1 << 20, stream)
+            e1.record()
+            torch.cuda.synchronize()
+            extras["f32_2in_1out_4MiB"] = dict(
+                stats(t), host_call_us=round(host_us, 2), back_to_back_us_per_launch=round(e0.elapsed_time(e1) * 1e3 / n_calls, 2),
+                note="median_us = one launch between two events; host_call_us = Python ctypes call incl. the library's "
+                     "argument checks and hipLaunchKernel, nothing waited for; back_to_back = 2000 launches between two events")
 
         # ---- unaligned operands: i32 4 -> 1, 2^28-57 elements, every buffer 4..60 bytes off 64 ----
         if want("unaligned"):

@@ -4,6 +4,7 @@
 // rounded up to 2 MiB (:60,70), nbytes <= 0 gives a null pointer (:61), live
 // allocations are tracked in a pointer-keyed map under a mutex (:50-51,121-144).
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -42,20 +43,22 @@ int compute_units() {
   return cus;
 }
 
-static std::mutex g_tuning_mutex;
-static Tuning g_tuning = {0, -1, -1, -1};
-static bool g_tuning_env_read = false;
+// Launch-shape overrides (tuning runs only).  Read on every launch, so lock-free: four relaxed
+// atomics, the environment consulted once.
+static std::atomic<int> g_tune_wg{0}, g_tune_cache{-1}, g_tune_lds{-1}, g_tune_unroll{-1};
+static std::once_flag g_tuning_env_once;
+
+static void read_tuning_env() {  // same knobs the host plugin lists as launch options
+  if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tune_wg.store(atoi(s), std::memory_order_relaxed);
+  if (const char *s = getenv("PCCL_HIP_NT")) g_tune_cache.store(std::max(0, std::min(2, atoi(s))), std::memory_order_relaxed);
+  if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tune_lds.store(atoi(s), std::memory_order_relaxed);
+  if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tune_unroll.store(atoi(s), std::memory_order_relaxed);
+}
 
 Tuning tuning() {
-  std::lock_guard<std::mutex> lock(g_tuning_mutex);
-  if (!g_tuning_env_read) {  // same knobs the host plugin lists as launch options
-    g_tuning_env_read = true;
-    if (const char *s = getenv("PCCL_HIP_WG_PER_CU")) g_tuning.workgroups_per_cu = atoi(s);
-    if (const char *s = getenv("PCCL_HIP_NT")) g_tuning.cache_treatment = std::max(0, std::min(2, atoi(s)));
-    if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tuning.lds_bytes = atoi(s);
-    if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tuning.unroll = atoi(s);
-  }
-  return g_tuning;
+  std::call_once(g_tuning_env_once, read_tuning_env);
+  return Tuning{g_tune_wg.load(std::memory_order_relaxed), g_tune_cache.load(std::memory_order_relaxed),
+                g_tune_lds.load(std::memory_order_relaxed), g_tune_unroll.load(std::memory_order_relaxed)};
 }
 
 // ---- where a buffer starts: placement by the memory-channel hash -------------------------
@@ -453,9 +456,8 @@ int pccl_hip_set_tuning(int workgroups_per_cu, int cache_treatment) {
   if (workgroups_per_cu < 0 || workgroups_per_cu > 64)
     return fail(PCCL_ERR_INVALID_ARG, "workgroups_per_cu %d outside [0, 64]", workgroups_per_cu);
   (void)tuning();  // make sure the environment was read before overriding it
-  std::lock_guard<std::mutex> lock(g_tuning_mutex);
-  g_tuning.workgroups_per_cu = workgroups_per_cu;
-  g_tuning.cache_treatment = cache_treatment < 0 ? -1 : std::min(cache_treatment, 2);
+  g_tune_wg.store(workgroups_per_cu, std::memory_order_relaxed);
+  g_tune_cache.store(cache_treatment < 0 ? -1 : std::min(cache_treatment, 2), std::memory_order_relaxed);
   return PCCL_OK;
 }
 
@@ -464,8 +466,7 @@ int pccl_hip_set_unroll(int unroll) {
   if (unroll != -1 && unroll != 0 && unroll != 1 && unroll != 4)
     return fail(PCCL_ERR_INVALID_ARG, "unroll %d is not -1, 0, 1 or 4", unroll);
   (void)tuning();
-  std::lock_guard<std::mutex> lock(g_tuning_mutex);
-  g_tuning.unroll = unroll;
+  g_tune_unroll.store(unroll, std::memory_order_relaxed);
   return PCCL_OK;
 }
 
@@ -473,8 +474,7 @@ int pccl_hip_set_occupancy_lds(int lds_bytes) {
   clear_error();
   if (lds_bytes > 160 * 1024) return fail(PCCL_ERR_INVALID_ARG, "lds_bytes %d exceeds the 160 KiB of a compute unit", lds_bytes);
   (void)tuning();
-  std::lock_guard<std::mutex> lock(g_tuning_mutex);
-  g_tuning.lds_bytes = lds_bytes < 0 ? -1 : lds_bytes;
+  g_tune_lds.store(lds_bytes < 0 ? -1 : lds_bytes, std::memory_order_relaxed);
   return PCCL_OK;
 }
 

@@ -46,6 +46,7 @@
 #include <cmath>
 #include <cstring>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "graph_queue_device.h"
@@ -439,13 +440,42 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // pre_dependencies_ (the hand-over itself goes through the signal word).
   std::vector<std::vector<int>> order_succ(n_ops);
   std::vector<int> order_pred(n_ops, 0);
-  for (int a : signal_ops) {
-    if (ops[a].primitive != PCCL_NOTIFY) continue;
-    for (int b : signal_ops)
-      if (ops[b].primitive == PCCL_GET_NOTIFIED && ops[b].ins[0] == ops[a].outs[0] && ops[b].count == ops[a].count) {
-        order_succ[a].push_back(b);
-        ++order_pred[b];
+  {
+    // NOTIFYs by signal word.  A GET_NOTIFIED(word, v) is satisfied by any NOTIFY(word, w >= v); it is
+    // ordered behind the one with the smallest such w (the first that can release it).  When that
+    // NOTIFY has another value than the GET asks for, the edge is only added if the GET is not
+    // itself upstream of the NOTIFY (a wait that an outside party satisfies, followed by a later
+    // notification on the same word, is a legitimate program, and the edge would close a cycle).
+    std::unordered_map<const void *, std::vector<int>> notifies;
+    for (int a : signal_ops)
+      if (ops[a].primitive == PCCL_NOTIFY) notifies[ops[a].outs[0]].push_back(a);
+    auto reaches = [&](int from, int to) {  // over dependency edges and the ordering edges so far
+      std::vector<char> seen(n_ops, 0);
+      std::vector<int> stack{from};
+      seen[from] = 1;
+      while (!stack.empty()) {
+        const int u = stack.back();
+        stack.pop_back();
+        if (u == to) return true;
+        for (int e = succ_start[u]; e < succ_start[u + 1]; ++e)
+          if (!seen[succ[e]]) { seen[succ[e]] = 1; stack.push_back(succ[e]); }
+        for (int v : order_succ[u])
+          if (!seen[v]) { seen[v] = 1; stack.push_back(v); }
       }
+      return false;
+    };
+    for (int b : signal_ops) {
+      if (ops[b].primitive != PCCL_GET_NOTIFIED) continue;
+      auto it = notifies.find(ops[b].ins[0]);
+      if (it == notifies.end()) continue;  // satisfied from outside the graph
+      int best = -1;
+      for (int a : it->second)
+        if (ops[a].count >= ops[b].count && (best < 0 || ops[a].count < ops[best].count)) best = a;
+      if (best < 0) continue;
+      if (ops[best].count != ops[b].count && reaches(b, best)) continue;
+      order_succ[best].push_back(b);
+      ++order_pred[b];
+    }
   }
   // level[i] = length of the longest dependency chain ending in op i
   std::vector<int> level(n_ops, 0);

@@ -116,7 +116,10 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   // default: one workgroup per chunk; a tuning run may cap it to a persistent grid
   long grid = chunks;
   if (t.workgroups_per_cu > 0) grid = std::min<long>(chunks, (long)pccl_host::compute_units() * t.workgroups_per_cu);
-  if (grid > 0x7fffffffl) grid = 0x7fffffffl;  // the kernel's chunk loop covers the rest
+  // (the general kernel's chunk loop covers whatever a clamped grid leaves; the lean kernel has no
+  // loop and sizes its own grid in launch_lean_nout, one workgroup per 4 KiB: 2^31 of them are 8 TiB
+  // per stream, more than the device holds)
+  if (grid > 0x7fffffffl) grid = 0x7fffffffl;
   // Occupancy cap for operands beyond the Infinity Cache.  Measured on MI355X: DRAM
   // efficiency is best with about 20 (workgroups x streams) resident per compute
   // unit, i.e. 2 workgroups for 8 -> 1 (+8 %), 5 for 2 -> 2 (+10 %), no cap for a

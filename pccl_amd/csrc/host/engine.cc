@@ -148,10 +148,28 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
                       (!in_moves || (apart(input, op->bound_in) && apart(input, op->bound_out))) &&
                       (!out_moves || (apart(output, op->bound_out) && apart(output, op->bound_in)));
     if (safe) {
-      if (in_moves) op->executor->rebindGraph(op->graph, op->bound_in, input, need, stream);
-      if (out_moves) op->executor->rebindGraph(op->graph, op->bound_out, output, need, stream);
-      op->bound_in = input;
-      op->bound_out = output;
+      // A previous exeOp of this op on another stream may still be reading the operand slots that a
+      // rebind rewrites behind `stream`: it ends first.
+      if (op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
+      try {
+        if (in_moves) {
+          op->executor->rebindGraph(op->graph, op->bound_in, input, need, stream);
+          op->bound_in = input;
+        }
+        if (out_moves) {
+          op->executor->rebindGraph(op->graph, op->bound_out, output, need, stream);
+          op->bound_out = output;
+        }
+      } catch (...) {
+        // half-moved operands are not worth tracking: the next exeOp builds the graph again
+        try {
+          op->executor->waitGraph(op->graph, stream);
+        } catch (...) {
+        }
+        op->executor->destroyGraph(op->graph);
+        op->graph = nullptr;
+        throw;
+      }
     } else {
       op->executor->waitGraph(op->graph, stream);
       op->executor->destroyGraph(op->graph);
@@ -161,6 +179,8 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
     }
   }
   op->executor->runGraph(op->graph, stream);
+  op->last_stream = stream;
+  op->last_stream_known = true;
 }
 
 void Engine::waitOp(const std::string &name, void *stream) {

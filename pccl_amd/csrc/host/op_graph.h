@@ -32,6 +32,8 @@ struct RegisteredOp {
   void *graph = nullptr;       // executor graph handle, built at first exeOp
   const void *bound_in = nullptr;
   const void *bound_out = nullptr;
+  void *last_stream = nullptr;       // the stream of the latest exeOp
+  bool last_stream_known = false;
   ~RegisteredOp();
 };
 

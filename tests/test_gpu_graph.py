@@ -811,3 +811,42 @@ def test_many_ops_stay_in_the_queue_under_tile_auto(hip, oracle):
     for r in range(1, 8):
         H.assert_bits_equal(bufs["out"][r].download(), bufs["out"][0].download(), "rank %d equals rank 0" % r)
     g.destroy()
+
+
+def test_get_notified_is_released_by_a_notify_of_a_larger_value(hip, oracle):
+    """GET_NOTIFIED(word, 3) completes on any value >= 3: a NOTIFY(word, 5) of the same graph satisfies it
+    and is what it is ordered behind.  And the legitimate reverse shape, a wait satisfied from outside
+    followed downstream by a NOTIFY of a larger value on the same word, builds (no cycle) and runs."""
+    import torch
+    n = 100_003
+    a = H.gen("f32", n, 801, 0)
+    da, dt, du = H.DevBuf(torch, "f32", n, 0, src=a), H.DevBuf(torch, "f32", n, 0), H.DevBuf(torch, "f32", n, 0)
+    sig = torch.zeros(4, dtype=torch.int32, device="cuda")
+    stream = _stream(torch)
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr], outs=[dt.ptr], count=n, deps=[]),
+           dict(primitive=2, signal=sig.data_ptr(), value=5, deps=[0]),
+           dict(primitive=3, signal=sig.data_ptr(), value=3, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[dt.ptr], outs=[du.ptr], count=n, deps=[2])]
+    g = hip.Graph(ops)
+    for it in range(3):
+        dt.view().fill_(0xFF)
+        du.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        g.run(stream)
+        assert g.status(stream) == (4, 4)
+        H.assert_bits_equal(du.download(), a, "copy behind GET(3) released by NOTIFY(5), run %d" % it)
+    g.destroy()
+    # wait from outside, then notify a larger value on the same word
+    ops = [dict(primitive=3, signal=sig.data_ptr() + 4, value=3, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[da.ptr], outs=[dt.ptr], count=n, deps=[0]),
+           dict(primitive=2, signal=sig.data_ptr() + 4, value=5, deps=[1])]
+    g = hip.Graph(ops)
+    base = g.next_signal_base()
+    sig[1] = base + 3
+    dt.view().fill_(0xFF)
+    torch.cuda.synchronize()
+    g.run(stream)
+    assert g.status(stream) == (3, 3)
+    H.assert_bits_equal(dt.download(), a, "copy released from outside")
+    assert int(sig[1].item()) == base + 5
+    g.destroy()
