@@ -148,6 +148,12 @@ int pccl_hip_set_occupancy_lds(int lds_bytes);
  * kernel wherever it applies, 1 or 4 = packs per lane of the general kernel. */
 int pccl_hip_set_unroll(int unroll);
 
+/* Walk override for tuning runs: which 4 KiB chunk of the streams workgroup k of a direct launch takes.
+ * 0 = chunk k; 1 = bits 5-7 of k XORed into its low three bits wherever the launch has one workgroup
+ * per chunk, so that the workgroups in flight on one XCD read from all 8 HBM channel groups whatever the
+ * operands' addresses are; -1 = built-in choice (rotated for operands beyond the Infinity Cache). */
+int pccl_hip_set_rotation(int rotate);
+
 /* ---- the op-batching path: a DAG of ops drained by one persistent kernel -- */
 
 /* One IR operation as the host hands it over: the C++ payload level of

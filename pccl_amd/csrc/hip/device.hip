@@ -45,7 +45,7 @@ int compute_units() {
 
 // Launch-shape overrides (tuning runs only).  Read on every launch, so lock-free: four relaxed
 // atomics, the environment consulted once.
-static std::atomic<int> g_tune_wg{0}, g_tune_cache{-1}, g_tune_lds{-1}, g_tune_unroll{-1};
+static std::atomic<int> g_tune_wg{0}, g_tune_cache{-1}, g_tune_lds{-1}, g_tune_unroll{-1}, g_tune_rotate{-1};
 static std::once_flag g_tuning_env_once;
 
 static void read_tuning_env() {  // same knobs the host plugin lists as launch options
@@ -53,12 +53,14 @@ static void read_tuning_env() {  // same knobs the host plugin lists as launch o
   if (const char *s = getenv("PCCL_HIP_NT")) g_tune_cache.store(std::max(0, std::min(2, atoi(s))), std::memory_order_relaxed);
   if (const char *s = getenv("PCCL_HIP_LDS_BYTES")) g_tune_lds.store(atoi(s), std::memory_order_relaxed);
   if (const char *s = getenv("PCCL_HIP_UNROLL")) g_tune_unroll.store(atoi(s), std::memory_order_relaxed);
+  if (const char *s = getenv("PCCL_HIP_ROTATE")) g_tune_rotate.store(atoi(s), std::memory_order_relaxed);
 }
 
 Tuning tuning() {
   std::call_once(g_tuning_env_once, read_tuning_env);
   return Tuning{g_tune_wg.load(std::memory_order_relaxed), g_tune_cache.load(std::memory_order_relaxed),
-                g_tune_lds.load(std::memory_order_relaxed), g_tune_unroll.load(std::memory_order_relaxed)};
+                g_tune_lds.load(std::memory_order_relaxed), g_tune_unroll.load(std::memory_order_relaxed),
+                g_tune_rotate.load(std::memory_order_relaxed)};
 }
 
 // ---- where a buffer starts: placement by the memory-channel hash -------------------------
@@ -467,6 +469,14 @@ int pccl_hip_set_unroll(int unroll) {
     return fail(PCCL_ERR_INVALID_ARG, "unroll %d is not -1, 0, 1 or 4", unroll);
   (void)tuning();
   g_tune_unroll.store(unroll, std::memory_order_relaxed);
+  return PCCL_OK;
+}
+
+int pccl_hip_set_rotation(int rotate) {
+  clear_error();
+  if (rotate < -1 || rotate > 1) return fail(PCCL_ERR_INVALID_ARG, "rotate %d is not -1, 0 or 1", rotate);
+  (void)tuning();
+  g_tune_rotate.store(rotate, std::memory_order_relaxed);
   return PCCL_OK;
 }
 

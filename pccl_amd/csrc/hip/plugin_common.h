@@ -29,6 +29,7 @@ struct Tuning {
   int cache_treatment;        // -1 = built-in choice, else 0 cacheable / 1 streaming / 2 streaming loads + write-through stores
   int lds_bytes;          // -1 = built-in choice, else dynamic LDS requested per workgroup
   int unroll;             // -1 = built-in choice, 0 = lean kernel where it applies, else packs per lane (1 or 4)
+  int rotate;             // -1 = built-in choice, 0 = workgroup k takes chunk k, 1 = rotated wherever the launch shape allows
 };
 Tuning tuning();
 

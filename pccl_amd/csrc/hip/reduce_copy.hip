@@ -140,6 +140,16 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
     if (es == 1 && n_in > 1) wgs = std::max(wgs, 4);
     if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
   }
+  // Workgroup -> chunk rotation (rotated_chunk in reduce_copy_kernel.h) wherever the launch has one
+  // workgroup per 4 KiB chunk and the operands are treated as streams (48 MiB in all and more).  It pays
+  // when the data comes from HBM and costs when it sits in the Infinity Cache.  bf16 on operands in
+  // separate allocations, TB/s without / with: the same buffers again and again, 128 MiB per buffer:
+  // 8 -> 1 6.69 / 6.95, 2 -> 2 6.81 / 7.20, 1 -> 1 6.61 / 6.91; 32 MiB per buffer (cache-resident):
+  // 2 -> 2 6.06 / 6.00, 1 -> 1 5.85 / 5.50, 4 -> 1 6.27 / 5.66; walks over distinct buffers (what a collective
+  // step sees), 32 MiB: 2 -> 2 5.67 / 6.02, 1 -> 1 5.73 / 5.92, 2 -> 1 5.97 / 6.23; 16 MiB: 5.44 / 5.76, 5.19 / 5.27,
+  // 5.21 / 5.47.
+  p.rotate = total_bytes >= (48l << 20) && unroll <= 1 && grid == chunks && t.rotate != 0;
+  if (t.rotate > 0 && unroll <= 1 && grid == chunks) p.rotate = 1;
   hipStream_t s = (hipStream_t)stream;
   if (n_in == 1) return launch_copy(es, unroll, aligned, mem, (unsigned)grid, lds, s, p);
   switch (dtype) {

@@ -58,6 +58,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_NT");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_LDS_BYTES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_UNROLL");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_ROTATE");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_TILE_BYTES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PLAN_LAUNCHES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PART_DEPS");

@@ -77,6 +77,7 @@ def lib():
         L.pccl_hip_set_tuning.argtypes = [ci, ci]
         L.pccl_hip_set_occupancy_lds.argtypes = [ci]
         L.pccl_hip_set_unroll.argtypes = [ci]
+        L.pccl_hip_set_rotation.argtypes = [ci]
         L.pccl_hip_graph_create.argtypes = [ctypes.POINTER(OpDesc), ci, cl, ctypes.POINTER(vp)]
         L.pccl_hip_graph_run_static.argtypes = [ctypes.POINTER(OpDesc), ci, cl, vp, ctypes.POINTER(ctypes.c_uint),
                                                 ctypes.POINTER(ctypes.c_uint)]
@@ -162,6 +163,10 @@ def placement_start(extent, nbytes, slack, before=()):
     start, code = ctypes.c_ulonglong(0), ctypes.c_uint(0)
     _check(lib().pccl_hip_placement_start(extent, nbytes, slack, addrs, sizes, n, ctypes.byref(start), ctypes.byref(code)))
     return start.value, code.value
+
+
+def set_rotation(rotate=-1):
+    _check(lib().pccl_hip_set_rotation(rotate))
 
 
 def set_tuning(workgroups_per_cu=0, cache_treatment=-1):
