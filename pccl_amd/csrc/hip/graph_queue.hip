@@ -84,9 +84,12 @@ struct Graph {
   unsigned int spin_limit = kDefaultSpinLimit;
   std::vector<char> image;      // pristine host copy of the arena
   size_t payload_off = 0;       // arena offset of the payload array
+  size_t chain_table_off = 0;   // ... and of the chain table, which follows it
   int n_ops = 0;
-  int total_tiles = 0;
+  int total_tiles = 0;          // queue entries
+  int all_tiles = 0;            // parts of all ops (>= total_tiles: an op that runs behind another in a chain queues none)
   int n_wg = 0;
+  int fixed_n_wg = 0;           // build_graph: launch this many workgroups instead of choosing
   int device = 0;
   unsigned int runs = 0;        // launches so far; run r uses signal values (r << 16) + value
   DrainKernel kernel = nullptr;
@@ -99,6 +102,12 @@ struct Graph {
   std::vector<int> topo;             // a topological order of the ops
   std::vector<unsigned char> part_edge;  // per dependency, in descs order: met part by part
   std::vector<unsigned char> part_eligible;  // per op: its dependencies may be met part by part
+  // chains (plan_chains): what the arena was built with; graph_rebind compares
+  std::vector<int> n_succ;                 // per op: ops that depend on it
+  std::vector<unsigned char> order_touch;  // per op: takes part in a NOTIFY -> GET_NOTIFIED ordering edge
+  std::vector<int> chain_words;            // kChainWords ints per op, as uploaded
+  std::vector<int> fixed_parts;            // build_graph: cut the ops like this instead of choosing (a rebuild in place:
+                                           // the arena's layout, and with it its size, follows from the part counts)
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
   bool as_launches = false;
   std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
@@ -326,6 +335,112 @@ bool plan_launches(const std::vector<pccl_op_desc> &ops, std::vector<pccl_op_des
   return take;
 }
 
+// ---- chains -------------------------------------------------------------------
+// B follows A in a chain when B depends on A alone, A is needed by B alone, both are cut alike and
+// part p of B may start as soon as part p of A is complete (single-part ops: always; otherwise the
+// part-by-part rule above).  Such a B gets no queue entries of its own: the workgroup that has run
+// part p of A goes on with part p of B, and so on down the chain.  Nothing is claimed, counted,
+// signalled or polled between the steps.  The chain's head carries the head's dependencies and the
+// tail's successors; when its last part is done every op of the chain is complete.  (A ring
+// all-reduce over ranks that live on one device is such chains, 14 ops long.)
+// Two ways to run a chain's part (graph_queue_device.h): op after op through memory (a barrier
+// between them), or, where every later op takes the previous op's output 0 as one of at most two
+// inputs and reads nothing else that the chain writes, in one pass with the value handed on in
+// registers ("forward").  (Packs are 16-byte aligned on the first op's output 0; the other operands
+// may sit at any element-aligned address, as for any part in this kernel.)
+// Returns kChainWords ints per op.
+std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
+                             const std::vector<unsigned char> &part_edge, const std::vector<int> &n_succ,
+                             const std::vector<unsigned char> &order_touch) {
+  const int n_ops = (int)ops.size();
+  std::vector<int> words((size_t)kChainWords * (size_t)std::max(n_ops, 1), 0);
+  std::vector<int> next(n_ops, -1), prev(n_ops, -1);
+  bool on = true, forward_on = true;
+  if (const char *env = getenv("PCCL_HIP_CHAINS")) on = env[0] != '0', forward_on = env[0] != '1' || env[1] != 'm';  // "1m": through memory only
+  auto is_data = [&](int i) { return ops[i].primitive != PCCL_NOTIFY && ops[i].primitive != PCCL_GET_NOTIFIED; };
+  auto bytes_of = [&](int i) { return (uintptr_t)ops[i].count * (uintptr_t)elem_bytes(ops[i].dtype); };
+  size_t at = 0;
+  for (int i = 0; i < n_ops; ++i) {
+    const size_t first_dep = at;
+    at += (size_t)ops[i].n_deps;
+    if (!on || ops[i].n_deps != 1 || order_touch[i] || !is_data(i)) continue;
+    const int a = ops[i].deps[0];
+    if (n_succ[a] != 1 || order_touch[a] || !is_data(a) || parts[a] != parts[i]) continue;
+    if (ops[a].count != ops[i].count || elem_bytes(ops[a].dtype) != elem_bytes(ops[i].dtype)) continue;
+    if (parts[i] > 1 && !part_edge[first_dep]) continue;
+    next[a] = i;
+    prev[i] = a;
+  }
+  for (int i = 0; i < n_ops; ++i) {
+    words[(size_t)kChainWords * i + kChainNext] = next[i];
+    words[(size_t)kChainWords * i + kChainLength] = 1;
+  }
+  int listed = 0;
+  for (int h = 0; h < n_ops; ++h) {
+    if (prev[h] >= 0 || next[h] < 0) continue;
+    std::vector<int> steps;
+    for (int u = h; u >= 0; u = next[u]) steps.push_back(u);
+    words[(size_t)kChainWords * h + kChainLength] = (int)steps.size();
+    // can the values be handed on in registers?
+    bool forward = forward_on && (int)steps.size() <= kMaxForwardSteps && ops[h].n_in <= 2;
+    for (int t : steps) forward = forward && ops[t].n_out <= 2;
+    const uintptr_t len = bytes_of(h);
+    std::vector<int> fed(steps.size(), 0);
+    for (size_t s = 0; forward && s < steps.size(); ++s) {
+      const pccl_op_desc &o = ops[steps[s]];
+      if (s == 0 || !forward) continue;
+      const void *handed = ops[steps[s - 1]].outs[0];
+      if (o.n_in > 2) { forward = false; break; }
+      int f = -1;
+      for (int k = 0; k < o.n_in; ++k)
+        if (o.ins[k] == handed && f < 0) f = k;
+      if (f < 0) { forward = false; break; }
+      fed[s] = f;
+      // whatever else the op reads must be something the chain never writes
+      for (int k = 0; k < o.n_in && forward; ++k) {
+        if (k == f) continue;
+        for (int t : steps)
+          for (int j = 0; j < ops[t].n_out && forward; ++j) {
+            const uintptr_t x = (uintptr_t)o.ins[k], y = (uintptr_t)ops[t].outs[j];
+            if (x < y + len && y < x + len) forward = false;
+          }
+      }
+    }
+    // ... and the first op's inputs too (an in-place first op is fine: it reads before it writes, pack by pack)
+    for (int k = 0; forward && k < ops[h].n_in; ++k)
+      for (size_t s = 1; s < steps.size() && forward; ++s)
+        for (int j = 0; j < ops[steps[s]].n_out && forward; ++j) {
+          const uintptr_t x = (uintptr_t)ops[h].ins[k], y = (uintptr_t)ops[steps[s]].outs[j];
+          if (x < y + len && y < x + len) forward = false;
+        }
+    if (forward) {
+      words[(size_t)kChainWords * h + kChainForward] = 1;
+      words[(size_t)kChainWords * h + kChainRow] = listed;  // first of its rows in the chain table (fill_chain_table)
+      listed += (int)steps.size();
+      for (size_t s = 1; s < steps.size(); ++s) words[(size_t)kChainWords * steps[s] + kChainForward] = fed[s];
+    }
+  }
+  return words;
+}
+
+// The rows of GraphControl::chain_table, from the payloads as they stand in the host image: for
+// every chain that runs in one pass, in op order of the heads, one row per op of the chain.
+void fill_chain_table(const std::vector<int> &words, int n_ops, const char *payloads, ForwardStep *rows) {
+  for (int h = 0; h < n_ops; ++h) {
+    if (!words[(size_t)kChainWords * h + kChainForward] || words[(size_t)kChainWords * h + kChainLength] < 2) continue;
+    ForwardStep *row = rows + words[(size_t)kChainWords * h + kChainRow];
+    for (int u = h; u >= 0; u = words[(size_t)kChainWords * u + kChainNext], ++row) {
+      const pccl_op_payload *pl = (const pccl_op_payload *)(payloads + kPayloadStride * (size_t)u);
+      const int fed = u == h ? 0 : words[(size_t)kChainWords * u + kChainForward];
+      row->fed = fed;
+      row->other = (u != h && pl->n_in_ == 2) ? (unsigned long long)(uintptr_t)pl->chunks_[1 - fed].addr_ : 0ull;
+      row->n_out = pl->n_out_;
+      row->out[0] = (unsigned long long)(uintptr_t)pl->chunks_[pl->n_in_].addr_;
+      row->out[1] = pl->n_out_ > 1 ? (unsigned long long)(uintptr_t)pl->chunks_[pl->n_in_ + 1].addr_ : 0ull;
+    }
+  }
+}
+
 // What pccl_hip_reduce_copy would refuse about a planned launch's operands, found at creation time.
 int check_launch(const pccl_op_desc &o) {
   const int es = elem_bytes(o.dtype);
@@ -503,6 +618,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
   }
   // ---- parts ------------------------------------------------------------------
+  std::vector<int> parts_by_level;  // the built-in choice for ops outside chains
   // A given tile_bytes cuts every op into parts of that size.  The built-in choice works per
   // dependency level and grows with the bytes the level writes: part = 16 KiB x (level bytes /
   // 8 MiB)^(2/3), within 8 KiB .. 128 KiB (for the 768 workgroups an MI355X holds of this kernel;
@@ -517,15 +633,30 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   {
     std::vector<long long> level_bytes(n_ops + 1, 0);
     for (int i = 0; i < n_ops; ++i) level_bytes[level[i]] += op_bytes[i];
+    parts_by_level.assign(n_ops, 1);
+    const long long most_bytes = *std::max_element(level_bytes.begin(), level_bytes.end());
     for (int i = 0; i < n_ops; ++i) {
-      long part_bytes = tile_bytes;
-      if (default_tile) {
-        const double want = 16384.0 * std::pow((double)level_bytes[level[i]] / (double)(8 << 20), 2.0 / 3.0) * (768.0 / (double)cap);
-        part_bytes = (long)std::min<long long>(std::max<long long>(((long long)want + 4095) / 4096 * 4096, 8 << 10), 128 << 10);
+      if (!G->fixed_parts.empty()) {
+        parts[i] = G->fixed_parts[i];
+        tiles += parts[i];
+        continue;
       }
-      long p = (op_bytes[i] + part_bytes - 1) / part_bytes;
-      if (default_tile) p = std::min<long>(p, (long)cap);
-      parts[i] = (int)std::max<long>(1, std::min<long>(p, 1 << 20));
+      long part_bytes = tile_bytes, even_bytes = tile_bytes;
+      if (default_tile) {
+        auto rule = [&](long long bytes) {
+          const double want = 16384.0 * std::pow((double)bytes / (double)(8 << 20), 2.0 / 3.0) * (768.0 / (double)cap);
+          return (long)std::min<long long>(std::max<long long>(((long long)want + 4095) / 4096 * 4096, 8 << 10), 128 << 10);
+        };
+        part_bytes = rule(level_bytes[level[i]]);
+        even_bytes = rule(most_bytes);
+      }
+      auto cut = [&](long bytes) {
+        long p = (op_bytes[i] + bytes - 1) / bytes;
+        if (default_tile) p = std::min<long>(p, (long)cap);
+        return (int)std::max<long>(1, std::min<long>(p, 1 << 20));
+      };
+      parts_by_level[i] = cut(part_bytes);
+      parts[i] = cut(even_bytes);  // one size for every level until the chains are known (below): ops of equal length cut alike
       tiles += parts[i];
     }
     if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
@@ -577,6 +708,88 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->parts = parts;
   G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
   G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
+  // ---- chains (plan_chains) ------------------------------------------------------
+  G->n_succ = n_succ;
+  G->order_touch.assign(n_ops, 0);
+  for (int i = 0; i < n_ops; ++i) G->order_touch[i] = order_pred[i] != 0 || !order_succ[i].empty();
+  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch);
+  std::vector<int> chain_prev(n_ops, -1), chain_tail(n_ops, 0);
+  auto link_chains = [&] {
+    std::fill(chain_prev.begin(), chain_prev.end(), -1);
+    for (int i = 0; i < n_ops; ++i) {
+      const int nx = G->chain_words[(size_t)kChainWords * i + kChainNext];
+      if (nx >= 0) chain_prev[nx] = i;
+    }
+    for (int i = 0; i < n_ops; ++i) {
+      int t = i;
+      while (G->chain_words[(size_t)kChainWords * t + kChainNext] >= 0) t = G->chain_words[(size_t)kChainWords * t + kChainNext];
+      chain_tail[i] = t;  // (only read for ops that have entries)
+    }
+  };
+  link_chains();
+  // A part of a chain costs its workgroup some 20 us whatever its size (every op of the chain waits
+  // for the loads and stores of the one before), and the chain's ops queue no entries of their own
+  // that could fill the gaps when the resident workgroups finish a round unevenly.  So the built-in
+  // choice cuts a level whose entries start chains differently: the smallest part (4 KiB steps from
+  // 8 KiB) with which the level's entries fit the resident workgroups once - twice and so on from
+  // 96 KiB a part.  Measured on ring all-reduces over 8 virtual ranks, each a chain of 14 ops per
+  // rank: 64 MiB 315 us with the 64 KiB parts of the rule above (1.33 rounds), 252 us with 96 KiB
+  // (0.9), 264 us with 128 KiB (0.67); 16 MiB 86 -> 79.5 us; 4096-op schedule (288 chains, 64 single ops) 150 -> 133 us.
+  if (default_tile && G->fixed_parts.empty()) {
+    bool recut = false;
+    std::vector<char> settled(n_ops, 0);
+    std::vector<std::vector<int>> at_level(n_ops + 1);
+    for (int i = 0; i < n_ops; ++i)
+      if (chain_prev[i] < 0) at_level[level[i]].push_back(i);
+    for (const std::vector<int> &members : at_level) {
+      bool heads = false;
+      long long bytes = 0;
+      for (int i : members) {
+        heads = heads || G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0;
+        bytes += op_bytes[i];
+      }
+      if (!heads) continue;
+      const long long rounds = std::max<long long>(1, (bytes + (long long)cap * (96 << 10) - 1) / ((long long)cap * (96 << 10)));
+      long part_bytes = 8 << 10;
+      for (;; part_bytes += 4 << 10) {
+        long long entries = 0;
+        for (int i : members) entries += std::max<long long>(1, (op_bytes[i] + part_bytes - 1) / part_bytes);
+        if (entries <= rounds * (long long)cap || part_bytes >= (1 << 20)) break;
+      }
+      for (int i : members) {
+        const int p = (int)std::max<long long>(1, std::min<long long>((op_bytes[i] + part_bytes - 1) / part_bytes, cap));
+        for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext]) {
+          recut = recut || parts[u] != p;
+          parts[u] = p;
+          settled[u] = 1;
+        }
+      }
+    }
+    for (int i = 0; i < n_ops; ++i)
+      if (!settled[i]) {
+        recut = recut || parts[i] != parts_by_level[i];
+        parts[i] = parts_by_level[i];
+      }
+    if (recut) {
+      tiles = 0;
+      for (int i = 0; i < n_ops; ++i) tiles += parts[i];
+      long long t = 0;
+      for (int idx = 0; idx < n_ops; ++idx) {
+        first_entry[by_level[idx]] = (int)t;
+        t += parts[by_level[idx]];
+      }
+      G->parts = parts;
+      G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
+      G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
+      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch);
+      link_chains();
+    }
+  }
+  auto queued = [&](int i) { return chain_prev[i] < 0; };  // has entries of its own
+  long long live_tiles = 0;
+  for (int i = 0; i < n_ops; ++i)
+    if (queued(i)) live_tiles += parts[i];
+
   std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
   {
     size_t at = 0;
@@ -602,6 +815,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   const size_t off_opptr = off;   off = align_up(off + sizeof(void *) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_hdr = off;     off = align_up(off + sizeof(pccl_operation_layout_header) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_payload = off; off = align_up(off + kPayloadStride * (size_t)std::max(n_ops, 1), 256);
+  // (the chain table follows the payloads directly: graph_rebind uploads the two as one block)
+  const size_t off_chain_table = off; off = align_up(off + sizeof(ForwardStep) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_succ = off;    off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_succ_part = off; off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_hot = off;     off = align_up(off + sizeof(HotWord) * kHotWords, 256);
@@ -611,6 +826,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   const size_t off_gbase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_ebase = off;   off = align_up(off + sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_groups = off;  off = align_up(off + sizeof(HotWord) * (size_t)kPartGroups * (size_t)std::max(n_grouped, 1), 256);
+  const size_t off_chain = off;   off = align_up(off + kChainWords * sizeof(int) * (size_t)std::max(n_ops, 1), 256);
   // One word per entry, 64 bytes apart: a word is polled by the workgroup that holds its entry
   // and bumped by others.  Packed 32 to a 128-byte line they cost more than the part-by-part
   // hand-over saves (ring all-reduce of 8 x 1 MiB: 82 us against 76 us with whole-op waits;
@@ -623,11 +839,16 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   if (part_words) off = align_up(off + (sizeof(unsigned int) << part_shift) * (size_t)(tiles + kQueues), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
-  const size_t off_entries = off; off = align_up(off + 8 * (size_t)std::max<long long>(tiles, 1) + 8 * kQueues, 256);
+  const size_t off_qcount = off;  off = align_up(off + sizeof(int) * kQueues, 256);
+  // room for an entry per part of every op, an equal share per queue: where the queues start must not
+  // depend on how many entries the chains leave to be queued (graph_rebind can change that)
+  const size_t queue_room = (size_t)((std::max<long long>(tiles, 1) + kQueues - 1) / kQueues);
+  const size_t off_entries = off; off = align_up(off + 8 * queue_room * kQueues, 256);
   const size_t arena_bytes = off;
 
   G->n_ops = n_ops;
-  G->total_tiles = (int)tiles;
+  G->total_tiles = (int)live_tiles;  // entries that are queued; the arena has room for an entry per part of every op
+  G->all_tiles = (int)tiles;
   G->payload_off = off_payload;
   G->kernel = kernel;
   if (hipGetDevice(&G->device) != hipSuccess) return fail(PCCL_ERR_NO_DEVICE, "no current device");
@@ -684,7 +905,11 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     }
   }
   C->spin_limit = G->spin_limit;
-  C->total_tiles = (int)tiles;
+  C->queue_count = (const int *)(dev + off_qcount);
+  C->chain = (const int *)(dev + off_chain);
+  C->chain_table = (const ForwardStep *)(dev + off_chain_table);
+  G->chain_table_off = off_chain_table;
+  memcpy(img + off_chain, G->chain_words.data(), sizeof(int) * G->chain_words.size());
   hot[kHotCompleted].value = 0;
   hot[kHotTotal].value = (unsigned int)n_ops;
   hot[kHotRun].value = run_number;
@@ -700,6 +925,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       for (int first = 0; first < most; first += block)
         for (int idx = lo; idx < hi; ++idx) {
           const int i = by_level[idx];
+          if (!queued(i)) continue;  // runs behind its chain's head
           for (int p = first; p < std::min(first + block, parts[i]); ++p, ++t)
             qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32));
         }
@@ -707,13 +933,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     }
   }
   {
-    size_t pos = off_entries;
     for (int q = 0; q < kQueues; ++q) {
+      const size_t pos = off_entries + 8 * queue_room * (size_t)q;
       ((pccl_ring_buffer **)(img + off_qptr))[q] = (pccl_ring_buffer *)(dev + off_ring + 256 * (size_t)q);
       pccl_ring_buffer *R = (pccl_ring_buffer *)(img + off_ring + 256 * (size_t)q);
       C->queue_head[q] = &((pccl_ring_buffer *)(dev + off_ring + 256 * (size_t)q))->head_;
       C->queue_entries[q] = (const unsigned long long *)(dev + pos);
-      C->queue_count[q] = (int)qe[q].size();
+      ((int *)(img + off_qcount))[q] = (int)qe[q].size();
       R->producer_ = 0;  // executor ids are the host layer's; one executor fills and drains
       R->consumer_ = 0;
       R->elem_size_ = (int)sizeof(pccl_queue_entry);
@@ -724,7 +950,6 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       R->producer_buffer_ = dev + pos;
       R->consumer_buffer_ = dev + pos;
       if (!qe[q].empty()) memcpy(img + pos, qe[q].data(), 8 * qe[q].size());
-      pos += 8 * qe[q].size();
     }
   }
 
@@ -743,8 +968,9 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     h->op_buffer_ = dev + off_payload + kPayloadStride * (size_t)i;
     h->next_op_uids_head_ = (int *)(dev + off_succ) + succ_start[i];
     PayloadSlot *slot = (PayloadSlot *)(img + off_payload + kPayloadStride * (size_t)i);
+    const int tail = chain_tail[i];  // (the op itself unless it heads a chain)
     slot->parts = parts[i];
-    slot->succ_start = succ_start[i];
+    slot->succ_start = succ_start[tail];
     pccl_op_payload *pl = &slot->payload;
     pl->primitive_ = o.primitive;
     pl->compute_ = o.compute;
@@ -752,16 +978,18 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     pl->n_out_ = o.n_out;
     pl->pre_dependencies_ = h->pre_dependencies_;
     pl->part_preds_ = (unsigned char)n_part_pred[i];
-    pl->part_nexts_ = (unsigned char)n_part_next[i];
-    pl->num_next_ops_ = h->num_next_ops_;
+    pl->part_nexts_ = (unsigned char)n_part_next[tail];
+    pl->num_next_ops_ = (unsigned char)n_succ[tail];
     // signal ops: the only operand is the signal word, num_elems_ carries the value
     for (int k = 0; k < o.n_in; ++k) pl->chunks_[k] = pccl_chunk_meta{o.dtype, (void *)o.ins[k], o.count};
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
   }
+  fill_chain_table(G->chain_words, n_ops, img + off_payload, (ForwardStep *)(img + off_chain_table));
   if (n_edges) memcpy(img + off_succ, succ.data(), sizeof(int) * n_edges);
   if (n_edges) memcpy(img + off_succ_part, succ_part_base.data(), sizeof(int) * n_edges);
   // never more workgroups than entries
-  G->n_wg = (int)std::max<long long>(1, std::min<long long>(tiles, cap));
+  // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
+  G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
 
   e = fixed ? hipMemcpyAsync(dev, img, arena_bytes, hipMemcpyHostToDevice, fixed->stream)
             : hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
@@ -891,7 +1119,8 @@ int pccl_hip_graph_trace(void *graph, int enable) {
   GraphControl *C = (GraphControl *)G->image.data();
   G->trace_on = enable != 0;
   if (!enable) { C->trace = nullptr; return PCCL_OK; }  // the buffer stays until the graph is destroyed
-  const size_t bytes = sizeof(unsigned long long) * kTraceWords * (size_t)std::max(G->total_tiles, 1);
+  // (room for a record per part of every op: a rebind may change how many of them are queued)
+  const size_t bytes = sizeof(unsigned long long) * kTraceWords * (size_t)std::max(G->all_tiles, 1);
   if (!G->trace) {
     hipError_t e = hipMalloc((void **)&G->trace, bytes);
     if (e != hipSuccess) {
@@ -997,7 +1226,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // contents are built again from the moved ops, in place (its layout does not depend on
   // addresses, and launches recorded by stream capture point at it); earlier runs on `stream`
   // finish first.  Only a failed upload can leave the graph unusable.
-  if (classify_dependencies(next, G->parts, G->topo, &G->part_eligible) != G->part_edge) {
+  // ... and so does which ops run as chains behind each other, and how (plan_chains).
+  const std::vector<unsigned char> edges_after = classify_dependencies(next, G->parts, G->topo, &G->part_eligible);
+  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
     fresh.descs.swap(next);
@@ -1005,6 +1236,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.trace = G->trace;
     fresh.trace_on = G->trace_on;
     fresh.spin_limit = G->spin_limit;
+    fresh.fixed_parts = G->parts;
+    fresh.fixed_n_wg = G->n_wg;
     char *old_dev = G->dev;
     // The run number goes on from where the DEVICE stands, not from the count of graph_run
     // calls: every replay of a recorded launch has moved the device's word on as well, and a
@@ -1023,7 +1256,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->arena_bytes = fresh.arena_bytes;
     G->image.swap(fresh.image);
     G->payload_off = fresh.payload_off;
+    G->chain_table_off = fresh.chain_table_off;
     G->total_tiles = fresh.total_tiles;
+    G->all_tiles = fresh.all_tiles;
     G->n_wg = fresh.n_wg;
     G->device = fresh.device;
     G->kernel = fresh.kernel;
@@ -1032,6 +1267,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->topo.swap(fresh.topo);
     G->part_edge.swap(fresh.part_edge);
     G->part_eligible.swap(fresh.part_eligible);
+    G->n_succ.swap(fresh.n_succ);
+    G->order_touch.swap(fresh.order_touch);
+    G->chain_words.swap(fresh.chain_words);
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
@@ -1044,7 +1282,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   }
   // ordered after earlier runs on `stream`; the source is pageable host memory,
   // so the call returns once the bytes are staged
-  PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->payload_off, payloads, kPayloadStride * (size_t)G->n_ops,
+  fill_chain_table(G->chain_words, G->n_ops, payloads, (ForwardStep *)(G->image.data() + G->chain_table_off));
+  PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->payload_off, payloads,
+                                G->chain_table_off + sizeof(ForwardStep) * (size_t)G->n_ops - G->payload_off,
                                 hipMemcpyHostToDevice, (hipStream_t)stream));
   return PCCL_OK;
 }

@@ -46,11 +46,14 @@ struct GraphControl {
                                           // part-by-part dependencies that have arrived
   int part_shift;
   const int *succ_part_base;              // beside succ: entry index of part 0 of a successor released part by part
+  const int *chain;                       // per op, kChainWords ints: see kChain* below
+  const struct ForwardStep *chain_table;  // one row per op of every forward chain, chain after chain
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
-  int queue_count[kQueues];
+  const int *queue_count;                 // entries on each queue: in memory, not here, because which ops queue entries
+                                          // (chains do not) can change with the operands' addresses, and what is in
+                                          // this block is frozen into any launch that a stream capture has recorded
   unsigned int spin_limit;
-  int total_tiles;
 };
 
 // An op of many parts does not count them on one word: atomics on one address are carried out
@@ -61,6 +64,17 @@ struct GraphControl {
 // which for these ops starts at kPartGroups instead of required_executors_.
 constexpr int kPartGroups = 8;
 constexpr int kGroupThreshold = 16;
+
+// Chains (ops that run behind another op in the same workgroup, part by part): per op
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+constexpr int kChainWords = 4;
+constexpr int kChainNext = 0;     // the op that runs behind this one, or -1
+constexpr int kChainLength = 1;   // for the op a chain starts with: ops in it (1 for an op outside any chain)
+constexpr int kChainForward = 2;  // head: 1 if the whole chain runs in one pass with values handed on in registers
+                                  // (run_chain_forward); another op of such a chain: which of its inputs is the
+                                  // previous op's output 0
+constexpr int kChainRow = 3;      // head of a forward chain: its first row in GraphControl::chain_table
+constexpr int kMaxForwardSteps = 16;
 
 // indices into GraphControl::hot
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
@@ -241,6 +255,151 @@ __device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, long lo,
   }
 }
 
+// ---- a whole chain in one pass -----------------------------------------------------
+// For chains in which every op after the first reads the previous op's output 0 as one of at most two
+// inputs (a ring step: what the neighbour produced, plus the local chunk; or a plain copy of it) and nothing
+// else of the chain's outputs is read inside the chain: the value a lane has just stored is the value the
+// next op would load, so it stays in registers.  Packs are cut so that the first op's output 0 is 16-byte
+// aligned; the other operands are read and written at whatever element-aligned address that gives them.
+// Per pack a lane loads the first op's inputs and every later op's other input up front (they depend on
+// nothing), then folds and stores op after op.  The 14-op chain of a ring all-reduce over 8 resident
+// ranks reads 8 packs and writes 14 instead of reading 21 and writing 14, with no store -> load round
+// trip between the steps.  Bit for bit what the ops give one after the other: each step rounds to the
+// element type exactly where the store would.
+template <class D, class Op>
+__device__ __forceinline__ u32x4 fold_two(const u32x4 &a, const u32x4 &b) {
+  const u32x4 v[2] = {a, b};
+  return fold_pack<D, Op, 2>(v);
+}
+
+// What the pass needs to know of one op of the chain.  The host keeps a table of these rows beside the
+// payloads (and moves the addresses with them on a rebind); a part stages its chain's rows in LDS with
+// one load per lane.  Walking the chain op by op through the payloads costs three dependent loads per
+// op (next op, its payload, the operand address): 2 us per op on an idle device, more under load, and
+// that was all the time the pass took.
+struct ForwardStep {
+  unsigned long long other;   // the input that is not handed on (ops after the first with two inputs), else 0
+  unsigned long long out[2];  // outputs
+  int n_out;
+  int fed;                    // which input the handed-on value is (two-input ops after the first)
+};
+static_assert(sizeof(ForwardStep) == 32, "two 16-byte loads per row");
+
+__device__ __forceinline__ unsigned long long uniform64(unsigned long long v) {  // the same in every lane: into scalar registers
+  const unsigned int lo = __builtin_amdgcn_readfirstlane((unsigned int)v), hi = __builtin_amdgcn_readfirstlane((unsigned int)(v >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+template <class D, class Op>
+__device__ __forceinline__ void run_chain_forward(const GraphControl &g, const pccl_op_payload *hp, int n_steps, int first_row, long lo, long count) {
+  typedef typename D::elem_t E;
+  constexpr int kEpp = 16 / D::kElemBytes;
+  constexpr int kBatch = 2;  // packs a lane carries through the chain at a time (8 KiB per workgroup and stream)
+  constexpr int kAhead = 8;  // ops whose other input is requested ahead of the value reaching them
+  __shared__ __attribute__((aligned(16))) ForwardStep s_step[kMaxForwardSteps];
+  const int head_n_in = hp->n_in_;
+  if (threadIdx.x < 2u * (unsigned)n_steps)  // two lanes per row
+    ((u32x4 *)s_step)[threadIdx.x] = ((const u32x4 *)(g.chain_table + first_row))[threadIdx.x];
+  __syncthreads();
+  // the elements before output 0's first 16-byte boundary are left to the edge code below
+  const unsigned long long out0 = (unsigned long long)hp->chunks_[head_n_in].addr_ + (unsigned long long)lo * D::kElemBytes;
+  long peel = (long)((16 - (out0 & 15)) & 15) / D::kElemBytes;
+  if (peel > count) peel = count;
+  const long n_packs = (count - peel) / kEpp;
+  const size_t body = (size_t)(lo + peel) * D::kElemBytes;  // byte offset of the first pack from every operand's base
+  for (long base = 0; base < n_packs; base += (long)kBlock * kBatch) {
+    const size_t chunk = body + (size_t)base * 16;  // uniform
+    const long left = n_packs - base;               // packs from here on; the lane's pack u exists if threadIdx.x + u * kBlock < left
+    unsigned int off[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const long q = (long)threadIdx.x + (long)u * kBlock;
+      off[u] = (unsigned int)((q < left ? q : left - 1) * 16);  // a lane without pack u re-reads the last pack and stores nothing for it
+    }
+    // The loads of a chain depend on nothing the chain computes, so they go out well ahead of the
+    // value: the first op's inputs and the other input of the ops among the next kAhead that have one,
+    // together (up to 18 packs per lane in flight), then fold and store op after op, then the next
+    // kAhead.  Loads never stand behind stores in the wavefront's queue (its wait counter treats
+    // completion as in order, and a write-through store's acknowledgement takes microseconds).
+    u32x4 cur[kBatch], in1[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      cur[u] = load_pack<D, true, kMemCoherent>((const char *)hp->chunks_[0].addr_ + chunk, off[u]);
+      if (head_n_in == 2) in1[u] = load_pack<D, true, kMemCoherent>((const char *)hp->chunks_[1].addr_ + chunk, off[u]);
+    }
+    for (int s0 = 0; s0 < n_steps; s0 += kAhead) {
+      u32x4 other[kAhead][kBatch];
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        const int s = s0 + i;
+        if (s == 0 || s >= n_steps) continue;
+        const unsigned long long from = uniform64(s_step[s].other);
+        if (from == 0ull) continue;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) other[i][u] = load_pack<D, true, kMemCoherent>((const char *)from + chunk, off[u]);
+      }
+      if (s0 == 0 && head_n_in == 2) {
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) cur[u] = fold_two<D, Op>(cur[u], in1[u]);
+      }
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        const int s = s0 + i;
+        if (s >= n_steps) continue;
+        if (s > 0 && uniform64(s_step[s].other) != 0ull) {
+          const int fed = __builtin_amdgcn_readfirstlane(s_step[s].fed);
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u) cur[u] = fed == 0 ? fold_two<D, Op>(cur[u], other[i][u]) : fold_two<D, Op>(other[i][u], cur[u]);
+        }
+        const int n_out = __builtin_amdgcn_readfirstlane(s_step[s].n_out);
+        for (int j = 0; j < n_out; ++j) {
+          char *to = (char *)uniform64(s_step[s].out[j]) + chunk;
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u)
+            if ((long)threadIdx.x + (long)u * kBlock < left) store_pack<D, true, kMemCoherent>(to, off[u], cur[u]);
+        }
+      }
+    }
+  }
+  // the elements before the first pack and behind the last one (fewer than two packs' worth): one per
+  // lane of the last wavefront, again with every load ahead of the first store
+  if (threadIdx.x >= kBlock - kWave) {
+    const long tail_begin = peel + n_packs * kEpp, n_edge = peel + (count - tail_begin);
+    const long e = (long)threadIdx.x - (kBlock - kWave);
+    if (e < n_edge) {
+      const long i = lo + (e < peel ? e : tail_begin + (e - peel));
+      E cur = load_elem<E, kMemCoherent>((const E *)hp->chunks_[0].addr_ + i), second = cur;
+      if (head_n_in == 2) second = load_elem<E, kMemCoherent>((const E *)hp->chunks_[1].addr_ + i);
+      E other[kMaxForwardSteps];
+#pragma unroll
+      for (int s = 1; s < kMaxForwardSteps; ++s) {
+        other[s] = cur;
+        if (s >= n_steps) continue;
+        const unsigned long long from = uniform64(s_step[s].other);
+        if (from != 0ull) other[s] = load_elem<E, kMemCoherent>((const E *)from + i);
+      }
+      if (head_n_in == 2) {
+        const E x[2] = {cur, second};
+        cur = D::template elem<Op, 2>(x);
+      }
+#pragma unroll
+      for (int s = 0; s < kMaxForwardSteps; ++s) {
+        if (s >= n_steps) continue;
+        if (s > 0 && uniform64(s_step[s].other) != 0ull) {
+          const int fed = __builtin_amdgcn_readfirstlane(s_step[s].fed);
+          E x[2];
+          x[fed] = cur;
+          x[1 - fed] = other[s];
+          cur = D::template elem<Op, 2>(x);
+        }
+        const int n_out = __builtin_amdgcn_readfirstlane(s_step[s].n_out);
+        for (int j = 0; j < n_out; ++j) store_elem<E, kMemCoherent>((E *)uniform64(s_step[s].out[j]) + i, cur);
+      }
+    }
+  }
+  settle_stores();
+}
+
 #define AGENT __HIP_MEMORY_SCOPE_AGENT
 
 // Trace record of a queue entry (entry t of queue q is record t * kQueues + q), times in ticks
@@ -277,7 +436,7 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // behind the ticket (memory operations of a wavefront return in order).
 template <class DrawTicket>
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const OpFacts &op, int uid, int part, int home,
+                                            const OpFacts &op, int uid, int part, int home, int chain_ops,
                                             DrawTicket draw_ticket) {
   const int parts = op.parts;
   // successors that need only this part of the op (they come first in the successor list):
@@ -323,13 +482,15 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   const int *next = g.succ + op.succ_start;
   for (int s = n_part_next; s < n_next; ++s)
     __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
-  __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, 1u, __ATOMIC_RELAXED, AGENT);
+  // (an op that heads a chain stands for all the chain's ops: they ran behind it, part by part)
+  __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, (unsigned int)chain_ops, __ATOMIC_RELAXED, AGENT);
   if (!drawn) draw_ticket();
 }
 
 template <int DT, class Op>
-__global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3))) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
   __shared__ unsigned long long s_entry;
+  __shared__ i32x4 s_chain;  // the claimed op's kChainWords words
   __shared__ int s_go;
   __shared__ int s_last;
   if constexpr (DT != kAnyDtype) Dtype<DT>::wave_init();
@@ -348,6 +509,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
   const PayloadSlot *slot = nullptr;
   int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
   OpFacts cur_op = {1, 0, 0};     // ... and its op's facts (uniform)
+  int cur_chain_ops = 1;          // ... and how many ops it stands for: the chain it heads, or itself
   unsigned long long *cur_trace = nullptr;  // its trace record (thread 0 only)
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   // Signal values are offset by (run number << 16).  The run number lives on the device (not
@@ -367,6 +529,9 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
       int first_q = -1, first_t = 0;
       unsigned int aborted = 0;
       auto draw_ticket = [&] {
+        // (the workgroup's very first ticket does not wait for the queue lengths to arrive from memory:
+        // there are no more workgroups than entries at creation, so its home queue has one for it)
+        if (!h) first_q = home;
         for (int i = 0; i < kQueues && first_q < 0; ++i) {
           const int q = (home + i) % kQueues;
           if (!(exhausted & (1u << q)) && g.queue_count[q] > 0) first_q = q;
@@ -376,12 +541,13 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
       };
       if (h) {
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, h, cur_op, cur_uid, cur_part, home, draw_ticket);
+        finish_part(g, h, cur_op, cur_uid, cur_part, home, cur_chain_ops, draw_ticket);
       } else {
         draw_ticket();
       }
       int go = 0;
       unsigned long long e = 0;
+      i32x4 chain_words = {-1, 1, 0, 0};
       size_t entry_index = 0;  // of e in the global order
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
       // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
@@ -433,6 +599,7 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;
+        chain_words = *(const i32x4 *)(g.chain + kChainWords * uid);
         const unsigned int n_pred = (w12 & 0xffu) - part_preds;  // whole-op dependencies
         if (n_pred != 0 && arrived != n_pred &&
             !bounded_wait(abort_flag, spin_limit, [&] {
@@ -469,11 +636,12 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, hc, OpFacts::of(sc), uid, 0, home, [] {});
+        finish_part(g, hc, OpFacts::of(sc), uid, 0, home, 1, [] {});
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
       s_go = go;
+      s_chain = chain_words;
     }
     __syncthreads();
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
@@ -485,14 +653,35 @@ __global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl 
     slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
     const pccl_op_payload *pl = &slot->payload;
     cur_op = OpFacts::of(slot);
+    const int chain_next = __builtin_amdgcn_readfirstlane(s_chain[kChainNext]);
+    cur_chain_ops = __builtin_amdgcn_readfirstlane(s_chain[kChainLength]);
     const long count = pl->chunks_[0].num_elems_;
     const long per = part_elems(count, cur_op.parts);
     const long lo = (long)part * per;
     long n = count - lo;
     if (n > per) n = per;
     if (n > 0) {
-      if constexpr (DT == kAnyDtype) run_part_any(pl, lo, n);
-      else run_part<DT, Op>(pl, lo, n);
+      bool forwarded = false;
+      if constexpr (DT != kAnyDtype) {
+        // (the instance that picks the fold per op keeps to the plain chain walk below)
+        if (chain_next >= 0 && __builtin_amdgcn_readfirstlane(s_chain[kChainForward])) {
+          run_chain_forward<Dtype<DT>, Op>(g, pl, cur_chain_ops, __builtin_amdgcn_readfirstlane(s_chain[kChainRow]), lo, n);
+          forwarded = true;
+        }
+      }
+      if (!forwarded) {
+        if constexpr (DT == kAnyDtype) run_part_any(pl, lo, n);
+        else run_part<DT, Op>(pl, lo, n);
+        // The ops chained behind this one, same part: every wavefront has waited for its own stores
+        // (run_part ends that way), the barrier makes that true of the whole workgroup, and the next
+        // op's loads read past the L2 like every load here.  The chain index is uniform.
+        for (int next = chain_next; next >= 0; next = g.chain[kChainWords * next + kChainNext]) {
+          __syncthreads();
+          const pccl_op_payload *npl = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
+          if constexpr (DT == kAnyDtype) run_part_any(npl, lo, n);
+          else run_part<DT, Op>(npl, lo, n);
+        }
+      }
     }
     // every store of this part has reached the point of coherence (run_part waits)
     // before thread 0 hands the part over at the top of the next iteration; the

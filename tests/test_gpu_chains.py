@@ -1,0 +1,219 @@
+"""GPU parity of chains in the op queue: an op that depends on one op alone, which nothing else
+depends on, queues no entries of its own; the workgroup that ran part p of the first goes on with
+part p of the second.  Where every later op takes the previous op's output as one of at most two
+inputs the whole chain runs in one pass with the value handed on in registers.  Either way the
+bits are those of the ops executed one after the other by the CPU checker."""
+import numpy as np
+import pytest
+
+import helpers as H
+import schedules as S
+
+pytestmark = pytest.mark.gpu
+
+
+def _stream(torch):
+    return torch.cuda.current_stream().cuda_stream
+
+
+class Pool:
+    """Named buffers, each on the host (for the CPU checker) and on the device, at a chosen offset
+    from a 256-byte boundary."""
+
+    def __init__(self, torch, dtype):
+        self.torch, self.dtype, self.host, self.dev = torch, dtype, {}, {}
+
+    def add(self, name, count, offset=0, src=None):
+        self.host[name] = np.zeros(count, dtype=H.STORAGE[self.dtype]) if src is None else src.copy()
+        self.dev[name] = H.DevBuf(self.torch, self.dtype, count, offset, src=src)
+        return self
+
+    def ops_for(self, ops, where):
+        out = []
+        for o in ops:
+            d = dict(o, dtype=self.dtype)
+            pick = (lambda n: self.host[n][:o["count"]]) if where == "host" else (lambda n: self.dev[n].ptr)
+            d["ins"], d["outs"] = [pick(n) for n in o["ins"]], [pick(n) for n in o["outs"]]
+            out.append(d)
+        return out
+
+    def check(self, names, what):
+        for n in names:
+            H.assert_bits_equal(self.dev[n].download(), self.host[n], "%s: %s" % (what, n))
+            assert self.dev[n].guards_intact(), "%s: wrote outside %s" % (what, n)
+
+
+def _run(torch, hip, g, n_ops):
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (n_ops, n_ops)
+
+
+@pytest.mark.parametrize("dtype,compute", [("bf16", "sum"), ("f16", "max"), ("f32", "sum"), ("f64", "prod"),
+                                           ("i32", "min"), ("u32", "max"), ("f8e4m3", "sum"), ("f8e5m2", "max")])
+def test_ring_chains_in_one_pass(hip, oracle, monkeypatch, dtype, compute):
+    """Ring all-reduce over 8 virtual ranks: per chunk a chain of 14 ops (7 folds, 7 copies).  Chunk
+    sizes with elements before the first and behind the last 16-byte pack; operands 16-byte aligned
+    or not, inputs and outputs alike in their low address bits or not (down to one element);
+    several parts per op or one."""
+    import torch
+    es = H.ELEM_BYTES[dtype]
+    for sizes, offsets, tile in (([1000, 37, 20011], (0, 0), 0), ([5003, 1], (es * 3, es * 3), 0),
+                                 ([70001], (es, es), 16 << 10), ([4099], (0, max(4, es)), 8 << 10), ([3001, 50], (es, 3 * es), 0)):
+        ops, per_rank = S.ring_allreduce_ops(8, sizes, dtype=dtype, compute=compute)
+        # (values near 1 keep a product of eight of them finite)
+        kw = dict(mean=1.0, sigma=0.05) if compute == "prod" else dict(sigma=1.0)
+        host = {"in": [H.gen(dtype, per_rank, 900, r, **kw) for r in range(8)],
+                "out": [np.zeros(per_rank, dtype=H.STORAGE[dtype]) for _ in range(8)]}
+        order = oracle.topo_sort(len(ops), S.edges_of(ops))
+        oracle.run_ops(S.materialise(ops, lambda b, r, e, n: host[b][r][e:e + n]), order)
+        dev = {"in": [H.DevBuf(torch, dtype, per_rank, offsets[0], src=host["in"][r]) for r in range(8)],
+               "out": [H.DevBuf(torch, dtype, per_rank, offsets[1]) for _ in range(8)]}
+        bound = S.materialise(ops, lambda b, r, e, n: dev[b][r].ptr + e * es)
+        monkeypatch.setenv("PCCL_HIP_CHAINS", "0")
+        plain = hip.Graph(bound, tile_bytes=tile)
+        monkeypatch.setenv("PCCL_HIP_CHAINS", "1")
+        g = hip.Graph(bound, tile_bytes=tile)
+        # 14 ops share the entries of one (the built-in choice may also cut a chain into fewer parts)
+        if tile:
+            assert g.info()["n_tiles"] * 14 == plain.info()["n_tiles"], (sizes, offsets)
+        else:
+            assert g.info()["n_tiles"] * 14 <= plain.info()["n_tiles"], (sizes, offsets)
+        plain.destroy()
+        for it in range(2):
+            for b in dev["out"]:
+                b.view().fill_(0xFF)
+            _run(torch, hip, g, len(ops))
+            for r in range(8):
+                H.assert_bits_equal(dev["out"][r].download(), host["out"][r], "%s %s sizes %s offsets %s run %d rank %d"
+                                    % (dtype, compute, sizes, offsets, it, r))
+                assert dev["out"][r].guards_intact()
+        g.destroy()
+
+
+def test_two_outputs_and_value_handed_on_as_second_input(hip, oracle):
+    """t, t2 = a + b;  u = c + t (the handed-on value is input 1);  v, w = copy(u);  x = v + d."""
+    import torch
+    for count, offset in ((100003, 0), (9, 8), (3 * 1000 * 1000 + 5, 4)):
+        pool = Pool(torch, "f32")
+        for k, n in enumerate("abcd"):
+            pool.add(n, count, offset, src=H.gen("f32", count, 910, k))
+        for n in ("t", "t2", "u", "v", "w", "x"):
+            pool.add(n, count, offset)
+        ops = [dict(compute="sum", ins=["a", "b"], outs=["t", "t2"], count=count, deps=[]),
+               dict(compute="sum", ins=["c", "t"], outs=["u"], count=count, deps=[0]),
+               dict(compute="sum", ins=["u"], outs=["v", "w"], count=count, deps=[1]),
+               dict(compute="sum", ins=["v", "d"], outs=["x"], count=count, deps=[2])]
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        g = hip.Graph(pool.ops_for(ops, "dev"))
+        assert g.info()["n_tiles"] >= 1
+        _run(torch, hip, g, 4)
+        pool.check(("t", "t2", "u", "v", "w", "x"), "count %d offset %d" % (count, offset))
+        g.destroy()
+
+
+def test_chain_that_reads_what_it_wrote_earlier_goes_through_memory(hip, oracle):
+    """t = a + b;  u = t + c;  t = u + t (in place, reads op 0's output again);  v = copy(t): the ops still
+    run behind each other in one workgroup, but every op reads its inputs from memory."""
+    import torch
+    for count in (200003, 5 * 1000 * 1000 + 1):
+        pool = Pool(torch, "bf16")
+        for k, n in enumerate("abc"):
+            pool.add(n, count, 0, src=H.gen("bf16", count, 920, k))
+        for n in "tuv":
+            pool.add(n, count, 0)
+        ops = [dict(compute="sum", ins=["a", "b"], outs=["t"], count=count, deps=[]),
+               dict(compute="sum", ins=["t", "c"], outs=["u"], count=count, deps=[0]),
+               dict(compute="sum", ins=["u", "t"], outs=["t"], count=count, deps=[1]),
+               dict(compute="sum", ins=["t"], outs=["v"], count=count, deps=[2])]
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        g = hip.Graph(pool.ops_for(ops, "dev"))
+        _run(torch, hip, g, 4)
+        pool.check("tuv", "count %d" % count)
+        g.destroy()
+
+
+def test_mixed_computes_and_more_ops_than_one_pass_holds(hip, oracle):
+    """x1 = x0 + a, x2 = max(x1, b), x3 = x2 * c, ... 20 ops in a row: ops that do not share one
+    fold run in the kernel instance that picks the fold per op, which takes chains through memory;
+    the same 20 ops with one fold are more than one pass holds and go through memory as well."""
+    import torch
+    count = 50021
+    for computes in (["sum", "max", "prod", "min"] * 5, ["sum"] * 20):
+        pool = Pool(torch, "f32")
+        for k, n in enumerate("abc"):
+            pool.add(n, count, 0, src=H.gen("f32", count, 930, k, mean=1.0, sigma=0.1))
+        for k in range(21):
+            pool.add("x%d" % k, count, 0, src=H.gen("f32", count, 930, 5) if k == 0 else None)
+        ops = [dict(compute=c, ins=["x%d" % k, "abc"[k % 3]], outs=["x%d" % (k + 1)], count=count, deps=[k - 1] if k else [])
+               for k, c in enumerate(computes)]
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        g = hip.Graph(pool.ops_for(ops, "dev"), tile_bytes=64 << 10)
+        assert g.info()["n_tiles"] == 4  # one chain, four parts
+        _run(torch, hip, g, 20)
+        pool.check(["x%d" % k for k in range(1, 21)], "computes %s" % computes[:4])
+        g.destroy()
+
+
+def test_chains_between_a_fan_out_and_a_fan_in(hip, oracle):
+    """s = a + b feeds two chains of four ops each; z = (end of chain 1) + (end of chain 2).  The head of a
+    chain waits for s, and z waits for both chains' last ops."""
+    import torch
+    for count, tile in ((1000, 0), (700001, 16 << 10)):
+        pool = Pool(torch, "bf16")
+        for k, n in enumerate("abcd"):
+            pool.add(n, count, 0, src=H.gen("bf16", count, 940, k))
+        names = ["s", "z"] + ["p%d" % k for k in range(4)] + ["q%d" % k for k in range(4)]
+        for n in names:
+            pool.add(n, count, 0)
+        ops = [dict(compute="sum", ins=["a", "b"], outs=["s"], count=count, deps=[])]
+        for chain, extra in (("p", "c"), ("q", "d")):
+            for k in range(4):
+                src = "s" if k == 0 else "%s%d" % (chain, k - 1)
+                dep = 0 if k == 0 else len(ops) - 1
+                ops.append(dict(compute="sum", ins=[src, extra] if k % 2 == 0 else [src], outs=["%s%d" % (chain, k)],
+                                count=count, deps=[dep]))
+        ops.append(dict(compute="sum", ins=["p3", "q3"], outs=["z"], count=count, deps=[4, 8]))
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        g = hip.Graph(pool.ops_for(ops, "dev"), tile_bytes=tile)
+        for _ in range(3):  # the graph re-arms itself
+            for n in names:
+                pool.dev[n].view().fill_(0xFF)
+            _run(torch, hip, g, len(ops))
+            pool.check(names, "count %d" % count)
+        g.destroy()
+
+
+def test_rebind_moves_the_chains_operands(hip, oracle):
+    """A chain that runs in one pass keeps its operand addresses in a table beside the payloads;
+    graph_rebind moves both, to a buffer of the same alignment and to one 4 bytes off it."""
+    import torch
+    count = 300007
+    pool = Pool(torch, "f32")
+    for k, n in enumerate("abc"):
+        pool.add(n, count, 0, src=H.gen("f32", count, 950, k))
+    for n in ("t", "u", "v"):
+        pool.add(n, count, 0)
+    ops = [dict(compute="sum", ins=["a", "b"], outs=["t"], count=count, deps=[]),
+           dict(compute="sum", ins=["t", "c"], outs=["u"], count=count, deps=[0]),
+           dict(compute="sum", ins=["u"], outs=["v"], count=count, deps=[1])]
+    oracle.run_ops(pool.ops_for(ops, "host"))
+    g = hip.Graph(pool.ops_for(ops, "dev"))
+    entries = g.info()["n_tiles"]
+    _run(torch, hip, g, 3)
+    pool.check("tuv", "before the rebind")
+    # u moves to a fresh buffer with the same alignment, then to one 4 bytes off it
+    at = pool.dev["u"]
+    for offset in (0, 4):
+        moved = H.DevBuf(torch, "f32", count, offset)
+        g.rebind(at.ptr, moved.ptr, 4 * count, _stream(torch))
+        assert g.info()["n_tiles"] == entries
+        at.view().fill_(0x11)
+        pool.dev["v"].view().fill_(0xFF)
+        _run(torch, hip, g, 3)
+        H.assert_bits_equal(moved.download(), pool.host["u"], "u after the move (offset %d)" % offset)
+        assert moved.guards_intact()
+        pool.check("tv", "after the move (offset %d)" % offset)
+        assert (at.download().view(np.uint32) == 0x11111111).all(), "the old buffer was written after the rebind"
+        keep = at  # (alive until the next rebind has gone through)
+        at = moved
+    g.destroy()
