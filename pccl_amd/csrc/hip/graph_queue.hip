@@ -57,16 +57,16 @@ using pccl_host::fail;
 
 namespace {
 
-DrainKernel drain_for(int dtype, int compute) {
+DrainKernel drain_for(int dtype, int compute, bool forward) {
   switch (dtype) {
-    case PCCL_F32: return drain_for_compute<PCCL_F32>(compute);
-    case PCCL_I32: return drain_for_compute<PCCL_I32>(compute);
-    case PCCL_BF16: return drain_for_compute<PCCL_BF16>(compute);
-    case PCCL_F16: return drain_for_compute<PCCL_F16>(compute);
-    case PCCL_F8E4M3: return drain_for_compute<PCCL_F8E4M3>(compute);
-    case PCCL_F8E5M2: return drain_for_compute<PCCL_F8E5M2>(compute);
-    case PCCL_F64: return drain_for_compute<PCCL_F64>(compute);
-    default: return drain_for_compute<PCCL_U32>(compute);
+    case PCCL_F32: return forward ? drain_forward_for_compute<PCCL_F32>(compute) : drain_for_compute<PCCL_F32>(compute);
+    case PCCL_I32: return forward ? drain_forward_for_compute<PCCL_I32>(compute) : drain_for_compute<PCCL_I32>(compute);
+    case PCCL_BF16: return forward ? drain_forward_for_compute<PCCL_BF16>(compute) : drain_for_compute<PCCL_BF16>(compute);
+    case PCCL_F16: return forward ? drain_forward_for_compute<PCCL_F16>(compute) : drain_for_compute<PCCL_F16>(compute);
+    case PCCL_F8E4M3: return forward ? drain_forward_for_compute<PCCL_F8E4M3>(compute) : drain_for_compute<PCCL_F8E4M3>(compute);
+    case PCCL_F8E5M2: return forward ? drain_forward_for_compute<PCCL_F8E5M2>(compute) : drain_for_compute<PCCL_F8E5M2>(compute);
+    case PCCL_F64: return forward ? drain_forward_for_compute<PCCL_F64>(compute) : drain_for_compute<PCCL_F64>(compute);
+    default: return forward ? drain_forward_for_compute<PCCL_U32>(compute) : drain_for_compute<PCCL_U32>(compute);
   }
 }
 
@@ -90,6 +90,8 @@ struct Graph {
   int all_tiles = 0;            // parts of all ops (>= total_tiles: an op that runs behind another in a chain queues none)
   int n_wg = 0;
   int fixed_n_wg = 0;           // build_graph: launch this many workgroups instead of choosing
+  DrainKernel fixed_kernel = nullptr;  // build_graph: ... and this kernel instance
+  bool forward_capable = false; // the instance has the code that runs a chain in one pass
   int device = 0;
   unsigned int runs = 0;        // launches so far; run r uses signal values (r << 16) + value
   DrainKernel kernel = nullptr;
@@ -351,12 +353,12 @@ bool plan_launches(const std::vector<pccl_op_desc> &ops, std::vector<pccl_op_des
 // Returns kChainWords ints per op.
 std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
                              const std::vector<unsigned char> &part_edge, const std::vector<int> &n_succ,
-                             const std::vector<unsigned char> &order_touch) {
+                             const std::vector<unsigned char> &order_touch, bool allow_forward) {
   const int n_ops = (int)ops.size();
   std::vector<int> words((size_t)kChainWords * (size_t)std::max(n_ops, 1), 0);
   std::vector<int> next(n_ops, -1), prev(n_ops, -1);
-  bool on = true, forward_on = true;
-  if (const char *env = getenv("PCCL_HIP_CHAINS")) on = env[0] != '0', forward_on = env[0] != '1' || env[1] != 'm';  // "1m": through memory only
+  bool on = true, forward_on = allow_forward;
+  if (const char *env = getenv("PCCL_HIP_CHAINS")) on = env[0] != '0', forward_on = forward_on && (env[0] != '1' || env[1] != 'm');  // "1m": through memory only
   auto is_data = [&](int i) { return ops[i].primitive != PCCL_NOTIFY && ops[i].primitive != PCCL_GET_NOTIFIED; };
   auto bytes_of = [&](int i) { return (uintptr_t)ops[i].count * (uintptr_t)elem_bytes(ops[i].dtype); };
   size_t at = 0;
@@ -532,13 +534,22 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // copy-only graphs: element size of the ops decides nothing but alignment assumptions
   if (g_dtype < 0) { g_dtype = PCCL_BF16; g_compute = PCCL_SUM; }
   // launch width: as many workgroups as the chip holds of this kernel instance
-  const DrainKernel kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute);
-  int occ = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void *)kernel, kBlock, 0) != hipSuccess || occ < 1) {
-    (void)hipGetLastError();
-    occ = 4;
+  // (two instances per dtype and fold: with and without the code that runs a chain in one pass.  Which
+  // of them runs is settled once the chains are known, below; the launch width must hold for both.  A
+  // rebuild in place keeps the instance: launches that a stream capture has recorded carry it.)
+  const DrainKernel plain_kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute, false);
+  const DrainKernel forward_kernel = mixed ? nullptr : drain_for(g_dtype, g_compute, true);
+  const bool allow_forward = G->fixed_kernel ? G->forward_capable : !mixed;
+  int occ = 8;
+  for (DrainKernel k : {plain_kernel, forward_kernel}) {
+    if (!k) continue;
+    int o = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, (const void *)k, kBlock, 0) != hipSuccess || o < 1) {
+      (void)hipGetLastError();
+      o = 4;
+    }
+    occ = std::min(occ, o);
   }
-  occ = std::min(occ, 8);
   const long long cap = (long long)pccl_host::compute_units() * occ;
   // ---- acyclicity (Kahn) -----------------------------------------------------
   std::vector<int> succ_start(n_ops + 1, 0);
@@ -653,7 +664,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       auto cut = [&](long bytes) {
         long p = (op_bytes[i] + bytes - 1) / bytes;
         if (default_tile) p = std::min<long>(p, (long)cap);
-        return (int)std::max<long>(1, std::min<long>(p, 1 << 20));
+        return (int)std::max<long>(1, std::min<long>(p, kMaxParts));
       };
       parts_by_level[i] = cut(part_bytes);
       parts[i] = cut(even_bytes);  // one size for every level until the chains are known (below): ops of equal length cut alike
@@ -712,7 +723,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->n_succ = n_succ;
   G->order_touch.assign(n_ops, 0);
   for (int i = 0; i < n_ops; ++i) G->order_touch[i] = order_pred[i] != 0 || !order_succ[i].empty();
-  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch);
+  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, allow_forward);
   std::vector<int> chain_prev(n_ops, -1), chain_tail(n_ops, 0);
   auto link_chains = [&] {
     std::fill(chain_prev.begin(), chain_prev.end(), -1);
@@ -781,7 +792,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       G->parts = parts;
       G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
       G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
-      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch);
+      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, allow_forward);
       link_chains();
     }
   }
@@ -839,7 +850,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   if (part_words) off = align_up(off + (sizeof(unsigned int) << part_shift) * (size_t)(tiles + kQueues), 256);
   const size_t off_ring = off;    off = align_up(off + 256 * (size_t)kQueues, 256);  // one RingBuffer per 256-byte line
   const size_t off_qptr = off;    off = align_up(off + sizeof(void *) * kQueues, 256);
-  const size_t off_qcount = off;  off = align_up(off + sizeof(int) * kQueues, 256);
+  const size_t off_qcount = off;  off = align_up(off + sizeof(int) * (kQueues + 1), 256);  // queue lengths, mode word
   // room for an entry per part of every op, an equal share per queue: where the queues start must not
   // depend on how many entries the chains leave to be queued (graph_rebind can change that)
   const size_t queue_room = (size_t)((std::max<long long>(tiles, 1) + kQueues - 1) / kQueues);
@@ -850,7 +861,15 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->total_tiles = (int)live_tiles;  // entries that are queued; the arena has room for an entry per part of every op
   G->all_tiles = (int)tiles;
   G->payload_off = off_payload;
-  G->kernel = kernel;
+  if (G->fixed_kernel) {
+    G->kernel = G->fixed_kernel;
+  } else {
+    G->forward_capable = false;
+    for (int i = 0; i < n_ops && forward_kernel; ++i)
+      if (chain_prev[i] < 0 && G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 && G->chain_words[(size_t)kChainWords * i + kChainForward])
+        G->forward_capable = true;
+    G->kernel = G->forward_capable ? forward_kernel : plain_kernel;
+  }
   if (hipGetDevice(&G->device) != hipSuccess) return fail(PCCL_ERR_NO_DEVICE, "no current device");
   G->dev = nullptr;
   G->arena_bytes = arena_bytes;
@@ -927,7 +946,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
           const int i = by_level[idx];
           if (!queued(i)) continue;  // runs behind its chain's head
           for (int p = first; p < std::min(first + block, parts[i]); ++p, ++t)
-            qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32));
+            qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32) |
+                                      (G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 ? kEntryChainHead : 0ull));
         }
       lo = hi;
     }
@@ -990,6 +1010,11 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // never more workgroups than entries
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
   G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
+  {
+    bool own = live_tiles <= (long long)G->n_wg;  // every entry has a workgroup to itself
+    if (const char *env = getenv("PCCL_HIP_OWN_ENTRIES")) own = own && env[0] != '0';
+    ((int *)(img + off_qcount))[kQueues] = own ? 1 : 0;
+  }
 
   e = fixed ? hipMemcpyAsync(dev, img, arena_bytes, hipMemcpyHostToDevice, fixed->stream)
             : hipMemcpy(dev, img, arena_bytes, hipMemcpyHostToDevice);
@@ -1228,7 +1253,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // finish first.  Only a failed upload can leave the graph unusable.
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
   const std::vector<unsigned char> edges_after = classify_dependencies(next, G->parts, G->topo, &G->part_eligible);
-  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch) != G->chain_words) {
+  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch, G->forward_capable) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
     fresh.descs.swap(next);
@@ -1238,6 +1263,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.spin_limit = G->spin_limit;
     fresh.fixed_parts = G->parts;
     fresh.fixed_n_wg = G->n_wg;
+    fresh.fixed_kernel = G->kernel;
+    fresh.forward_capable = G->forward_capable;
     char *old_dev = G->dev;
     // The run number goes on from where the DEVICE stands, not from the count of graph_run
     // calls: every replay of a recorded launch has moved the device's word on as well, and a

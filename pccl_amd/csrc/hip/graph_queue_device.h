@@ -50,7 +50,8 @@ struct GraphControl {
   const struct ForwardStep *chain_table;  // one row per op of every forward chain, chain after chain
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
-  const int *queue_count;                 // entries on each queue: in memory, not here, because which ops queue entries
+  const int *queue_count;                 // entries on each queue, then the mode word (1: no more entries than workgroups,
+                                          // each workgroup takes the entry of its own number): in memory, not here, because which ops queue entries
                                           // (chains do not) can change with the operands' addresses, and what is in
                                           // this block is frozen into any launch that a stream capture has recorded
   unsigned int spin_limit;
@@ -75,6 +76,10 @@ constexpr int kChainForward = 2;  // head: 1 if the whole chain runs in one pass
                                   // previous op's output 0
 constexpr int kChainRow = 3;      // head of a forward chain: its first row in GraphControl::chain_table
 constexpr int kMaxForwardSteps = 16;
+// A queue entry: op uid | part << 32 | (op heads a chain) << 51.  The flag saves every other entry the
+// load of its op's chain words.
+constexpr int kMaxParts = 1 << 19;
+constexpr unsigned long long kEntryChainHead = 1ull << 51;
 
 // indices into GraphControl::hot
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
@@ -487,8 +492,11 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   if (!drawn) draw_ticket();
 }
 
-template <int DT, class Op>
-__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3))) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
+// The kernel's body.  FORWARD: with the code that runs a chain in one pass (run_chain_forward).  That
+// code needs 80 registers more than the rest, and compiled into the one kernel it cost graphs
+// without such chains 3 % (14 ops of 32 MiB: 197 -> 203 us), so it is an instance of its own.
+template <int DT, class Op, bool FORWARD>
+__device__ __forceinline__ void drain_body(const GraphControl &g) {
   __shared__ unsigned long long s_entry;
   __shared__ i32x4 s_chain;  // the claimed op's kChainWords words
   __shared__ int s_go;
@@ -498,6 +506,20 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
   unsigned int *abort_flag = &hot[kHotAbort].value;
   const unsigned int spin_limit = g.spin_limit;
   const int home = blockIdx.x % kQueues;
+  // With no more entries than workgroups every workgroup has an entry to itself: workgroup b takes
+  // entry b of the global order (entry b / kQueues of its home queue) and leaves when that is done.
+  // No ticket is drawn, and no workgroup goes round the eight queues at the end to find each of them
+  // empty (eight returning atomics, one after the other: 14.9 -> 11 us for a graph of one 64 KiB op).
+  // Dependencies point backwards in the global order and workgroups are started in order, so the
+  // lowest-numbered workgroup still running never waits for one that has not started.
+  // The mode word sits behind the queue lengths in memory, not in the kernel arguments: a rebind can
+  // change the number of entries (see GraphControl::queue_count).  Thread 0 reads it before its first
+  // claim, together with the entry that would be its own (a load from inside the queue's room even
+  // where it is not used), and keeps it as a bit of `exhausted`.
+  constexpr unsigned int kOwnEntry = 1u << 31, kAllQueues = (1u << kQueues) - 1u;
+  // Thread 0 keeps the queue lengths in LDS: it needs one at every claim, and a scalar load that has
+  // dropped out of the cache costs a trip to the L2 behind the data traffic (0.6 us per part measured).
+  __shared__ int s_queue_count[kQueues + 1];
 
   // Loop shape matters: thread 0's bookkeeping for the part just finished and its
   // claim of the next entry sit in ONE conditional block per iteration, and the
@@ -528,13 +550,35 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
       // two round trips overlap instead of following each other (see finish_part).
       int first_q = -1, first_t = 0;
       unsigned int aborted = 0;
+      unsigned long long own_e = 0;
       auto draw_ticket = [&] {
-        // (the workgroup's very first ticket does not wait for the queue lengths to arrive from memory:
-        // there are no more workgroups than entries at creation, so its home queue has one for it)
-        if (!h) first_q = home;
+        if (!h) {
+          // The workgroup's first claim.  A ticket of its home queue is requested before the mode word
+          // and the queue lengths are there (there are no more workgroups than entries at creation, so
+          // the home queue has an entry for it); with an entry of its own the ticket goes unused, and
+          // the queue heads it moved are set back with all the others when the run ends.
+          const int ticket = __hip_atomic_fetch_add(g.queue_head[home], 1, __ATOMIC_RELAXED, AGENT);
+          const int mode = g.queue_count[kQueues];
+          own_e = g.queue_entries[home][blockIdx.x / kQueues];
+#pragma unroll
+          for (int q = 0; q < kQueues; ++q) s_queue_count[q] = g.queue_count[q];
+          first_q = home;
+          if (mode) {
+            exhausted = kOwnEntry;
+            first_t = (int)(blockIdx.x / kQueues);
+          } else {
+            first_t = ticket;
+            aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
+          }
+          return;
+        }
+        if (exhausted & kOwnEntry) {
+          exhausted |= kAllQueues;
+          return;
+        }
         for (int i = 0; i < kQueues && first_q < 0; ++i) {
           const int q = (home + i) % kQueues;
-          if (!(exhausted & (1u << q)) && g.queue_count[q] > 0) first_q = q;
+          if (!(exhausted & (1u << q)) && s_queue_count[q] > 0) first_q = q;
         }
         if (first_q >= 0) first_t = __hip_atomic_fetch_add(g.queue_head[first_q], 1, __ATOMIC_RELAXED, AGENT);
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
@@ -557,11 +601,12 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
         for (int i = 0; i < kQueues && !go; ++i) {
           const int q = (home + i) % kQueues;
           if (exhausted & (1u << q)) continue;
-          const int n = g.queue_count[q];
+          const int n = s_queue_count[q];
           int t = n;
           if (q == first_q) {  // the ticket requested above
             t = first_t;
             first_q = -1;
+            if (exhausted & kOwnEntry) exhausted |= kAllQueues;  // (it is the only entry this workgroup takes)
           } else if (n > 0) {
             t = __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT);
           }
@@ -571,12 +616,12 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
             // which do not queue behind the vector memory traffic of the parts in flight on
             // this compute unit.  What they read is constant during a run.
             const int qs = __builtin_amdgcn_readfirstlane(q), ts = __builtin_amdgcn_readfirstlane(t);
-            e = g.queue_entries[qs][ts];
+            e = (exhausted & kOwnEntry) ? own_e : g.queue_entries[qs][ts];
             entry_index = (size_t)ts * kQueues + qs;
             go = 1;
             if (g.trace) {
               cur_trace = g.trace + entry_index * kTraceWords;
-              cur_trace[kTraceWhat] = e | ((unsigned long long)blockIdx.x << 52);
+              cur_trace[kTraceWhat] = (e & ~kEntryChainHead) | ((unsigned long long)blockIdx.x << 52);
               cur_trace[kTraceClaimed] = wall_clock64();
             }
             if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
@@ -595,11 +640,12 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
         // that word's only reader and clears it for the next run.
         const unsigned int w12 = *word12(hc);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
-        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + ((size_t)(g.entry_base[uid] + (int)(e >> 32)) << g.part_shift) : nullptr;
+        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + ((size_t)(g.entry_base[uid] + (int)((e & ~kEntryChainHead) >> 32)) << g.part_shift) : nullptr;
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;
-        chain_words = *(const i32x4 *)(g.chain + kChainWords * uid);
+        if (e & kEntryChainHead) chain_words = *(const i32x4 *)(g.chain + kChainWords * uid);
+        else chain_words = i32x4{-1, 1, 0, 0};
         const unsigned int n_pred = (w12 & 0xffu) - part_preds;  // whole-op dependencies
         if (n_pred != 0 && arrived != n_pred &&
             !bounded_wait(abort_flag, spin_limit, [&] {
@@ -646,7 +692,7 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
     __syncthreads();
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
     const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
-    const int part = __builtin_amdgcn_readfirstlane((int)(s_entry >> 32));
+    const int part = __builtin_amdgcn_readfirstlane((int)((s_entry & ~kEntryChainHead) >> 32));
     cur_uid = uid;
     cur_part = part;
     h = &g.headers[uid];
@@ -662,24 +708,25 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
     if (n > per) n = per;
     if (n > 0) {
       bool forwarded = false;
-      if constexpr (DT != kAnyDtype) {
-        // (the instance that picks the fold per op keeps to the plain chain walk below)
+      if constexpr (FORWARD && DT != kAnyDtype) {
         if (chain_next >= 0 && __builtin_amdgcn_readfirstlane(s_chain[kChainForward])) {
           run_chain_forward<Dtype<DT>, Op>(g, pl, cur_chain_ops, __builtin_amdgcn_readfirstlane(s_chain[kChainRow]), lo, n);
           forwarded = true;
         }
       }
       if (!forwarded) {
-        if constexpr (DT == kAnyDtype) run_part_any(pl, lo, n);
-        else run_part<DT, Op>(pl, lo, n);
-        // The ops chained behind this one, same part: every wavefront has waited for its own stores
-        // (run_part ends that way), the barrier makes that true of the whole workgroup, and the next
-        // op's loads read past the L2 like every load here.  The chain index is uniform.
-        for (int next = chain_next; next >= 0; next = g.chain[kChainWords * next + kChainNext]) {
+        // The op, then the ops chained behind it, same part: every wavefront has waited for its own
+        // stores (run_part ends that way), the barrier makes that true of the whole workgroup, and the
+        // next op's loads read past the L2 like every load here.  The chain index is uniform.
+        // (One call site for both: a second inlined copy of run_part cost the kernel its registers.)
+        const pccl_op_payload *step = pl;
+        for (int next = chain_next;;) {
+          if constexpr (DT == kAnyDtype) run_part_any(step, lo, n);
+          else run_part<DT, Op>(step, lo, n);
+          if (next < 0) break;
           __syncthreads();
-          const pccl_op_payload *npl = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
-          if constexpr (DT == kAnyDtype) run_part_any(npl, lo, n);
-          else run_part<DT, Op>(npl, lo, n);
+          step = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
+          next = g.chain[kChainWords * next + kChainNext];
         }
       }
     }
@@ -714,11 +761,25 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
   }
 }
 
+template <int DT, class Op>
+__global__ void __launch_bounds__(kBlock) drain_graph_kernel(const GraphControl g) {  // by value: every field arrives through the kernarg segment
+  drain_body<DT, Op, false>(g);
+}
+
+// (three wavefronts per SIMD like the plain instance: the allocator's own choice was two)
+template <int DT, class Op>
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3))) drain_graph_forward_kernel(const GraphControl g) {
+  drain_body<DT, Op, true>(g);
+}
+
 typedef void (*DrainKernel)(const GraphControl);
 
 // The instances of one dtype; defined in graph_queue_inst_<dtype>.hip.
 template <int DT>
 DrainKernel drain_for_compute(int compute);
+// ... and those with the one-pass chain code; defined in graph_queue_fwd_<dtype>.hip.
+template <int DT>
+DrainKernel drain_forward_for_compute(int compute);
 
 // The instance for graphs whose REDUCE ops do not share one (dtype, compute) pair;
 // defined in graph_queue_inst_any.hip.
@@ -732,6 +793,17 @@ DrainKernel drain_for_any();
       case PCCL_PROD: return drain_graph_kernel<DT, OpProd>;     \
       case PCCL_MIN: return drain_graph_kernel<DT, OpMin>;       \
       default: return drain_graph_kernel<DT, OpMax>;             \
+    }                                                            \
+  }
+
+#define PCCL_DEFINE_DRAIN_FORWARD_FOR_COMPUTE(DT)                        \
+  template <>                                                    \
+  DrainKernel drain_forward_for_compute<DT>(int compute) {               \
+    switch (compute) {                                           \
+      case PCCL_SUM: return drain_graph_forward_kernel<DT, OpSum>;       \
+      case PCCL_PROD: return drain_graph_forward_kernel<DT, OpProd>;     \
+      case PCCL_MIN: return drain_graph_forward_kernel<DT, OpMin>;       \
+      default: return drain_graph_forward_kernel<DT, OpMax>;             \
     }                                                            \
   }
 

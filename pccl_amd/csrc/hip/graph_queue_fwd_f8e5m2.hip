@@ -1,0 +1,7 @@
+// graph_queue_fwd_f8e5m2.hip -- the f8e5m2 instances of the drain kernel that carry the one-pass chain
+// code (one per compute op).
+#include "graph_queue_device.h"
+
+namespace pccl_queue {
+PCCL_DEFINE_DRAIN_FORWARD_FOR_COMPUTE(PCCL_F8E5M2)
+}  // namespace pccl_queue
