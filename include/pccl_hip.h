@@ -196,7 +196,15 @@ typedef struct pccl_op_desc {
  * the built-in part sizes.  For such a graph graph_status reports all ops complete once the stream has
  * drained, graph_info a null layout, graph_trace PCCL_ERR_UNSUPPORTED; a launch recorded by stream
  * capture keeps the addresses it was recorded with, whatever graph_rebind does later.
- * PCCL_HIP_PLAN_LAUNCHES=0 sends everything to the queue. */
+ * PCCL_HIP_PLAN_LAUNCHES=0 sends everything to the queue.
+ * Chains: an op that depends on one op alone, which nothing else depends on and which is cut like
+ * it, queues no entries of its own; the workgroup that has run part p of its predecessor goes on
+ * with its part p (and keeps the value in registers where the op takes the predecessor's output 0
+ * as one of at most two inputs).  A level of the graph whose entries start such chains is cut by
+ * the built-in choice into the smallest parts (from 8 KiB) with which its entries fit the resident
+ * workgroups once.  Results, graph_status and graph_rebind are as without chains;
+ * graph_info's n_tiles and the timeline count the entries that are queued.  PCCL_HIP_CHAINS=0
+ * switches chains off. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
@@ -248,7 +256,9 @@ int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capa
  * execution it allows. */
 int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int *parts, unsigned char *kinds);
 
-/* Device address of the GraphBufferLayout and launch facts, for inspection. */
+/* Device address of the GraphBufferLayout and launch facts, for inspection: n_tiles = queue entries
+ * (parts of the ops that queue entries; ops that run behind another op in a chain queue none), or the
+ * number of launches for a graph that runs as plain launches; n_workgroups = width of the launch. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 
 /* signal_base the NEXT pccl_hip_graph_run of this graph will use: a party outside the

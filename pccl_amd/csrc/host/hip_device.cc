@@ -63,6 +63,8 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PLAN_LAUNCHES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_PART_DEPS");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_ORDER_BLOCK");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAINS");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_OWN_ENTRIES");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;

@@ -678,13 +678,17 @@ def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, 
     g.destroy()
 
 
-def test_graph_beside_a_kernel_that_occupies_the_gpu(hip, oracle):
+@pytest.mark.parametrize("chains,size", [("0", 30_001), ("1", 30_001), ("0", 3_000_001)])
+def test_graph_beside_a_kernel_that_occupies_the_gpu(hip, oracle, monkeypatch, chains, size):
     """The drain's workgroups wait for each other inside one launch, so it needs its queues' workgroups
     resident.  With another stream's long elementwise kernels holding compute units at the same time the
-    run must still complete every op (no bounded wait may give up), bit-exact."""
+    run must still complete every op (no bounded wait may give up), bit-exact: with every op queueing
+    its own entries (112 ops that wait for each other through the queue; one workgroup per entry at
+    the small size, tickets at the large one) and with the ring's steps chained."""
     import torch
     from pccl_amd import lang
-    world, size = 8, 30_001
+    monkeypatch.setenv("PCCL_HIP_CHAINS", chains)
+    world = 8
     ir, per_rank = lang.ring_allreduce(world, size, dtype="bf16")
     low = ir.lower()
     host_in = [H.gen("bf16", per_rank, 611, r) for r in range(world)]
