@@ -256,6 +256,16 @@ int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capa
  * execution it allows. */
 int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int *parts, unsigned char *kinds);
 
+/* Which ops the executor would run behind each other in one workgroup (chains, see graph_create), as
+ * a host-only rule like the one above: given the ops, their part counts and the element size of the
+ * graph's kernel instance (forward_elem_bytes; 0 = no chain may run in one pass), writes four ints per
+ * op: the op that runs behind it (-1: none); for an op that starts a chain the number of ops in it
+ * (else 1); for an op that starts a chain 1 if the chain runs in one pass with the value kept in
+ * registers, for another op of such a chain the index of the input that is its predecessor's
+ * output 0; and, for an op that starts a one-pass chain, the first of the chain's rows in the
+ * executor's operand table.  Touches no device. */
+int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, int forward_elem_bytes, int *words);
+
 /* Device address of the GraphBufferLayout and launch facts, for inspection: n_tiles = queue entries
  * (parts of the ops that queue entries; ops that run behind another op in a chain queue none), or the
  * number of launches for a graph that runs as plain launches; n_workgroups = width of the launch. */

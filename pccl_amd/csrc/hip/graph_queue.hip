@@ -92,6 +92,7 @@ struct Graph {
   int fixed_n_wg = 0;           // build_graph: launch this many workgroups instead of choosing
   DrainKernel fixed_kernel = nullptr;  // build_graph: ... and this kernel instance
   bool forward_capable = false; // the instance has the code that runs a chain in one pass
+  int kernel_elem_bytes = 0;    // element size of the instance's dtype
   int device = 0;
   unsigned int runs = 0;        // launches so far; run r uses signal values (r << 16) + value
   DrainKernel kernel = nullptr;
@@ -353,11 +354,14 @@ bool plan_launches(const std::vector<pccl_op_desc> &ops, std::vector<pccl_op_des
 // Returns kChainWords ints per op.
 std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
                              const std::vector<unsigned char> &part_edge, const std::vector<int> &n_succ,
-                             const std::vector<unsigned char> &order_touch, bool allow_forward) {
+                             const std::vector<unsigned char> &order_touch, int forward_elem_bytes) {
   const int n_ops = (int)ops.size();
   std::vector<int> words((size_t)kChainWords * (size_t)std::max(n_ops, 1), 0);
   std::vector<int> next(n_ops, -1), prev(n_ops, -1);
-  bool on = true, forward_on = allow_forward;
+  // forward_elem_bytes: element size of the kernel instance's dtype if it has the one-pass code, else 0.
+  // A chain of copies may have another element size than the graph's REDUCE ops (a copy moves bytes
+  // of its own dtype): such a chain goes through memory, where every op is run by its own rule.
+  bool on = true, forward_on = forward_elem_bytes > 0;
   if (const char *env = getenv("PCCL_HIP_CHAINS")) on = env[0] != '0', forward_on = forward_on && (env[0] != '1' || env[1] != 'm');  // "1m": through memory only
   auto is_data = [&](int i) { return ops[i].primitive != PCCL_NOTIFY && ops[i].primitive != PCCL_GET_NOTIFIED; };
   auto bytes_of = [&](int i) { return (uintptr_t)ops[i].count * (uintptr_t)elem_bytes(ops[i].dtype); };
@@ -384,7 +388,8 @@ std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::ve
     for (int u = h; u >= 0; u = next[u]) steps.push_back(u);
     words[(size_t)kChainWords * h + kChainLength] = (int)steps.size();
     // can the values be handed on in registers?
-    bool forward = forward_on && (int)steps.size() <= kMaxForwardSteps && ops[h].n_in <= 2;
+    bool forward = forward_on && (int)steps.size() <= kMaxForwardSteps && ops[h].n_in <= 2 &&
+                   elem_bytes(ops[h].dtype) == forward_elem_bytes;
     for (int t : steps) forward = forward && ops[t].n_out <= 2;
     const uintptr_t len = bytes_of(h);
     std::vector<int> fed(steps.size(), 0);
@@ -531,15 +536,24 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   }
   for (int i = 0; i < n_ops; ++i)
     if (n_succ[i] > 255) return fail(PCCL_ERR_GRAPH, "op %d: %d successors exceed num_next_ops_ (unsigned char)", i, n_succ[i]);
-  // copy-only graphs: element size of the ops decides nothing but alignment assumptions
-  if (g_dtype < 0) { g_dtype = PCCL_BF16; g_compute = PCCL_SUM; }
+  // copy-only graphs: the kernel instance of the first op's dtype (a chain of copies of that element
+  // size can then run in one pass; nothing else depends on the choice)
+  if (g_dtype < 0) {
+    g_dtype = PCCL_BF16;
+    g_compute = PCCL_SUM;
+    for (int i = 0; i < n_ops; ++i)
+      if (ops[i].primitive != PCCL_NOTIFY && ops[i].primitive != PCCL_GET_NOTIFIED) {
+        g_dtype = ops[i].dtype;
+        break;
+      }
+  }
   // launch width: as many workgroups as the chip holds of this kernel instance
   // (two instances per dtype and fold: with and without the code that runs a chain in one pass.  Which
   // of them runs is settled once the chains are known, below; the launch width must hold for both.  A
   // rebuild in place keeps the instance: launches that a stream capture has recorded carry it.)
   const DrainKernel plain_kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute, false);
   const DrainKernel forward_kernel = mixed ? nullptr : drain_for(g_dtype, g_compute, true);
-  const bool allow_forward = G->fixed_kernel ? G->forward_capable : !mixed;
+  const int forward_elem_bytes = (G->fixed_kernel ? G->forward_capable : !mixed) ? elem_bytes(g_dtype) : 0;
   int occ = 8;
   for (DrainKernel k : {plain_kernel, forward_kernel}) {
     if (!k) continue;
@@ -723,7 +737,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->n_succ = n_succ;
   G->order_touch.assign(n_ops, 0);
   for (int i = 0; i < n_ops; ++i) G->order_touch[i] = order_pred[i] != 0 || !order_succ[i].empty();
-  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, allow_forward);
+  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, forward_elem_bytes);
   std::vector<int> chain_prev(n_ops, -1), chain_tail(n_ops, 0);
   auto link_chains = [&] {
     std::fill(chain_prev.begin(), chain_prev.end(), -1);
@@ -792,7 +806,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       G->parts = parts;
       G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
       G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
-      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, allow_forward);
+      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, forward_elem_bytes);
       link_chains();
     }
   }
@@ -861,6 +875,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->total_tiles = (int)live_tiles;  // entries that are queued; the arena has room for an entry per part of every op
   G->all_tiles = (int)tiles;
   G->payload_off = off_payload;
+  G->kernel_elem_bytes = elem_bytes(g_dtype);
   if (G->fixed_kernel) {
     G->kernel = G->fixed_kernel;
   } else {
@@ -1253,7 +1268,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // finish first.  Only a failed upload can leave the graph unusable.
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
   const std::vector<unsigned char> edges_after = classify_dependencies(next, G->parts, G->topo, &G->part_eligible);
-  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch, G->forward_capable) != G->chain_words) {
+  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
     fresh.descs.swap(next);
@@ -1354,6 +1369,27 @@ int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int
   const std::vector<unsigned char> flags = classify_dependencies(descs, part_counts, topo);
   if (n_deps && !kinds) return fail(PCCL_ERR_INVALID_ARG, "classify_dependencies: kinds is null");
   if (n_deps) memcpy(kinds, flags.data(), n_deps);
+  return PCCL_OK;
+}
+
+int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, int forward_elem_bytes, int *words) {
+  pccl_host::clear_error();
+  if (n_ops < 0 || (n_ops > 0 && (!ops || !parts || !words))) return fail(PCCL_ERR_INVALID_ARG, "plan_chains: bad arguments");
+  std::vector<unsigned char> kinds;
+  {
+    size_t n_deps = 0;
+    for (int i = 0; i < n_ops; ++i) n_deps += (size_t)std::max(ops[i].n_deps, 0);
+    kinds.assign(std::max<size_t>(n_deps, 1), 0);
+  }
+  const int rc = pccl_hip_classify_dependencies(ops, n_ops, parts, kinds.data());  // checks the ops as well
+  if (rc != PCCL_OK) return rc;
+  std::vector<pccl_op_desc> descs(ops, ops + n_ops);
+  std::vector<int> part_counts(parts, parts + n_ops), n_succ(n_ops, 0);
+  for (int i = 0; i < n_ops; ++i)
+    for (int d = 0; d < ops[i].n_deps; ++d) ++n_succ[ops[i].deps[d]];
+  const std::vector<unsigned char> untouched(n_ops, 0);
+  const std::vector<int> plan = plan_chains(descs, part_counts, kinds, n_succ, untouched, forward_elem_bytes);
+  if (n_ops) memcpy(words, plan.data(), sizeof(int) * (size_t)kChainWords * (size_t)n_ops);
   return PCCL_OK;
 }
 

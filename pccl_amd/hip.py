@@ -86,6 +86,7 @@ def lib():
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.pccl_hip_classify_dependencies.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), vp]
+        L.pccl_hip_plan_chains.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ci, ctypes.POINTER(ci)]
         L.pccl_hip_graph_dependency_kinds.argtypes = [vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_trace.argtypes = [vp, ci]
         L.pccl_hip_graph_read_trace.argtypes = [vp, vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
@@ -247,6 +248,16 @@ def classify_dependencies(ops, parts):
     pa = (ctypes.c_int * max(len(ops), 1))(*parts)
     _check(lib().pccl_hip_classify_dependencies(arr, len(ops), pa, kinds))
     return list(kinds)[:n_deps]
+
+
+def plan_chains(ops, parts, forward_elem_bytes):
+    """The executor's chain plan for these ops (host only): per op a tuple (next op or -1, ops in the
+    chain it starts or 1, one-pass flag / index of the handed-on input, first row of its operand table)."""
+    arr, keep = _op_descs(ops)
+    pa = (ctypes.c_int * max(len(ops), 1))(*parts)
+    words = (ctypes.c_int * max(4 * len(ops), 1))()
+    _check(lib().pccl_hip_plan_chains(arr, len(ops), pa, forward_elem_bytes, words))
+    return [tuple(words[4 * i:4 * i + 4]) for i in range(len(ops))]
 
 
 STATIC_ARENA_BYTES = 8 << 20

@@ -1,0 +1,133 @@
+"""The executor's chain plan (pccl_hip_plan_chains, host only): which ops run behind each other in one
+workgroup, and which chains may run in one pass with the value kept in registers.  No GPU needed:
+operands are plain numbers that stand for device addresses."""
+import pytest
+
+from pccl_amd import hip
+
+ES = 4  # f32
+
+
+def op(ins, outs, deps, count=1000, dtype="f32", compute="sum"):
+    return dict(dtype=dtype, compute=compute, ins=[a for a in ins], outs=[a for a in outs], count=count, deps=list(deps))
+
+
+def buf(k, n=1000):
+    """Address of buffer k: buffers are far enough apart not to overlap."""
+    return 0x100000 + k * (n * 16 + 4096)
+
+
+def test_single_predecessor_and_successor_make_a_chain():
+    a, b, c, t, u, v = (buf(k) for k in range(6))
+    ops = [op([a, b], [t], []), op([t, c], [u], [0]), op([u], [v], [1])]
+    plan = hip.plan_chains(ops, [1, 1, 1], ES)
+    assert [p[0] for p in plan] == [1, 2, -1]           # 0 -> 1 -> 2
+    assert plan[0][1] == 3 and plan[1][1] == 1 and plan[2][1] == 1
+    assert plan[0][2] == 1 and plan[0][3] == 0          # one pass, rows from 0
+    assert plan[1][2] == 0                              # the handed-on value is input 0 of op 1
+    # ... input 1 when the operands are the other way round
+    ops[1] = op([c, t], [u], [0])
+    assert hip.plan_chains(ops, [1, 1, 1], ES)[1][2] == 1
+
+
+def test_no_chain_across_a_fan_out_or_a_fan_in():
+    a, b, c, t, u, v, w = (buf(k) for k in range(7))
+    fan_out = [op([a, b], [t], []), op([t, c], [u], [0]), op([t], [v], [0])]
+    assert [p[0] for p in hip.plan_chains(fan_out, [1, 1, 1], ES)] == [-1, -1, -1]
+    fan_in = [op([a, b], [t], []), op([a, c], [u], []), op([t, u], [v], [0, 1]), op([v], [w], [2])]
+    plan = hip.plan_chains(fan_in, [1, 1, 1, 1], ES)
+    assert [p[0] for p in plan] == [-1, -1, 3, -1]      # only 2 -> 3
+    assert plan[2][1] == 2 and plan[2][2] == 1
+
+
+def test_ops_cut_differently_or_of_other_length_do_not_chain():
+    a, b, c, t, u = (buf(k, 100000) for k in range(5))
+    ops = [op([a, b], [t], [], count=100000), op([t, c], [u], [0], count=100000)]
+    assert hip.plan_chains(ops, [4, 4], ES)[0][0] == 1
+    assert hip.plan_chains(ops, [4, 5], ES)[0][0] == -1
+    ops[1] = op([t, c], [u], [0], count=99999)
+    assert hip.plan_chains(ops, [4, 4], ES)[0][0] == -1
+
+
+def test_many_part_ops_chain_only_where_part_p_needs_part_p():
+    n = 100000
+    a, b, c, t, u = (buf(k, n) for k in range(5))
+    lined_up = [op([a, b], [t], [], count=n), op([t, c], [u], [0], count=n)]
+    assert hip.classify_dependencies(lined_up, [8, 8]) == [1]
+    assert hip.plan_chains(lined_up, [8, 8], ES)[0][0] == 1
+    shifted = [op([a, b], [t], [], count=n), op([t + 64 * ES, c], [u], [0], count=n)]   # reads t 64 elements further on
+    assert hip.classify_dependencies(shifted, [8, 8]) == [0]
+    assert hip.plan_chains(shifted, [8, 8], ES)[0][0] == -1
+    # with one part each the whole op is done before the next starts: a chain again, but through memory
+    plan = hip.plan_chains(shifted, [1, 1], ES)
+    assert plan[0][0] == 1 and plan[0][2] == 0
+
+
+def test_one_pass_needs_the_predecessors_output_as_an_input_and_no_other_look_at_the_chain():
+    a, b, c, t, u, v = (buf(k) for k in range(6))
+    # op 2 reads t again, which the chain wrote: through memory
+    ops = [op([a, b], [t], []), op([t, c], [u], [0]), op([u, t], [v], [1])]
+    plan = hip.plan_chains(ops, [1, 1, 1], ES)
+    assert [p[0] for p in plan] == [1, 2, -1] and plan[0][2] == 0
+    # op 1 does not read op 0's output at all (ordered behind it for another reason): through memory
+    ops = [op([a, b], [t], []), op([c, a], [u], [0])]
+    plan = hip.plan_chains(ops, [1, 1], ES)
+    assert plan[0][0] == 1 and plan[0][2] == 0
+    # the handed-on value must be OUTPUT 0 of the predecessor
+    ops = [op([a, b], [t, v], []), op([v, c], [u], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 0
+    ops = [op([a, b], [v, t], []), op([v, c], [u], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 1
+    # in place on the first op's own input is fine (read before written, pack by pack) ...
+    ops = [op([a, b], [a], []), op([a, c], [u], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 1
+    # ... a later op writing over the first op's input is not
+    ops = [op([a, b], [t], []), op([t, c], [a], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 0
+
+
+def test_one_pass_limits():
+    bufs = [buf(k) for k in range(64)]
+    chain = lambda n: [op([bufs[k], bufs[40]], [bufs[k + 1]], [k - 1] if k else []) for k in range(n)]
+    assert hip.plan_chains(chain(16), [1] * 16, ES)[0][1:3] == (16, 1)
+    assert hip.plan_chains(chain(17), [1] * 17, ES)[0][1:3] == (17, 0)   # more ops than one pass holds
+    # first op with more than two inputs
+    ops = [op(bufs[:3], [bufs[10]], []), op([bufs[10], bufs[4]], [bufs[11]], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][1:3] == (2, 0)
+    # more than two outputs somewhere
+    ops = [op(bufs[:2], [bufs[10]], []), op([bufs[10]], bufs[11:14], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[0][1:3] == (2, 0)
+    # no one-pass code in the kernel instance (forward_elem_bytes 0), or of another element size
+    assert hip.plan_chains(chain(3), [1] * 3, 0)[0][1:3] == (3, 0)
+    assert hip.plan_chains(chain(3), [1] * 3, 2)[0][1:3] == (3, 0)
+
+
+def test_rows_of_the_operand_table_follow_the_chains_in_op_order():
+    bufs = [buf(k) for k in range(40)]
+    # chain A: ops 0 -> 3 -> 5; chain B: ops 1 -> 2; single op 4
+    ops = [op([bufs[0], bufs[1]], [bufs[10]], []),
+           op([bufs[2], bufs[3]], [bufs[11]], []),
+           op([bufs[11], bufs[4]], [bufs[12]], [1]),
+           op([bufs[10], bufs[5]], [bufs[13]], [0]),
+           op([bufs[6]], [bufs[14]], []),
+           op([bufs[13]], [bufs[15]], [3])]
+    plan = hip.plan_chains(ops, [1] * 6, ES)
+    assert [p[0] for p in plan] == [3, 2, -1, 5, -1, -1]
+    assert plan[0][1:] == (3, 1, 0) and plan[1][1:] == (2, 1, 3)
+    assert plan[4][1] == 1
+
+
+def test_signal_ops_do_not_chain():
+    a, b, t, u = (buf(k) for k in range(4))
+    sig = 0x900000
+    ops = [op([a, b], [t], []), dict(primitive=2, signal=sig, value=1, deps=[0]),
+           dict(primitive=3, signal=sig + 4, value=1, deps=[]), op([t], [u], [2])]
+    assert [p[0] for p in hip.plan_chains(ops, [1, 1, 1, 1], ES)] == [-1, -1, -1, -1]
+
+
+def test_bad_arguments_are_refused():
+    a, b, t = (buf(k) for k in range(3))
+    with pytest.raises(hip.PcclError):
+        hip.plan_chains([op([a, b], [t], [5])], [1], ES)      # dependency on an op that does not exist
+    with pytest.raises(hip.PcclError):
+        hip.plan_chains([op([a, b], [t], [])], [0], ES)       # no parts

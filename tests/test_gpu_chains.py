@@ -217,3 +217,43 @@ def test_rebind_moves_the_chains_operands(hip, oracle):
         keep = at  # (alive until the next rebind has gone through)
         at = moved
     g.destroy()
+
+
+def test_chains_of_copies_with_an_element_size_of_their_own(hip, oracle):
+    """A copy moves bytes of its own dtype, whatever the graph's REDUCE ops are: chains of copies in a
+    graph without any REDUCE op (the kernel instance then follows the first op's dtype), and chains of
+    f64 / f32 / 1-byte copies beside bf16 reductions."""
+    import torch
+    count = 70003
+    for reduce_dtype, copy_dtypes in ((None, ["f64", "f32", "f8e4m3"]), (None, ["bf16", "f64"]), ("bf16", ["f64", "f32", "f8e5m2", "bf16"])):
+        ops_dev, ops_host, checks, sources = [], [], [], []
+        if reduce_dtype:
+            a, b = H.gen(reduce_dtype, count, 960, 0), H.gen(reduce_dtype, count, 960, 1)
+            da, db = H.DevBuf(torch, reduce_dtype, count, 0, src=a), H.DevBuf(torch, reduce_dtype, count, 0, src=b)
+            dt = H.DevBuf(torch, reduce_dtype, count, 0)
+            ht = np.zeros(count, dtype=H.STORAGE[reduce_dtype])
+            ops_dev.append(dict(dtype=reduce_dtype, compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]))
+            ops_host.append(dict(dtype=reduce_dtype, compute="sum", ins=[a, b], outs=[ht], count=count))
+            checks.append((dt, ht, "sum"))
+        for k, dtype in enumerate(copy_dtypes):
+            src = H.gen(dtype, count, 961, k)
+            dev = [H.DevBuf(torch, dtype, count, H.ELEM_BYTES[dtype] * (j % 3), src=src if j == 0 else None) for j in range(5)]
+            sources.append(dev[0])  # (stays allocated while the graph reads it)
+            host = [src] + [np.zeros(count, dtype=H.STORAGE[dtype]) for _ in range(4)]
+            for j in range(4):  # x0 -> x1 -> x2 -> x3 -> x4
+                deps = [len(ops_dev) - 1] if j else []
+                ops_dev.append(dict(dtype=dtype, compute="sum", ins=[dev[j].ptr], outs=[dev[j + 1].ptr], count=count, deps=deps))
+                ops_host.append(dict(dtype=dtype, compute="sum", ins=[host[j]], outs=[host[j + 1]], count=count))
+                checks.append((dev[j + 1], host[j + 1], "%s copy %d" % (dtype, j)))
+        oracle.run_ops(ops_host)
+        for tile in (1 << 20, 16 << 10):
+            g = hip.Graph(ops_dev, tile_bytes=tile)
+            if tile == 1 << 20:  # one part per op: an entry per chain of copies, one for the reduction
+                assert g.info()["n_tiles"] == len(copy_dtypes) + (1 if reduce_dtype else 0)
+            for dev_buf, _, _ in checks:
+                dev_buf.view().fill_(0xFF)
+            _run(torch, hip, g, len(ops_dev))
+            for dev_buf, want, what in checks:
+                H.assert_bits_equal(dev_buf.download(), want, "%s (reduce dtype %s, parts of %d)" % (what, reduce_dtype, tile))
+                assert dev_buf.guards_intact(), what
+            g.destroy()
