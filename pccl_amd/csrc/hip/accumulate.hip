@@ -24,6 +24,7 @@ struct AccLaunch {
   long head;     // elements before the first 16-byte pack of output 0
   long n_packs;  // 16-byte packs in the body
   long count;
+  int rotate;    // workgroup -> chunk rotation (rotated_chunk, reduce_copy_kernel.h)
 };
 
 // One pack per lane with a compile-time number of destinations: 1 + NOUT loads in flight per
@@ -96,10 +97,11 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(const AccLaunch p) {
   D::wave_init();
   typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
-  const long pack = (long)blockIdx.x * kBlock + threadIdx.x;
+  const unsigned chunk = p.rotate ? rotated_chunk(blockIdx.x, gridDim.x) : blockIdx.x;
+  const long pack = (long)chunk * kBlock + threadIdx.x;
   if (pack < p.n_packs) {
     // (wave-uniform base, lane offset) addressing: the workgroup's 4 KiB of every stream
-    const size_t wg = (size_t)p.head * D::kElemBytes + (size_t)blockIdx.x * (kBlock * 16);
+    const size_t wg = (size_t)p.head * D::kElemBytes + (size_t)chunk * (kBlock * 16);
     const unsigned int off = threadIdx.x * 16u;
     switch (p.n_out) {
       case 1: accumulate_pack<D, Op, ALIGNED, kLd, kSt, 1>(p, wg, off); break;
@@ -210,6 +212,8 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
     const int wgs = std::max(2, std::min(8, (20 + streams / 2) / streams));
     if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
   }
+  // the chunk order of large launches, as for reduce_copy (one workgroup per chunk here always)
+  p.rotate = t.rotate > 0 || (t.rotate != 0 && beyond_cache);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, mem, grid, lds, s, p);
