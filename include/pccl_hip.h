@@ -200,7 +200,8 @@ typedef struct pccl_op_desc {
  * Chains: an op that depends on one op alone, which nothing else depends on and which is cut like
  * it, queues no entries of its own; the workgroup that has run part p of its predecessor goes on
  * with its part p (and keeps the value in registers where the op takes the predecessor's output 0
- * as one of at most two inputs).  A level of the graph whose entries start such chains is cut by
+ * as one of at most two inputs; an output that a later op of the same such chain writes again at the
+ * same address is then not stored by the earlier op: nothing could read it).  A level of the graph whose entries start such chains is cut by
  * the built-in choice into the smallest parts (from 8 KiB) with which its entries fit the resident
  * workgroups once.  Results, graph_status and graph_rebind are as without chains;
  * graph_info's n_tiles and the timeline count the entries that are queued.  PCCL_HIP_CHAINS=0

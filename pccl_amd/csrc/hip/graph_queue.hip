@@ -432,18 +432,37 @@ std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::ve
 
 // The rows of GraphControl::chain_table, from the payloads as they stand in the host image: for
 // every chain that runs in one pass, in op order of the heads, one row per op of the chain.
+// An output that a later op of the same chain writes again at the same address is left out of its
+// row: nothing can read the earlier value (the op's only successor is the next op of the chain, which
+// gets the value in registers, and whatever else the chain reads is nothing the chain writes), and
+// part p of the later op covers the same elements as part p of the earlier one.  In a ring
+// all-reduce the partial sums that the reduce-scatter steps leave in the ranks' output buffers are
+// such outputs, overwritten by the all-gather copies behind them: a chunk's chain then writes 8
+// streams instead of 14.
 void fill_chain_table(const std::vector<int> &words, int n_ops, const char *payloads, ForwardStep *rows) {
+  std::vector<const pccl_op_payload *> steps;
   for (int h = 0; h < n_ops; ++h) {
     if (!words[(size_t)kChainWords * h + kChainForward] || words[(size_t)kChainWords * h + kChainLength] < 2) continue;
     ForwardStep *row = rows + words[(size_t)kChainWords * h + kChainRow];
-    for (int u = h; u >= 0; u = words[(size_t)kChainWords * u + kChainNext], ++row) {
-      const pccl_op_payload *pl = (const pccl_op_payload *)(payloads + kPayloadStride * (size_t)u);
+    steps.clear();
+    for (int u = h; u >= 0; u = words[(size_t)kChainWords * u + kChainNext])
+      steps.push_back((const pccl_op_payload *)(payloads + kPayloadStride * (size_t)u));
+    size_t at = 0;
+    for (int u = h; u >= 0; u = words[(size_t)kChainWords * u + kChainNext], ++row, ++at) {
+      const pccl_op_payload *pl = steps[at];
       const int fed = u == h ? 0 : words[(size_t)kChainWords * u + kChainForward];
       row->fed = fed;
       row->other = (u != h && pl->n_in_ == 2) ? (unsigned long long)(uintptr_t)pl->chunks_[1 - fed].addr_ : 0ull;
-      row->n_out = pl->n_out_;
-      row->out[0] = (unsigned long long)(uintptr_t)pl->chunks_[pl->n_in_].addr_;
-      row->out[1] = pl->n_out_ > 1 ? (unsigned long long)(uintptr_t)pl->chunks_[pl->n_in_ + 1].addr_ : 0ull;
+      row->n_out = 0;
+      row->out[0] = row->out[1] = 0ull;
+      for (int j = 0; j < pl->n_out_; ++j) {
+        const void *addr = pl->chunks_[pl->n_in_ + j].addr_;
+        bool written_again = false;
+        for (size_t t = at + 1; t < steps.size() && !written_again; ++t)
+          for (int k = 0; k < steps[t]->n_out_; ++k)
+            if (steps[t]->chunks_[steps[t]->n_in_ + k].addr_ == addr) written_again = true;
+        if (!written_again) row->out[row->n_out++] = (unsigned long long)(uintptr_t)addr;
+      }
     }
   }
 }

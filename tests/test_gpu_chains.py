@@ -257,3 +257,35 @@ def test_chains_of_copies_with_an_element_size_of_their_own(hip, oracle):
                 H.assert_bits_equal(dev_buf.download(), want, "%s (reduce dtype %s, parts of %d)" % (what, reduce_dtype, tile))
                 assert dev_buf.guards_intact(), what
             g.destroy()
+
+
+def test_an_output_written_again_later_in_the_chain(hip, oracle):
+    """t, keep = a + b;  t = t + c (in place);  u = copy(t);  t = u + d (writes t a third time);  w = t + a: one
+    chain, run in one pass, which may skip the stores of t that it overwrites itself.  x = copy(t) and
+    y = t + keep run behind it and read what the chain left in memory, which must be what the ops leave
+    when run one by one."""
+    import torch
+    for count, tile in ((50021, 0), (9, 0), (2 * 1000 * 1000 + 3, 32 << 10)):
+        pool = Pool(torch, "bf16")
+        for k, n in enumerate("abcd"):
+            pool.add(n, count, 0, src=H.gen("bf16", count, 970, k))
+        names = ("t", "keep", "u", "w", "x", "y")
+        for n in names:
+            pool.add(n, count, 0)
+        ops = [dict(compute="sum", ins=["a", "b"], outs=["t", "keep"], count=count, deps=[]),
+               dict(compute="sum", ins=["t", "c"], outs=["t"], count=count, deps=[0]),
+               dict(compute="sum", ins=["t"], outs=["u"], count=count, deps=[1]),
+               dict(compute="sum", ins=["u", "d"], outs=["t"], count=count, deps=[2]),
+               dict(compute="sum", ins=["t", "a"], outs=["w"], count=count, deps=[3]),
+               dict(compute="sum", ins=["t"], outs=["x"], count=count, deps=[4]),
+               dict(compute="sum", ins=["t", "keep"], outs=["y"], count=count, deps=[4])]
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        plan = hip.plan_chains(pool.ops_for(ops, "dev"), [1] * 7, 2)
+        assert [p[0] for p in plan] == [1, 2, 3, 4, -1, -1, -1] and plan[0][1:3] == (5, 1)  # one chain of 5, one pass
+        g = hip.Graph(pool.ops_for(ops, "dev"), tile_bytes=tile)
+        for _ in range(2):
+            for n in names:
+                pool.dev[n].view().fill_(0xFF)
+            _run(torch, hip, g, 7)
+            pool.check(names, "count %d" % count)
+        g.destroy()
