@@ -800,6 +800,20 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
         for (int i : members) entries += std::max<long long>(1, (op_bytes[i] + part_bytes - 1) / part_bytes);
         if (entries <= rounds * (long long)cap || part_bytes >= (1 << 20)) break;
       }
+      // Uneven entries (ops of many sizes, most of them too short to cut) leave the round's last
+      // workgroups streaming alone: parts of 16 KiB, drawn by ticket in two or three rounds, even that
+      // out (4096-op schedule, ops of 8-224 KiB: 98 -> 89 us; uniform ring chunks lose with them).
+      if (part_bytes > (16 << 10)) {
+        long long entries = 0, longest = 0;
+        for (int i : members) {
+          const long long n = std::max<long long>(1, (op_bytes[i] + part_bytes - 1) / part_bytes);
+          entries += n;
+          longest = std::max(longest, (op_bytes[i] + n - 1) / n);
+        }
+        bool balance = true;
+        if (const char *env = getenv("PCCL_HIP_CHAIN_BALANCE")) balance = env[0] != '0';
+        if (balance && entries > 0 && longest * entries * 5 > bytes * 6) part_bytes = 16 << 10;  // longest > 1.2 x mean
+      }
       for (int i : members) {
         const int p = (int)std::max<long long>(1, std::min<long long>((op_bytes[i] + part_bytes - 1) / part_bytes, cap));
         for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext]) {
@@ -1045,8 +1059,12 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
   G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
   {
-    bool own = live_tiles <= (long long)G->n_wg;  // every entry has a workgroup to itself
-    if (const char *env = getenv("PCCL_HIP_OWN_ENTRIES")) own = own && env[0] != '0';
+    // entries without tickets (graph_queue_device.h): when they are few per workgroup; beyond one
+    // each the mapping of entries to workgroups needs every queue to have the same number of workgroups
+    long long rounds = 1;
+    if (const char *env = getenv("PCCL_HIP_OWN_ENTRIES")) rounds = atoll(env);
+    const bool own = rounds > 0 && (live_tiles <= (long long)G->n_wg ||
+                                    (G->n_wg % kQueues == 0 && live_tiles <= rounds * (long long)G->n_wg));
     ((int *)(img + off_qcount))[kQueues] = own ? 1 : 0;
   }
 

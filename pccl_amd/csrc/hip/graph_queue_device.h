@@ -506,12 +506,14 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   unsigned int *abort_flag = &hot[kHotAbort].value;
   const unsigned int spin_limit = g.spin_limit;
   const int home = blockIdx.x % kQueues;
-  // With no more entries than workgroups every workgroup has an entry to itself: workgroup b takes
-  // entry b of the global order (entry b / kQueues of its home queue) and leaves when that is done.
-  // No ticket is drawn, and no workgroup goes round the eight queues at the end to find each of them
-  // empty (eight returning atomics, one after the other: 14.9 -> 11 us for a graph of one 64 KiB op).
-  // Dependencies point backwards in the global order and workgroups are started in order, so the
-  // lowest-numbered workgroup still running never waits for one that has not started.
+  // Entries without tickets: workgroup b takes entries b, b + W, b + 2 W, ... of the global order (W
+  // workgroups; entry b / kQueues + k * W / kQueues of its home queue) and leaves when its home queue
+  // has no more.  No ticket is drawn, and no workgroup goes round the eight queues at the end to find
+  // each of them empty (eight returning atomics, one after the other: 14.9 -> 11 us for a graph of one
+  // 64 KiB op).  The host asks for it (mode word) when the entries are few per workgroup.
+  // Dependencies point backwards in the global order, a workgroup takes its entries in that order
+  // and workgroups are started in order, so the owner of the lowest-numbered unfinished entry is
+  // always at that entry and never waits for one that has not started.
   // The mode word sits behind the queue lengths in memory, not in the kernel arguments: a rebind can
   // change the number of entries (see GraphControl::queue_count).  Thread 0 reads it before its first
   // claim, together with the entry that would be its own (a load from inside the queue's room even
@@ -519,7 +521,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   constexpr unsigned int kOwnEntry = 1u << 31, kAllQueues = (1u << kQueues) - 1u;
   // Thread 0 keeps the queue lengths in LDS: it needs one at every claim, and a scalar load that has
   // dropped out of the cache costs a trip to the L2 behind the data traffic (0.6 us per part measured).
-  __shared__ int s_queue_count[kQueues + 1];
+  __shared__ int s_queue_count[kQueues + 1];  // [kQueues]: the workgroup's next entry on its home queue (entries without tickets)
+  const int own_stride = (int)((gridDim.x + kQueues - 1) / kQueues);
 
   // Loop shape matters: thread 0's bookkeeping for the part just finished and its
   // claim of the next entry sit in ONE conditional block per iteration, and the
@@ -551,12 +554,19 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       int first_q = -1, first_t = 0;
       unsigned int aborted = 0;
       unsigned long long own_e = 0;
+      // the workgroup's next entry without a ticket: its place on the home queue, requested at once if there is one
+      auto next_own = [&] {
+        const int t = s_queue_count[kQueues];
+        s_queue_count[kQueues] = t + own_stride;
+        if (t < s_queue_count[home]) own_e = g.queue_entries[home][t];
+        return t;
+      };
       auto draw_ticket = [&] {
         if (!h) {
           // The workgroup's first claim.  A ticket of its home queue is requested before the mode word
           // and the queue lengths are there (there are no more workgroups than entries at creation, so
-          // the home queue has an entry for it); with an entry of its own the ticket goes unused, and
-          // the queue heads it moved are set back with all the others when the run ends.
+          // the home queue has an entry for it); without tickets it goes unused, and the queue heads it
+          // moved are set back with all the others when the run ends.
           const int ticket = __hip_atomic_fetch_add(g.queue_head[home], 1, __ATOMIC_RELAXED, AGENT);
           const int mode = g.queue_count[kQueues];
           own_e = g.queue_entries[home][blockIdx.x / kQueues];
@@ -564,8 +574,9 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           for (int q = 0; q < kQueues; ++q) s_queue_count[q] = g.queue_count[q];
           first_q = home;
           if (mode) {
-            exhausted = kOwnEntry;
+            exhausted = kOwnEntry | (kAllQueues & ~(1u << home));  // (only the home queue is this workgroup's business)
             first_t = (int)(blockIdx.x / kQueues);
+            s_queue_count[kQueues] = first_t + own_stride;
           } else {
             first_t = ticket;
             aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
@@ -573,7 +584,9 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           return;
         }
         if (exhausted & kOwnEntry) {
-          exhausted |= kAllQueues;
+          first_q = home;
+          first_t = next_own();
+          aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
           return;
         }
         for (int i = 0; i < kQueues && first_q < 0; ++i) {
@@ -606,7 +619,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           if (q == first_q) {  // the ticket requested above
             t = first_t;
             first_q = -1;
-            if (exhausted & kOwnEntry) exhausted |= kAllQueues;  // (it is the only entry this workgroup takes)
+          } else if (exhausted & kOwnEntry) {  // (behind a signal op, which thread 0 has carried out itself)
+            t = next_own();
           } else if (n > 0) {
             t = __hip_atomic_fetch_add(g.queue_head[q], 1, __ATOMIC_RELAXED, AGENT);
           }

@@ -65,6 +65,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_ORDER_BLOCK");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAINS");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_OWN_ENTRIES");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAIN_BALANCE");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;

@@ -261,9 +261,14 @@ def _signal_ring_ops(world, size, signals_ptr, dev_in, dev_out, es=2, dtype="bf1
     return ops, sym
 
 
-def test_ring_allreduce_over_signal_words(hip, oracle):
+@pytest.mark.parametrize("size,tile,own_rounds", [(3001, 0, None), (30001, 8192, "16"), (30001, 8192, "0")])
+def test_ring_allreduce_over_signal_words(hip, oracle, monkeypatch, size, tile, own_rounds):
+    """(Second and third case: more entries than workgroups, taken without tickets in several rounds
+    per workgroup, and by ticket.)"""
     import torch
-    world, size = 8, 3001
+    if own_rounds is not None:
+        monkeypatch.setenv("PCCL_HIP_OWN_ENTRIES", own_rounds)
+    world = 8
     per = world * size
     host_in = [H.gen("bf16", per, 81 + it, 0) for it in range(2)]  # two runs, different inputs
     d_in = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
@@ -271,7 +276,8 @@ def test_ring_allreduce_over_signal_words(hip, oracle):
     signals = torch.zeros(64, dtype=torch.int32, device="cuda")
     ops, sym = _signal_ring_ops(world, size, signals.data_ptr(), d_in, d_out)
     assert sum(1 for o in ops if o.get("primitive") == 2) == world * (2 * world - 2)
-    g = hip.Graph(ops)
+    g = hip.Graph(ops, tile_bytes=tile)
+    assert tile == 0 or g.info()["n_tiles"] > g.info()["n_workgroups"]
     # CPU replay of the data ops: program order of creation is a valid order
     for it in range(2):
         ins = [H.gen("bf16", per, 90 + 10 * it, r) for r in range(world)]
