@@ -289,3 +289,92 @@ def test_an_output_written_again_later_in_the_chain(hip, oracle):
             _run(torch, hip, g, 7)
             pool.check(names, "count %d" % count)
         g.destroy()
+
+
+def _random_chain_graph(rng, torch, dtype, compute, count):
+    """Several chains in one graph.  Each chain: a first op with one or two inputs, then 1..19 ops that
+    mostly take the previous op's output 0 (as input 0 or 1, alone or with an outside buffer), sometimes
+    read an earlier output of the chain instead of an outside buffer, write one or two outputs, and
+    sometimes write over an earlier output of the chain or work in place.  Returns named buffers
+    (host + device) and the ops in both forms."""
+    es = H.ELEM_BYTES[dtype]
+    host, dev = {}, {}
+
+    def new(name, src=None):
+        off = int(rng.integers(0, 4)) * es if rng.random() < 0.5 else 0
+        host[name] = np.zeros(count, dtype=H.STORAGE[dtype]) if src is None else src
+        dev[name] = H.DevBuf(torch, dtype, count, off, src=src)
+        return name
+
+    kw = dict(kind="uniform", lo=0.5, hi=1.5) if compute == "prod" and dtype not in ("i32", "u32") else {}
+    if compute == "prod" and dtype in ("i32", "u32"):
+        kw = dict(lo=0, hi=3)
+    outside = [new("in%d" % k, H.gen(dtype, count, int(rng.integers(1 << 20)), k, **kw)) for k in range(4)]
+    ops = []
+    for c in range(int(rng.integers(1, 4))):
+        written = []  # buffers this chain has written (no other chain touches them; `outside` is read-only)
+        for s in range(int(rng.integers(2, 21))):
+            if s == 0:
+                ins = [outside[k] for k in rng.permutation(4)[:int(rng.integers(1, 3))]]
+            else:
+                handed = ops[-1]["outs"][0]
+                earlier = [n for n in written if n != handed]
+                r = rng.random()
+                if r < 0.35:
+                    ins = [handed]
+                elif r < 0.9 or not earlier:
+                    ins = [handed, outside[int(rng.integers(4))]]
+                else:  # reads something else the chain wrote earlier: such a chain goes through memory
+                    ins = [handed, earlier[int(rng.integers(len(earlier)))]]
+                if len(ins) == 2 and rng.random() < 0.5:
+                    ins.reverse()
+            outs = []
+            for j in range(1 if rng.random() < 0.75 else 2):
+                r = rng.random()
+                again = [n for n in written if n not in outs]
+                if r < 0.2 and again:
+                    outs.append(again[int(rng.integers(len(again)))])   # writes an earlier output again (maybe in place)
+                else:
+                    outs.append(new("c%d_%d_%d" % (c, s, j)))
+            ops.append(dict(compute=compute, ins=ins, outs=outs, count=count, deps=[len(ops) - 1] if s else []))
+            written += [n for n in outs if n not in written]
+    return host, dev, ops
+
+
+def test_random_chains(hip, oracle):
+    """Seeded sweep over chains of 2..20 ops with one or two inputs and outputs per op, operands at
+    arbitrary element-aligned offsets, ops that work in place, write over or read again what the chain
+    wrote earlier, all dtypes and folds, one part per op and several: bit for bit the memory that the
+    ops leave when run one after the other."""
+    import torch
+    scale = max(1, int(__import__("os").environ.get("PCCL_TEST_SWEEP_SCALE", "1")))
+    rng = np.random.default_rng(20240 + (0 if scale == 1 else 7919))
+    dtypes = ["f32", "i32", "bf16", "f16", "f8e4m3", "f8e5m2", "f64", "u32"]
+    one_pass = 0
+    for case in range(60 * scale):
+        dtype = dtypes[int(rng.integers(len(dtypes)))]
+        compute = ["sum", "prod", "min", "max"][int(rng.integers(4))]
+        count = int(np.exp(rng.uniform(0, np.log(200_000))))
+        host, dev, ops = _random_chain_graph(rng, torch, dtype, compute, count)
+        bound = lambda where: [dict(o, dtype=dtype, ins=[(host[n] if where == "host" else dev[n].ptr) for n in o["ins"]],
+                                    outs=[(host[n] if where == "host" else dev[n].ptr) for n in o["outs"]]) for o in ops]
+        oracle.run_ops(bound("host"))
+        tile = [0, 4096, 16 << 10, 1 << 20][int(rng.integers(4))]
+        plan = hip.plan_chains(bound("dev"), [1] * len(ops), H.ELEM_BYTES[dtype])
+        one_pass += sum(1 for p in plan if p[0] >= 0 and p[1] > 1 and p[2] == 1)
+        g = hip.Graph(bound("dev"), tile_bytes=tile)
+        for run in range(2):
+            _run(torch, hip, g, len(ops))
+            if run == 0:  # the second run starts from what the first left (in-place ops): compare after the first,
+                what = "case %d (%s %s count %d, %d ops, parts of %d)" % (case, dtype, compute, count, len(ops), tile)
+                for n in host:
+                    got, want = dev[n].download(), host[n]
+                    if dtype in ("f8e4m3", "f8e5m2"):  # any NaN encoding of the format counts as NaN
+                        wn, gn = np.isnan(oracle.widen(dtype, want)), np.isnan(oracle.widen(dtype, got))
+                        assert np.array_equal(wn, gn), what + ": NaN positions in " + n
+                        got, want = np.where(wn, 0, got), np.where(wn, 0, want)
+                    H.assert_bits_equal(got, want, what + ": " + n)
+                    assert dev[n].guards_intact(), what + ": wrote outside " + n
+                break
+        g.destroy()
+    assert one_pass >= 20 * scale  # the sweep does reach the one-pass code
