@@ -299,8 +299,8 @@ template <class D, class Op>
 __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const pccl_op_payload *hp, int n_steps, int first_row, long lo, long count) {
   typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
-  constexpr int kBatch = 2;  // packs a lane carries through the chain at a time (8 KiB per workgroup and stream)
-  constexpr int kAhead = 8;  // ops whose other input is requested ahead of the value reaching them
+  constexpr int kBatch = 4;  // packs a lane carries through the chain at a time (16 KiB per workgroup and stream)
+  constexpr int kAhead = 4;  // ops whose other input is requested ahead of the value reaching them
   __shared__ __attribute__((aligned(16))) ForwardStep s_step[kMaxForwardSteps];
   const int head_n_in = hp->n_in_;
   if (threadIdx.x < 2u * (unsigned)n_steps)  // two lanes per row
@@ -323,9 +323,13 @@ __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const p
     }
     // The loads of a chain depend on nothing the chain computes, so they go out well ahead of the
     // value: the first op's inputs and the other input of the ops among the next kAhead that have one,
-    // together (up to 18 packs per lane in flight), then fold and store op after op, then the next
-    // kAhead.  Loads never stand behind stores in the wavefront's queue (its wait counter treats
-    // completion as in order, and a write-through store's acknowledgement takes microseconds).
+    // together (up to 24 packs per lane in flight), then fold and store op after op, then the next
+    // kAhead.  Within a group no load stands behind a store in the wavefront's queue (its wait counter
+    // treats completion as in order, and a write-through store's acknowledgement takes microseconds).
+    // Bytes in flight per round trip count for more than round trips: 4 packs x 4 ops ahead against
+    // 2 x 8 (one group for a ring chunk's six folds instead of two): 4096-op schedule 89 -> 82 us, ring
+    // all-reduce 8 x 8 MiB 42 -> 34 us, 8 x 32 MiB 110 -> 97 us (8 x 1 MiB 16.5 -> 18.4 us: its 8 KiB
+    // parts are half a block); 3 x 6: 98 / 33 / 100 us.
     u32x4 cur[kBatch], in1[kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
