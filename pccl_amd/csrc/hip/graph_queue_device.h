@@ -85,8 +85,8 @@ constexpr unsigned long long kEntryChainHead = 1ull << 51;
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
 constexpr int kHotTotal = 1;      // *layout.total_operator (never written during a run)
 constexpr int kHotAbort = 2;      // set when a bounded wait gave up
-constexpr int kHotExit = 3;       // workgroups that have left the current run
-constexpr int kHotDone = 4;       // kQueues counters of finished ops, summed at the end
+constexpr int kHotExit = 3;       // 64 bits: workgroups that have left the current run | ops they completed << 32
+constexpr int kHotDone = 4;       // (kQueues words, unused: the ops completed are counted on kHotExit)
 constexpr int kHotRun = kHotDone + kQueues;  // number of the current run (first run = 1), bumped by the last workgroup out
 constexpr int kHotWords = kHotRun + 1;
 
@@ -154,7 +154,7 @@ __device__ __forceinline__ void run_part_body(const RcOperands &a, long head, lo
   }
   if (threadIdx.x >= kBlock - kWave)
     edge_elems<D, Op, NIN, kMemCoherent>(a, head, head + n_packs * kEpp, count, (int)threadIdx.x - (kBlock - kWave));
-  settle_stores();
+  // (the caller waits for the stores where someone will read them during the run)
 }
 
 // SLIM: only the variant that tolerates unaligned streams (keeps the any-dtype instance small).
@@ -406,7 +406,6 @@ __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const p
       }
     }
   }
-  settle_stores();
 }
 
 #define AGENT __HIP_MEMORY_SCOPE_AGENT
@@ -445,7 +444,7 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // behind the ticket (memory operations of a wavefront return in order).
 template <class DrawTicket>
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
-                                            const OpFacts &op, int uid, int part, int home, int chain_ops,
+                                            const OpFacts &op, int uid, int part, unsigned int *done_ops, int chain_ops,
                                             DrawTicket draw_ticket) {
   const int parts = op.parts;
   // successors that need only this part of the op (they come first in the successor list):
@@ -492,7 +491,7 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
   for (int s = n_part_next; s < n_next; ++s)
     __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
   // (an op that heads a chain stands for all the chain's ops: they ran behind it, part by part)
-  __hip_atomic_fetch_add(&g.hot[kHotDone + home].value, (unsigned int)chain_ops, __ATOMIC_RELAXED, AGENT);
+  *done_ops += (unsigned int)chain_ops;  // (the workgroup reports its count when it leaves)
   if (!drawn) draw_ticket();
 }
 
@@ -505,6 +504,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   __shared__ i32x4 s_chain;  // the claimed op's kChainWords words
   __shared__ int s_go;
   __shared__ int s_last;
+  __shared__ unsigned int s_done;  // ops this workgroup has completed (thread 0 only)
+  if (threadIdx.x == 0) s_done = 0;
   if constexpr (DT != kAnyDtype) Dtype<DT>::wave_init();
   HotWord *hot = g.hot;
   unsigned int *abort_flag = &hot[kHotAbort].value;
@@ -602,7 +603,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       };
       if (h) {
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, h, cur_op, cur_uid, cur_part, home, cur_chain_ops, draw_ticket);
+        finish_part(g, h, cur_op, cur_uid, cur_part, &s_done, cur_chain_ops, draw_ticket);
       } else {
         draw_ticket();
       }
@@ -700,7 +701,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, hc, OpFacts::of(sc), uid, 0, home, 1, [] {});
+        finish_part(g, hc, OpFacts::of(sc), uid, 0, &s_done, 1, [] {});
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
@@ -742,39 +743,44 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           if constexpr (DT == kAnyDtype) run_part_any(step, lo, n);
           else run_part<DT, Op>(step, lo, n);
           if (next < 0) break;
+          settle_stores();
           __syncthreads();
           step = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
           next = g.chain[kChainWords * next + kChainNext];
         }
       }
     }
-    // every store of this part has reached the point of coherence (run_part waits)
-    // before thread 0 hands the part over at the top of the next iteration; the
-    // barrier also keeps s_entry / s_go from being rewritten while still being read
+    // Every store of this part has reached the point of coherence before thread 0 hands the part
+    // over at the top of the next iteration: each wavefront waits for its own write-through stores,
+    // the barrier makes that true of the workgroup.  Where nobody is told (the op, or the chain's
+    // last op, has no successor in the graph) nobody reads the data before the kernel has ended,
+    // and the wait is left out: one memory round trip less for the last ops of a graph.
+    // The barrier also keeps s_entry / s_go from being rewritten while still being read.
+    if (cur_op.num_next_ops() > 0) settle_stores();
     __syncthreads();
   }
 
-  // leave: the last workgroup out re-arms the graph for the next run
+  // leave: the last workgroup out re-arms the graph for the next run.  One returning atomic per
+  // workgroup carries both facts, "one more has left" (low word) and "it completed this many ops"
+  // (high word), so the last one out has the total without reading anything else.  No wait
+  // stands before it: what the workgroup told others during the run (arrivals, counts put back for
+  // the next run) has either been waited for where it mattered or only matters to the next launch.
+  unsigned int total_done = 0;
   if (threadIdx.x == 0) {
-    settle_stores();  // this workgroup's counter updates land before it counts as gone
-    const unsigned int e = __hip_atomic_fetch_add(&hot[kHotExit].value, 1u, __ATOMIC_RELAXED, AGENT);
-    s_last = (e == gridDim.x - 1);
+    unsigned long long *exits = (unsigned long long *)&hot[kHotExit].value;  // (the word has a 256-byte line to itself)
+    const unsigned long long before = __hip_atomic_fetch_add(exits, ((unsigned long long)s_done << 32) | 1ull, __ATOMIC_RELAXED, AGENT);
+    s_last = ((unsigned int)before == gridDim.x - 1);
+    total_done = (unsigned int)(before >> 32) + s_done;
   }
   __syncthreads();
   if (!__builtin_amdgcn_readfirstlane(s_last)) return;
   if (threadIdx.x == 0) {
     const bool aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0;
-    unsigned int done = 0;
-    for (int q = 0; q < kQueues; ++q) {
-      done += __hip_atomic_load(&hot[kHotDone + q].value, __ATOMIC_RELAXED, AGENT);
-      // after an abort the per-op state is inconsistent: leave it for the host to restore
-      if (!aborted) {
-        __hip_atomic_store(&hot[kHotDone + q].value, 0u, __ATOMIC_RELAXED, AGENT);
-        __hip_atomic_store(g.queue_head[q], 0, __ATOMIC_RELAXED, AGENT);
-      }
-    }
-    __hip_atomic_store(&hot[kHotCompleted].value, done, __ATOMIC_RELAXED, AGENT);
-    __hip_atomic_store(&hot[kHotExit].value, 0u, __ATOMIC_RELAXED, AGENT);
+    // after an abort the per-op state is inconsistent: leave it for the host to restore
+    if (!aborted)
+      for (int q = 0; q < kQueues; ++q) __hip_atomic_store(g.queue_head[q], 0, __ATOMIC_RELAXED, AGENT);
+    __hip_atomic_store(&hot[kHotCompleted].value, total_done, __ATOMIC_RELAXED, AGENT);
+    __hip_atomic_store((unsigned long long *)&hot[kHotExit].value, 0ull, __ATOMIC_RELAXED, AGENT);
     __hip_atomic_fetch_add(&hot[kHotRun].value, 1u, __ATOMIC_RELAXED, AGENT);
   }
 }
