@@ -1,5 +1,6 @@
-"""GPU parity at the full sizes of the five baseline configurations.  Inputs are seeded on the
-device, downloaded once, and the CPU checker (threaded form, same arithmetic as the scalar form)
+"""GPU parity at the full sizes of the five baseline configurations.  Inputs are the CPU checker's
+seeded inputs (its splitmix64 counter generator, evaluated on the device and pinned against the host
+form), downloaded once, and the CPU checker (threaded form, same arithmetic as the scalar form)
 computes the expected bytes; every comparison is bit-exact."""
 import numpy as np
 import pytest
@@ -16,20 +17,58 @@ def _stream(torch):
     return torch.cuda.current_stream().cuda_stream
 
 
-def _dev_random(torch, dtype, count, seed, kind="normal", sigma=1.0, lo=0.5, hi=2.0):
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    if dtype == "i32":
-        return torch.randint(-(1 << 20), (1 << 20) + 1, (count,), dtype=torch.int32, device="cuda", generator=g)
-    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+_M64 = (1 << 64) - 1
+_GOLD = 0x9e3779b97f4a7c15
+
+
+def _s64(v):
+    """A 64-bit pattern as the signed value torch's int64 holds."""
+    v &= _M64
+    return v - (1 << 64) if v >> 63 else v
+
+
+def _mix64_int(z):
+    z &= _M64
+    z = ((z ^ (z >> 30)) * 0xbf58476d1ce4e5b9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94d049bb133111eb) & _M64
+    return z ^ (z >> 31)
+
+
+def _mix64_dev(z):
+    """splitmix64's finaliser on an int64 tensor: products wrap, shifts are made logical."""
+    lsr = lambda x, k: (x >> k) & ((1 << (64 - k)) - 1)
+    z = (z ^ lsr(z, 30)) * _s64(0xbf58476d1ce4e5b9)
+    z = (z ^ lsr(z, 27)) * _s64(0x94d049bb133111eb)
+    return z ^ lsr(z, 31)
+
+
+def _dev_random(torch, dtype, count, seed, kind="normal", sigma=1.0, lo=0.5, hi=2.0, stream=0):
+    """Seeded input generated ON the device by the CPU checker's own counter generator
+    (oracle/pccl_oracle.c: rng_u64 = splitmix64 finaliser over (seed, stream, index); fill_int32,
+    fill_uniform_f32, then the type's round-to-nearest-even narrowing), so that the full-size inputs are
+    those of H.gen(dtype, count, seed, stream, kind="uniform", ...) bit for bit without a host
+    pass over gigabytes (test_device_generator_is_the_host_generator checks windows of it).
+    kind "normal" asks for zero mean and the given sigma: uniform in [-sigma * sqrt 3, sigma * sqrt 3)."""
+    key = _mix64_int(seed * _GOLD + stream + 0x632be59bd9b4e019)
+    if kind == "normal":
+        lo, hi = -sigma * 1.7320508, sigma * 1.7320508
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16, "i32": torch.int32}[dtype]
     out = torch.empty(count, dtype=tdt, device="cuda")
-    step = 1 << 26
+    step = 1 << 25
     for a in range(0, count, step):
         b = min(count, a + step)
-        if kind == "normal":
-            out[a:b] = (torch.randn(b - a, device="cuda", generator=g) * sigma).to(tdt)
+        idx = torch.arange(a + 1, b + 1, dtype=torch.int64, device="cuda")
+        x = _mix64_dev(idx * _s64(_GOLD) + _s64(key))
+        if dtype == "i32":
+            span = (1 << 21) + 1          # values in [-2^20, 2^20]
+            hi32, lo32 = (x >> 32) & 0xffffffff, x & 0xffffffff
+            out[a:b] = ((hi32 * ((1 << 32) % span) + lo32) % span - (1 << 20)).to(torch.int32)   # x mod span, x unsigned
         else:
-            out[a:b] = (torch.rand(b - a, device="cuda", generator=g) * (hi - lo) + lo).to(tdt)
+            u = ((x >> 40) & 0xffffff).to(torch.float32) * (1.0 / 16777216.0)
+            lo32f, d32f = np.float32(lo), np.float32(np.float32(hi) - np.float32(lo))
+            v = u * float(d32f)          # two roundings, as the checker's lo + (hi - lo) * u without contraction
+            v = v + float(lo32f)
+            out[a:b] = v.to(tdt)
     return out
 
 
@@ -45,6 +84,22 @@ def _expect(oracle, dtype, compute, host_ins):
     out = np.empty_like(host_ins[0])
     oracle.reduce_copy(dtype, compute, host_ins, [out], nthreads=THREADS)
     return out
+
+
+def test_device_generator_is_the_host_generator(hip, oracle):
+    """The inputs of the full-size tests are the CPU checker's seeded inputs: windows at the start, across
+    a chunk boundary of the device loop and at the end agree bit for bit, for every dtype used."""
+    import torch
+    count = (1 << 25) + 4099
+    windows = [slice(0, 1 << 16), slice((1 << 25) - 999, (1 << 25) + 999), slice(count - 4099, count)]
+    for dtype, kw, host_kw in (("i32", {}, dict(lo=-(1 << 20), hi=1 << 20)),
+                               ("f32", dict(kind="uniform", lo=0.5, hi=2.0), dict(kind="uniform", lo=0.5, hi=2.0)),
+                               ("bf16", dict(sigma=1e-2), dict(kind="uniform", lo=-1e-2 * 1.7320508, hi=1e-2 * 1.7320508)),
+                               ("f16", dict(kind="uniform", lo=-2.0, hi=2.0), dict(kind="uniform", lo=-2.0, hi=2.0))):
+        dev = _host(_dev_random(torch, dtype, count, 77, stream=3, **kw), dtype)
+        want = H.gen(dtype, count, 77, 3, **host_kw)
+        for w in windows:
+            H.assert_bits_equal(dev[w], want[w], "%s window %s" % (dtype, w))
 
 
 def test_config2_ring_rank_share_full_size(hip, oracle):
