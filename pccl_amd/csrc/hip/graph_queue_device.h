@@ -86,8 +86,7 @@ constexpr int kHotCompleted = 0;  // *layout.completed_operator
 constexpr int kHotTotal = 1;      // *layout.total_operator (never written during a run)
 constexpr int kHotAbort = 2;      // set when a bounded wait gave up
 constexpr int kHotExit = 3;       // 64 bits: workgroups that have left the current run | ops they completed << 32
-constexpr int kHotDone = 4;       // (kQueues words, unused: the ops completed are counted on kHotExit)
-constexpr int kHotRun = kHotDone + kQueues;  // number of the current run (first run = 1), bumped by the last workgroup out
+constexpr int kHotRun = 4;        // number of the current run (first run = 1), bumped by the last workgroup out
 constexpr int kHotWords = kHotRun + 1;
 
 // What a workgroup needs to run a part, on lines nothing writes during a run: the
