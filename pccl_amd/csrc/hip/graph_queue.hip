@@ -413,6 +413,16 @@ std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::ve
           }
       }
     }
+    // Two ops of the chain may write the same elements only at the same address (the later store then
+    // comes from the same lane, behind the earlier one, or replaces it: fill_chain_table); ranges that
+    // overlap at a shift would be written by different lanes in no particular order.
+    for (size_t s1 = 0; forward && s1 < steps.size(); ++s1)
+      for (size_t s2 = s1 + 1; forward && s2 < steps.size(); ++s2)
+        for (int j = 0; j < ops[steps[s1]].n_out && forward; ++j)
+          for (int k = 0; k < ops[steps[s2]].n_out && forward; ++k) {
+            const uintptr_t x = (uintptr_t)ops[steps[s1]].outs[j], y = (uintptr_t)ops[steps[s2]].outs[k];
+            if (x != y && x < y + len && y < x + len) forward = false;
+          }
     // ... and the first op's inputs too (an in-place first op is fine: it reads before it writes, pack by pack)
     for (int k = 0; forward && k < ops[h].n_in; ++k)
       for (size_t s = 1; s < steps.size() && forward; ++s)

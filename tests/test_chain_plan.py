@@ -86,6 +86,16 @@ def test_one_pass_needs_the_predecessors_output_as_an_input_and_no_other_look_at
     assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 0
 
 
+def test_outputs_of_a_one_pass_chain_may_coincide_but_not_overlap_at_a_shift():
+    a, b, c, t, u = (buf(k) for k in range(5))
+    same = [op([a, b], [t], []), op([t, c], [u], [0]), op([u], [t], [1])]          # writes t again, same address
+    assert hip.plan_chains(same, [1, 1, 1], ES)[0][1:3] == (3, 1)
+    shifted = [op([a, b], [t], []), op([t, c], [u], [0]), op([u], [t + 64], [1])]  # overlaps t 64 bytes on
+    assert hip.plan_chains(shifted, [1, 1, 1], ES)[0][1:3] == (3, 0)
+    apart = [op([a, b], [t], []), op([t, c], [u], [0]), op([u], [t + 1000 * ES], [1])]  # just behind t
+    assert hip.plan_chains(apart, [1, 1, 1], ES)[0][1:3] == (3, 1)
+
+
 def test_one_pass_limits():
     bufs = [buf(k) for k in range(64)]
     chain = lambda n: [op([bufs[k], bufs[40]], [bufs[k + 1]], [k - 1] if k else []) for k in range(n)]

@@ -378,3 +378,37 @@ def test_random_chains(hip, oracle):
                 break
         g.destroy()
     assert one_pass >= 20 * scale  # the sweep does reach the one-pass code
+
+
+def test_later_op_writes_over_an_earlier_output_at_a_shift(hip, oracle):
+    """t = a + b;  u = t + c;  t[16:] = copy(u): the last op's output overlaps the first op's 16 elements
+    further on.  Different lanes would write those elements in a one-pass chain, so the chain goes
+    through memory, where the later op's values are the ones that stay."""
+    import torch
+    for count in (1000, 300007):
+        a, b, c = (H.gen("f32", count, 980, k) for k in range(3))
+        da, db, dc = (H.DevBuf(torch, "f32", count, 0, src=x) for x in (a, b, c))
+        dt, du = H.DevBuf(torch, "f32", count + 16, 0), H.DevBuf(torch, "f32", count, 0)
+        ht, hu = np.zeros(count + 16, dtype=np.float32), np.zeros(count, dtype=np.float32)
+        ht.view(np.uint32)[:] = 0xFFFFFFFF
+        host_ops = [dict(dtype="f32", compute="sum", ins=[a, b], outs=[ht[:count]], count=count),
+                    dict(dtype="f32", compute="sum", ins=[ht[:count], c], outs=[hu], count=count),
+                    dict(dtype="f32", compute="sum", ins=[hu], outs=[ht[16:]], count=count)]
+        oracle.run_ops(host_ops)
+        ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+               dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0]),
+               dict(dtype="f32", compute="sum", ins=[du.ptr], outs=[dt.ptr + 64], count=count, deps=[1])]
+        plan = hip.plan_chains(ops, [1, 1, 1], 4)
+        assert [p[0] for p in plan] == [1, 2, -1] and plan[0][2] == 0   # one chain, not in one pass
+        g = hip.Graph(ops, tile_bytes=1 << 22)   # one part per op (several parts: the last dependency waits for the whole op)
+        for _ in range(3):
+            dt.view().fill_(0xFF)
+            _run(torch, hip, g, 3)
+            H.assert_bits_equal(dt.download(), ht, "t, count %d" % count)
+            H.assert_bits_equal(du.download(), hu, "u, count %d" % count)
+        g.destroy()
+        g = hip.Graph(ops, tile_bytes=16 << 10)
+        dt.view().fill_(0xFF)
+        _run(torch, hip, g, 3)
+        H.assert_bits_equal(dt.download(), ht, "t, count %d, several parts" % count)
+        g.destroy()
