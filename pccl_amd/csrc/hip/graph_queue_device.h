@@ -501,6 +501,8 @@ template <int DT, class Op, bool FORWARD>
 __device__ __forceinline__ void drain_body(const GraphControl &g) {
   __shared__ unsigned long long s_entry;
   __shared__ i32x4 s_chain;  // the claimed op's kChainWords words
+  __shared__ i32x4 s_facts;  // ... its part count, successor list and dependency counts (OpFacts)
+  __shared__ long s_count;   // ... and its element count
   __shared__ int s_go;
   __shared__ int s_last;
   __shared__ unsigned int s_done;  // ops this workgroup has completed (thread 0 only)
@@ -609,6 +611,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       int go = 0;
       unsigned long long e = 0;
       i32x4 chain_words = {-1, 1, 0, 0};
+      i32x4 op_facts = {1, 0, 0, 0};
+      long op_count = 0;
       size_t entry_index = 0;  // of e in the global order
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
       // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
@@ -662,6 +666,11 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;
+        // ... and with them what every wavefront needs to cut the part (part count and successor list from
+        // the far end of the slot, the element count), handed over through LDS: read after the barrier
+        // they were one more memory round trip in front of every part
+        op_facts = i32x4{sc->parts, sc->succ_start, (int)*(const unsigned int *)&sc->payload.pre_dependencies_, 0};
+        op_count = sc->payload.chunks_[0].num_elems_;
         if (e & kEntryChainHead) chain_words = *(const i32x4 *)(g.chain + kChainWords * uid);
         else chain_words = i32x4{-1, 1, 0, 0};
         const unsigned int n_pred = (w12 & 0xffu) - part_preds;  // whole-op dependencies
@@ -706,6 +715,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       s_entry = e;
       s_go = go;
       s_chain = chain_words;
+      s_facts = op_facts;
+      s_count = op_count;
     }
     __syncthreads();
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
@@ -716,10 +727,12 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
     h = &g.headers[uid];
     slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
     const pccl_op_payload *pl = &slot->payload;
-    cur_op = OpFacts::of(slot);
+    cur_op.parts = __builtin_amdgcn_readfirstlane(s_facts[0]);
+    cur_op.succ_start = __builtin_amdgcn_readfirstlane(s_facts[1]);
+    cur_op.counts = (unsigned int)__builtin_amdgcn_readfirstlane(s_facts[2]);
     const int chain_next = __builtin_amdgcn_readfirstlane(s_chain[kChainNext]);
     cur_chain_ops = __builtin_amdgcn_readfirstlane(s_chain[kChainLength]);
-    const long count = pl->chunks_[0].num_elems_;
+    const long count = (long)uniform64((unsigned long long)s_count);
     const long per = part_elems(count, cur_op.parts);
     const long lo = (long)part * per;
     long n = count - lo;
