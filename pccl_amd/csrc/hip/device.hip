@@ -88,7 +88,7 @@ Tuning tuning() {
 // the cost of a pair being how often (over sampled offsets) the two agree in the group bits,
 // weighted as measured (pair_cost below).  bf16 8 -> 1 on nine buffers allocated one by one: 256 MiB
 // 6.6-6.65 -> 6.85-6.95 TB/s, 128 MiB 6.58 -> 6.7; over random starts the same kernel ranges from
-// 5.8 to 7.0 TB/s.
+// 5.8 to 7.0 TB/s.  (The probe that found the functions: probe/channel_hash_probe.hip, `make probe`.)
 namespace placement {
 
 inline unsigned bit(uint64_t a, int k) { return (unsigned)((a >> k) & 1u); }
