@@ -280,13 +280,15 @@ int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_
  * caller that replays recorded runs adds 65536 per replay itself. */
 int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
 
-/* Bounds every wait inside the drain kernel to `polls` polls of a queue slot
- * (default about 2 million, a few seconds).  When a wait gives up the kernel
+/* Bounds every wait inside the drain kernel (for a dependency, for a signal word) to `microseconds`
+ * by the device's constant 100 MHz clock (default 2,000,000: two seconds; the kernel looks at the clock
+ * every 64 polls).  A caller whose graphs wait for peers, or run beside long kernels of other
+ * streams, raises it.  When a wait gives up the kernel
  * raises its abort flag, every workgroup leaves, and pccl_hip_graph_status
  * returns PCCL_ERR_GRAPH after restoring the graph's pristine state.  Takes effect
  * with the next pccl_hip_graph_run (a run recorded by stream capture keeps the limit it
  * was recorded with). */
-int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls);
+int pccl_hip_graph_set_spin_limit(void *graph, unsigned int microseconds);
 
 /* pccl_hip_graph_create + pccl_hip_graph_run in one call that allocates NO device memory: the
  * graph's device state (headers, payloads, counters, ready queues: what graph_create puts into a

@@ -39,7 +39,7 @@
 //   * per-op mutable state is restored by the op's last part and the run's
 //     last workgroup rewinds the ticket counters, so a finished graph is armed
 //     for its next run;
-//   * every wait is bounded: when a wait exceeds spin_limit polls the kernel
+//   * every wait is bounded: when a wait has lasted spin_limit microseconds the kernel
 //     raises the abort flag, all workgroups leave, and the host reports
 //     PCCL_ERR_GRAPH instead of hanging.
 #include <algorithm>
@@ -1462,16 +1462,16 @@ int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base) {
   return PCCL_OK;
 }
 
-int pccl_hip_graph_set_spin_limit(void *graph, unsigned int polls) {
+int pccl_hip_graph_set_spin_limit(void *graph, unsigned int microseconds) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_set_spin_limit: graph is null");
-  if (polls < 64) polls = 64;
+  const unsigned int limit = std::max(microseconds, 64u);  // (the kernel looks at the clock every 64 polls anyway)
   std::lock_guard<std::mutex> lock(G->mu);
-  G->spin_limit = polls;
+  G->spin_limit = limit;
   if (G->as_launches) return PCCL_OK;  // nothing waits inside plain launches
-  ((GraphControl *)G->image.data())->spin_limit = polls;
-  PCCL_HIP_CHECK(hipMemcpy(G->dev + offsetof(GraphControl, spin_limit), &polls, sizeof(polls), hipMemcpyHostToDevice));
+  ((GraphControl *)G->image.data())->spin_limit = limit;
+  PCCL_HIP_CHECK(hipMemcpy(G->dev + offsetof(GraphControl, spin_limit), &limit, sizeof(limit), hipMemcpyHostToDevice));
   return PCCL_OK;
 }
 

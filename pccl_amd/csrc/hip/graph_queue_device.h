@@ -13,7 +13,7 @@ namespace pccl_queue {
 using namespace pccl_dev;
 
 constexpr int kQueues = 8;  // one per XCD of an MI355X
-constexpr unsigned int kDefaultSpinLimit = 1u << 21;  // a few seconds of polling
+constexpr unsigned int kDefaultSpinLimit = 2000000u;  // microseconds a wait inside the kernel may last
 
 // Words that many workgroups update or poll, each alone on its 256-byte line.
 // Device-scope atomics and sc1 loads are served at the memory side; an ordinary
@@ -418,17 +418,24 @@ constexpr int kTraceClaimed = 1;
 constexpr int kTraceReady = 2;
 constexpr int kTraceDone = 3;
 
-// Polls `ready` until it holds.  Gives up (and raises the abort word, so that every
-// workgroup leaves) after spin_limit polls or when another workgroup has given up.
+// Polls `ready` until it holds.  Gives up (and raises the abort word, so that every workgroup
+// leaves) once the wait has lasted spin_limit microseconds by the device's constant 100 MHz clock, or
+// when another workgroup has given up.  A time, not a number of polls: how fast a poll returns
+// depends on what else the device is doing.  (The clock is looked at every 64 polls.)
 template <class Ready>
 __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned int spin_limit, Ready ready) {
   unsigned int spins = 0;
+  unsigned long long since = 0;
   while (!ready()) {
     __builtin_amdgcn_s_sleep(1);
-    if ((++spins & 63u) == 0 &&
-        (spins >= spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0)) {
-      __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
-      return false;
+    if ((++spins & 63u) == 0) {
+      const unsigned long long now = wall_clock64();
+      if (spins == 64u) since = now;
+      if (now - since >= (unsigned long long)spin_limit * 100ull ||
+          __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0) {
+        __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);
+        return false;
+      }
     }
   }
   return true;

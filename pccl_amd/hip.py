@@ -305,8 +305,9 @@ class Graph:
         _check(lib().pccl_hip_graph_next_signal_base(self._h, ctypes.byref(b)))
         return b.value
 
-    def set_spin_limit(self, polls):
-        _check(lib().pccl_hip_graph_set_spin_limit(self._h, polls))
+    def set_spin_limit(self, microseconds):
+        """How long a wait inside the kernel may last before the run gives up (default two seconds)."""
+        _check(lib().pccl_hip_graph_set_spin_limit(self._h, microseconds))
 
     def info(self):
         lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)
