@@ -139,6 +139,12 @@ int pccl_hip_accumulate(int dtype, int compute, const void *in, void *const *out
  * 1 = non-temporal loads and stores, 2 = non-temporal loads and write-through stores). */
 int pccl_hip_set_tuning(int workgroups_per_cu, int cache_treatment);
 
+/* pccl_hip_reduce_copy and pccl_hip_accumulate launch one workgroup per 4 KiB of every operand, and a
+ * launch holds at most 2^24 - 1 of them (just under 64 GiB per operand): longer operands run as
+ * several launches over consecutive slices of `bytes` each (a multiple of 4096, at most and by default
+ * 32 GiB; 0 = the default).  Smaller values only serve tests of that path. */
+int pccl_hip_set_slice_bytes(long bytes);
+
 /* Occupancy override for tuning runs: bytes of (unused) dynamic LDS requested per
  * workgroup, which caps the workgroups resident on a compute unit at
  * floor(160 KiB / lds_bytes); -1 = built-in choice, 0 = no cap. */
@@ -300,7 +306,10 @@ int pccl_hip_graph_set_spin_limit(void *graph, unsigned int microseconds);
  * itself).  A graph that needs more than the array holds (about 4,500 ops of three parts each) is
  * refused with PCCL_ERR_NOMEM and nothing is launched.  completed / total both NULL: returns without
  * waiting.  Otherwise waits for `stream` and reports the two counters of operator.h:32-33
- * (PCCL_ERR_GRAPH if the drain gave up).  All calls on one GPU share the one array: a call waits for
+ * (PCCL_ERR_GRAPH if the drain gave up; the next call then uploads the state afresh).  A caller that
+ * always passes NULL for both never learns that a wait gave up: later calls with the same ops launch
+ * onto the abandoned state, where every workgroup leaves at once.  Graphs that wait for peers on signal
+ * words should read the counters at least now and then.  All calls on one GPU share the one array: a call waits for
  * the previous one's stream before it rewrites the state, and calls issued at the same time from
  * several threads or onto streams that overlap race.  Not meant to be recorded by stream capture (the
  * upload reads host memory). */

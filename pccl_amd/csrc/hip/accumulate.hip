@@ -179,6 +179,18 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
     p.out[j] = (char *)outs[j];
   }
   if (count == 0) return PCCL_OK;
+  // (one workgroup per 4 KiB of every stream, and a grid times its 256 lanes must fit 32 bits: operands
+  // beyond 32 GiB run as launches over consecutive slices of that size, like pccl_hip_reduce_copy's)
+  const long slice = pccl_host::slice_bytes() / es;
+  if (count > slice) {
+    for (long lo = 0; lo < count; lo += slice) {
+      void *out_at[PCCL_MAX_OUTPUTS];
+      for (int j = 0; j < n_out; ++j) out_at[j] = (char *)outs[j] + lo * es;
+      const int rc = pccl_hip_accumulate(dtype, compute, (const char *)in + lo * es, out_at, n_out, std::min(slice, count - lo), stream);
+      if (rc != PCCL_OK) return rc;
+    }
+    return PCCL_OK;
+  }
   p.n_out = n_out;
   p.count = count;
   p.head = std::min<long>(count, (long)((16 - ((uintptr_t)outs[0] & 15)) & 15) / es);
@@ -213,7 +225,8 @@ extern "C" int pccl_hip_accumulate(int dtype, int compute, const void *in, void 
     if (wgs < 8) lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
   }
   // the chunk order of large launches, as for reduce_copy (one workgroup per chunk here always)
-  p.rotate = t.rotate > 0 || (t.rotate != 0 && beyond_cache);
+  // (and, as there, not for operands of 4 GiB and more each)
+  p.rotate = t.rotate > 0 || (t.rotate != 0 && beyond_cache && count * es < (4l << 30));
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case PCCL_F32: return launch_acc_op<PCCL_F32>(compute, aligned, mem, grid, lds, s, p);

@@ -1070,7 +1070,11 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
   {
     // entries without tickets (graph_queue_device.h): when they are few per workgroup; beyond one
-    // each the mapping of entries to workgroups needs every queue to have the same number of workgroups
+    // each the mapping of entries to workgroups needs every queue to have the same number of workgroups.
+    // With one entry each a workgroup only ever waits for workgroups that were started before it; with
+    // more (PCCL_HIP_OWN_ENTRIES > 1, not the default) a workgroup's second entry can wait for the first
+    // entry of a workgroup that has no compute unit yet, which is only safe while nothing else keeps
+    // the launch from being resident as a whole.
     long long rounds = 1;
     if (const char *env = getenv("PCCL_HIP_OWN_ENTRIES")) rounds = atoll(env);
     const bool own = rounds > 0 && (live_tiles <= (long long)G->n_wg ||

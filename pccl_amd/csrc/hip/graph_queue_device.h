@@ -425,12 +425,12 @@ constexpr int kTraceDone = 3;
 template <class Ready>
 __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned int spin_limit, Ready ready) {
   unsigned int spins = 0;
-  unsigned long long since = 0;
+  unsigned long long since = 0;  // 0: the clock has not been looked at yet
   while (!ready()) {
     __builtin_amdgcn_s_sleep(1);
     if ((++spins & 63u) == 0) {
-      const unsigned long long now = wall_clock64();
-      if (spins == 64u) since = now;
+      const unsigned long long now = wall_clock64() | 1ull;
+      if (since == 0) since = now;
       if (now - since >= (unsigned long long)spin_limit * 100ull ||
           __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0) {
         __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, AGENT);

@@ -33,6 +33,10 @@ struct Tuning {
 };
 Tuning tuning();
 
+// Longest stretch of an operand, in bytes, that one launch of pccl_hip_reduce_copy / pccl_hip_accumulate
+// covers (a multiple of 4 KiB; see pccl_hip_set_slice_bytes).
+long slice_bytes();
+
 }  // namespace pccl_host
 
 #define PCCL_HIP_CHECK(expr)                                                              \

@@ -74,6 +74,21 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   if (count == 0) return PCCL_OK;
   const pccl_host::Tuning t = pccl_host::tuning();
   const int es = pccl_host::pccl_dtype_bytes(dtype);
+  // A grid times its 256 lanes must fit 32 bits: 2^24 - 1 workgroups of 4 KiB each, just under 64 GiB
+  // per stream.  Longer operands run as launches over consecutive slices of 32 GiB (a multiple of
+  // 4 KiB: every slice has the alignment of the whole, and the same launch shape).
+  const long slice = pccl_host::slice_bytes() / es;
+  if (count > slice) {
+    for (long lo = 0; lo < count; lo += slice) {
+      const void *in_at[PCCL_MAX_INPUTS];
+      void *out_at[PCCL_MAX_OUTPUTS];
+      for (int k = 0; k < n_in; ++k) in_at[k] = (const char *)ins[k] + lo * es;
+      for (int j = 0; j < n_out; ++j) out_at[j] = (char *)outs[j] + lo * es;
+      rc = pccl_hip_reduce_copy(dtype, compute, in_at, n_in, out_at, n_out, std::min(slice, count - lo), stream);
+      if (rc != PCCL_OK) return rc;
+    }
+    return PCCL_OK;
+  }
   // Operands that together exceed what the 256 MB Infinity Cache can hold run one
   // pack per lane under an occupancy cap (below).  Streaming treatment starts earlier,
   // at 48 MiB: a collective step works on data that just arrived and will not be
@@ -87,13 +102,15 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   //    chunks, 452 vs 433 us at 64 MiB, when every step uses the same treatment; MIXING
   //    them is worse than either (write-through reductions followed by non-temporal
   //    copies: 249 and 467 us), which is why one rule covers reductions and copies;
-  //  - reductions over several GiB: i32 4 -> 1 at 1 GiB per operand 6.1 vs 6.0, unaligned
-  //    5.9 vs 5.4.
+  //  - reductions of three and more inputs over several GiB: i32 4 -> 1 at 1 GiB per operand 6.1 vs
+  //    6.0, unaligned 5.9 vs 5.4; bf16 4 -> 1 at 4 / 8 / 32 GiB per operand 6.25 / 6.31 / 6.17 vs 6.18 /
+  //    6.21 / 6.13.  Copies and 2 -> 1 of that size stay with write-through stores: copy at 4 .. 32 GiB
+  //    6.3 vs 6.6, 2 -> 1 6.26-6.46 vs 6.30-6.55.
   const long total_bytes = (long)(n_in + n_out) * count * es;
   const bool big = total_bytes > (192l << 20);
   int mem = kLaunchMemCached;
   if (total_bytes >= (48l << 20)) {
-    const bool non_temporal_stores = (n_in == 1 && n_out >= 3) || total_bytes > (4l << 30);
+    const bool non_temporal_stores = (n_in == 1 && n_out >= 3) || (n_in >= 3 && total_bytes > (4l << 30));
     mem = non_temporal_stores ? kLaunchMemStream : kLaunchMemStreamWriteThrough;
   }
   if (t.cache_treatment >= 0) mem = std::min(t.cache_treatment, (int)kLaunchMemStreamWriteThrough);
@@ -148,7 +165,13 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   // 2 -> 2 6.06 / 6.00, 1 -> 1 5.85 / 5.50, 4 -> 1 6.27 / 5.66; walks over distinct buffers (what a collective
   // step sees), 32 MiB: 2 -> 2 5.67 / 6.02, 1 -> 1 5.73 / 5.92, 2 -> 1 5.97 / 6.23; 16 MiB: 5.44 / 5.76, 5.19 / 5.27,
   // 5.21 / 5.47.
-  p.rotate = total_bytes >= (48l << 20) && unroll <= 1 && grid == chunks && t.rotate != 0;
+  // Not for operands of 4 GiB and more each: there the outcome turns on address bits beyond those the
+  // rotation was fitted to.  Slices of one 160 GiB allocation, operand size / distance between operands,
+  // TB/s without / with: copy 8 GiB / 8 GiB 6.68 / 6.75 but 8 / 32 6.66 / 6.14 and 16 / 16 6.67 / 5.68;
+  // 2 -> 1 4 / 4 6.28 / 6.69 but 4 / 32 6.64 / 6.08, 8 / 32 6.64 / 5.74, 16 / 16 6.53 / 5.96; 4 -> 1 4 / 4 5.93 / 6.51 but
+  // 4 / 32 6.09 / 5.67, 16 / 32 6.12 / 5.57.  Without it every such case stays within 5.9-6.7; at 1 GiB per
+  // operand the rotation wins or ties at every distance (4 -> 1: 6.03 / 6.27 .. 6.10 / 6.25).
+  p.rotate = total_bytes >= (48l << 20) && count * es < (4l << 30) && unroll <= 1 && grid == chunks && t.rotate != 0;
   if (t.rotate > 0 && unroll <= 1 && grid == chunks) p.rotate = 1;
   hipStream_t s = (hipStream_t)stream;
   if (n_in == 1) return launch_copy(es, unroll, aligned, mem, (unsigned)grid, lds, s, p);

@@ -78,6 +78,7 @@ def lib():
         L.pccl_hip_set_occupancy_lds.argtypes = [ci]
         L.pccl_hip_set_unroll.argtypes = [ci]
         L.pccl_hip_set_rotation.argtypes = [ci]
+        L.pccl_hip_set_slice_bytes.argtypes = [cl]
         L.pccl_hip_graph_create.argtypes = [ctypes.POINTER(OpDesc), ci, cl, ctypes.POINTER(vp)]
         L.pccl_hip_graph_run_static.argtypes = [ctypes.POINTER(OpDesc), ci, cl, vp, ctypes.POINTER(ctypes.c_uint),
                                                 ctypes.POINTER(ctypes.c_uint)]
@@ -168,6 +169,11 @@ def placement_start(extent, nbytes, slack, before=()):
 
 def set_rotation(rotate=-1):
     _check(lib().pccl_hip_set_rotation(rotate))
+
+
+def set_slice_bytes(nbytes=0):
+    """Longest stretch of an operand that one launch covers (0: the built-in 32 GiB)."""
+    _check(lib().pccl_hip_set_slice_bytes(nbytes))
 
 
 def set_tuning(workgroups_per_cu=0, cache_treatment=-1):

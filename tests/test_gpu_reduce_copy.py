@@ -278,6 +278,44 @@ def test_every_kernel_variant_through_the_knobs(hip, oracle):
         hip.set_occupancy_lds(-1)
 
 
+def test_operands_longer_than_one_launch_covers(hip, oracle):
+    """Operands beyond what a launch's grid can cover (32 GiB by default) run as several launches over
+    consecutive slices.  With the slice set to 64 KiB and 4 KiB: ragged counts, operands off the 16-byte
+    grid, reduce-copy and accumulate, against the checker; and the setter's argument checks."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    try:
+        for slice_bytes in (65536, 4096):
+            hip.set_slice_bytes(slice_bytes)
+            for dtype, compute, n_in, n_out, count, off in (("bf16", "sum", 8, 1, 100003, 0), ("f32", "max", 2, 2, 70001, 4),
+                                                            ("f8e4m3", "sum", 3, 1, 300001, 3), ("i32", "sum", 1, 3, 65537, 12),
+                                                            ("f64", "prod", 2, 1, 8192 * 3, 0), ("f16", "min", 4, 2, 32768, 2)):
+                es = H.ELEM_BYTES[dtype]
+                off = off // es * es
+                kw = dict(kind="uniform", lo=0.5, hi=2.0) if compute == "prod" else {}
+                ins = [H.gen(dtype, count, 410 + n_in, k, **kw) for k in range(n_in)]
+                want = oracle.reduce(dtype, compute, ins)
+                got = H.hip_reduce(torch, hip, dtype, compute, ins, n_out=n_out, in_offsets=[(off * (k + 1)) % 64 for k in range(n_in)],
+                                   out_offsets=[(off * (k + 2)) % 64 for k in range(n_out)])
+                for g in got:
+                    H.assert_bits_equal(g, want, "%s %s %d->%d count=%d slice=%d" % (dtype, compute, n_in, n_out, count, slice_bytes))
+                # accumulate: the first input folded into copies of the others
+                dsts = [H.DevBuf(torch, dtype, count, (off * (j + 1)) % 64, src=ins[min(j + 1, n_in - 1)]) for j in range(n_out)]
+                src = H.DevBuf(torch, dtype, count, off, src=ins[0])
+                hip.accumulate(dtype, compute, src.ptr, [d.ptr for d in dsts], count, stream)
+                torch.cuda.synchronize()
+                for j, d in enumerate(dsts):
+                    H.assert_bits_equal(d.download(), oracle.reduce(dtype, compute, [ins[min(j + 1, n_in - 1)], ins[0]]),
+                                        "accumulate %s %s count=%d slice=%d" % (dtype, compute, count, slice_bytes))
+                    assert d.guards_intact()
+        for bad in (100, 4097, -4096, (32 << 30) + 4096):
+            with pytest.raises(hip.PcclError) as e:
+                hip.set_slice_bytes(bad)
+            assert e.value.code == hip.ERR_INVALID_ARG
+    finally:
+        hip.set_slice_bytes(0)
+
+
 def test_group_allocation(hip, oracle):
     """pccl_hip_alloc_group: n buffers out of one allocation at the stated stride, usable as
     operands, freed through the first one."""
