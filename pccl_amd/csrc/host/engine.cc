@@ -171,6 +171,8 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
         throw;
       }
     } else {
+      // (the graph's device state goes away: every stream it may still be running on ends first)
+      if (op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
       op->executor->waitGraph(op->graph, stream);
       op->executor->destroyGraph(op->graph);
       op->graph = nullptr;
