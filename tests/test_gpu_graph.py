@@ -194,7 +194,7 @@ def test_bounded_wait_aborts_cleanly(hip, oracle):
            dict(dtype="f32", compute="sum", ins=[dt.ptr, db.ptr], outs=[du.ptr], count=count, deps=[0]),
            dict(dtype="f32", ins=[dt.ptr], outs=[dv.ptr], count=count, deps=[0])]
     g = hip.Graph(ops)
-    g.set_spin_limit(256)
+    g.set_spin_limit(20000)  # microseconds
     # GraphBufferLayout.operators (offset 16) -> headers; op 1's byte 12 is pre_dependencies_
     lay = g.info()["device_layout"]
     host = torch.empty(48, dtype=torch.uint8)
@@ -213,7 +213,7 @@ def test_bounded_wait_aborts_cleanly(hip, oracle):
         g.status(_stream(torch))
     assert e.value.code == hip.ERR_GRAPH
     # status restored the pristine graph: it runs correctly now
-    g.set_spin_limit(1 << 21)
+    g.set_spin_limit(2000000)
     _run_and_check(torch, hip, g, 3)
     H.assert_bits_equal(du.download(), oracle.reduce("f32", "sum", [oracle.reduce("f32", "sum", [a, b]), b]), "after reset")
     g.destroy()
@@ -311,7 +311,7 @@ def test_get_notified_from_outside_and_never(hip, oracle):
     ops = [dict(primitive=3, signal=sig.data_ptr(), value=7, deps=[]),
            dict(dtype="f32", compute="sum", ins=[da.ptr], outs=[do.ptr], count=count, deps=[0])]
     g = hip.Graph(ops)
-    g.set_spin_limit(512)
+    g.set_spin_limit(20000)  # microseconds
     base = g.next_signal_base()
     sig[0] = base + 7 - (1 << 32) if base + 7 >= (1 << 31) else base + 7
     torch.cuda.synchronize()
