@@ -626,16 +626,32 @@ def main():
                 note="median_us = one launch between two events; host_call_us = Python ctypes call incl. the library's "
                      "argument checks and hipLaunchKernel, nothing waited for; back_to_back = 2000 launches between two events")
 
-        # ---- unaligned operands: i32 4 -> 1, 2^28-57 elements, every buffer 4..60 bytes off 64 ----
+        # ---- unaligned operands: 4 -> 1, every buffer 4..60 bytes off a 64-byte boundary ----------
+        # (the counts of 2^24 elements and more from the list that the parity tests run; the four
+        # dtype / fold pairs at the longest prime count)
         if want("unaligned"):
-            cu = (1 << 28) - 57
-            pool = [torch.randint(-(1 << 20), 1 << 20, (cu + 64,), dtype=torch.int32, device="cuda") for _ in range(4)]
-            ou = torch.empty(cu + 64, dtype=torch.int32, device="cuda")
+            cmax = 1 << 28
             offs = [4, 12, 20, 60, 8]
-            ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
-            t = event_times_us(torch, lambda: hip.reduce_copy("i32", "sum", ptr_in, [ou.data_ptr() + offs[4]], cu, stream), 10, 2)
-            extras["unaligned_i32_4in_1out_1GiB"] = dict(stats(t), GBps_median=gbps(5 * 4 * cu, t[len(t) // 2]), byte_offsets=offs)
-            del pool, ou
+            ipool = [torch.randint(-(1 << 20), 1 << 20, (cmax + 64,), dtype=torch.int32, device="cuda") for _ in range(4)]
+            ou = torch.empty(cmax + 64, dtype=torch.int32, device="cuda")
+
+            def unaligned_leg(dtype, compute, pool, cu):
+                ptr_in = [pool[k].data_ptr() + offs[k] for k in range(4)]
+                t = event_times_us(torch, lambda: hip.reduce_copy(dtype, compute, ptr_in, [ou.data_ptr() + offs[4]], cu, stream), 20, 5)
+                return dict(stats(t), GBps_median=gbps(5 * 4 * cu, t[len(t) // 2]))
+
+            cu = (1 << 28) - 57
+            extras["unaligned_i32_4in_1out_1GiB"] = dict(unaligned_leg("i32", "sum", ipool, cu), byte_offsets=offs)
+            other = {}
+            for c, label in (((1 << 24) - 3, "2^24-3"), (1 << 28, "2^28")):
+                other["i32_sum_count_" + label] = unaligned_leg("i32", "sum", ipool, c)
+            other["i32_max_count_2^28-57"] = unaligned_leg("i32", "max", ipool, cu)
+            del ipool
+            fpool = [torch.empty(cmax + 64, dtype=torch.float32, device="cuda").uniform_(0.5, 2.0) for _ in range(4)]
+            other["f32_min_count_2^28-57"] = unaligned_leg("f32", "min", fpool, cu)
+            other["f32_prod_count_2^28-57"] = unaligned_leg("f32", "prod", fpool, cu)
+            extras["unaligned_i32_4in_1out_1GiB"]["other_counts_and_folds"] = other
+            del fpool, ou
 
         # ---- small ops: 64 KiB direct launch and through the queue --------------------------
         if want("op64k"):
