@@ -36,6 +36,26 @@ def test_every_declared_symbol_is_exported():
             assert hasattr(L, n), "%s declares %s but %s does not export it" % (header, n, os.path.basename(path))
 
 
+def test_host_only_entry_points_answer_without_a_device():
+    """The entry points that touch no device: element sizes by dtype code, the version string, the
+    setters' argument checks, the error text of the calling thread."""
+    from pccl_amd import hip
+    L = hip.lib()
+    for name, code in hip.DTYPES.items():
+        assert L.pccl_hip_dtype_bytes(code) == H.ELEM_BYTES[name], name
+    assert L.pccl_hip_dtype_bytes(99) == 0
+    L.pccl_hip_version.restype = ctypes.c_char_p
+    assert b"gfx950" in L.pccl_hip_version()
+    with pytest.raises(hip.PcclError) as e:
+        hip.set_slice_bytes(4097)
+    assert e.value.code == hip.ERR_INVALID_ARG and "4096" in str(e.value)
+    hip.set_slice_bytes(0)
+    with pytest.raises(hip.PcclError):
+        hip.set_rotation(5)
+    with pytest.raises(hip.PcclError):
+        hip.set_unroll(3)
+
+
 def test_layout_header_compiles_as_c_and_matches_reference_offsets(tmp_path):
     """pccl_op_layout.h is plain C; offsets are those of the reference's operator.h / chunk.h (LP64)."""
     src = tmp_path / "t.c"
