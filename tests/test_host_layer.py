@@ -432,3 +432,29 @@ def test_bench_refuses_more_than_one_gpu():
                        capture_output=True, text=True, timeout=60)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_product_uses_neither_the_checker_nor_working_files():
+    """The CPU checker under oracle/ is test infrastructure: nothing in the package or the public
+    headers may import, link or name it (or the builder's scratch folder); only tests/, smoke() and
+    the CPU-baseline leg of bench.py do."""
+    bad = []
+    pattern = re.compile(r"\boracle\b|\b_work\b|pccl_oracle")
+    for top in ("pccl_amd", "include"):
+        for folder, _, files in os.walk(os.path.join(ROOT, top)):
+            if "__pycache__" in folder or os.path.join("csrc", "build") in folder:
+                continue
+            for name in files:
+                if not name.endswith((".py", ".cc", ".h", ".hip", "Makefile")):
+                    continue
+                path = os.path.join(folder, name)
+                for n, line in enumerate(open(path, errors="replace"), 1):
+                    if pattern.search(line):
+                        bad.append("%s:%d: %s" % (os.path.relpath(path, ROOT), n, line.strip()))
+    assert not bad, "\n".join(bad)
+    # bench.py reaches the checker in its CPU-baseline leg only
+    lines = open(os.path.join(ROOT, "bench.py")).read().split("\n")
+    uses = [n for n, line in enumerate(lines) if re.search(r"\boracle\b", line) and not line.lstrip().startswith("#")]
+    start = next(n for n, line in enumerate(lines) if line.startswith("def cpu_baseline"))
+    end = next(n for n in range(start + 1, len(lines)) if lines[n].startswith("def "))
+    assert uses and all(start <= n < end for n in uses), [lines[n] for n in uses if not start <= n < end]
