@@ -406,10 +406,23 @@ int pccl_hip_free(void *p) {
   clear_error();
   if (!p) return PCCL_OK;
   // like hipFree, which this replaces for the caller: work that may still use the memory ends first
-  PCCL_HIP_CHECK(hipDeviceSynchronize());
+  // (on the device that holds it, which need not be the calling thread's current one)
+  int owner = -1, current = -1;
+  {
+    std::lock_guard<std::mutex> lock(g_mem_mutex);
+    auto it = mem_map().find(p);
+    if (it == mem_map().end())
+      return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_free: %p was not allocated by pccl_hip_alloc", p);
+    owner = it->second.slab->device;
+  }
+  PCCL_HIP_CHECK(hipGetDevice(&current));
+  if (owner != current) PCCL_HIP_CHECK(hipSetDevice(owner));
+  const hipError_t synced = hipDeviceSynchronize();
+  if (owner != current) PCCL_HIP_CHECK(hipSetDevice(current));
+  PCCL_HIP_CHECK(synced);
   std::lock_guard<std::mutex> lock(g_mem_mutex);
   auto it = mem_map().find(p);
-  if (it == mem_map().end())
+  if (it == mem_map().end())  // (another thread freed it meanwhile)
     return fail(PCCL_ERR_INVALID_ARG, "pccl_hip_free: %p was not allocated by pccl_hip_alloc", p);
   const Block b = it->second;
   mem_map().erase(it);
