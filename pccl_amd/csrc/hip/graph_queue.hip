@@ -8,7 +8,8 @@
 //     output (built-in choice: sized per dependency level, see "parts" below);
 //     a queue entry names (op_uid, part);
 //   * the entries of all ops are laid out once, at graph creation, in a
-//     topological order (dependency level, then op id, then part) and dealt
+//     topological order (dependency level; inside a level by where the ops'
+//     predecessors stand, then op id, the ops taking turns with blocks of parts) and dealt
 //     round-robin onto kQueues ready queues (GraphBufferLayout::ready_queues /
 //     num_queues; RingBuffer::tail_ = number of entries).  Workgroup w serves
 //     queue w % kQueues first -- workgroups are dispatched round-robin over the 8
@@ -26,6 +27,11 @@
 //   * where a successor is cut like the op and touches the same bytes part for part,
 //     its part p waits only for the op's part p (classify_dependencies below): every
 //     part of the op bumps the word of the successor's entry p when it is complete;
+//   * an op that follows one op alone, which nothing else needs, queues no entries: the
+//     workgroup that ran part p of the one goes on with part p of the other (plan_chains
+//     below), and where the value can stay in registers the whole chain is one pass;
+//   * when there are no more entries than workgroups, workgroup b simply takes entry b
+//     (no tickets; the mode word beside the queue lengths says so);
 //   * data moves between workgroups (possibly on different XCDs, whose L2s are not
 //     coherent with each other) through device-coherent accesses: parts load and
 //     store with sc1, wait for their stores, and only then touch the counters with
