@@ -211,7 +211,13 @@ typedef struct pccl_op_desc {
  * the built-in choice into the smallest parts (from 8 KiB) with which its entries fit the resident
  * workgroups once.  Results, graph_status and graph_rebind are as without chains;
  * graph_info's n_tiles and the timeline count the entries that are queued.  PCCL_HIP_CHAINS=0
- * switches chains off. */
+ * switches chains off.
+ * Signal ops that stand alone beside one data op ride on it: a NOTIFY whose only dependency is a
+ * COPY / REDUCE is stored by whoever completes that op, and a GET_NOTIFIED that one COPY / REDUCE
+ * alone depends on is polled by every part of that op (which takes over its dependencies); neither
+ * queues an entry, both count as complete with the data op.  In the device image the successor list
+ * of an op that carries a NOTIFY ends in -1 (next_op_uids_head_, num_next_ops_ counts it).
+ * PCCL_HIP_FUSE_SIGNALS=0 keeps every signal op an op of its own. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
@@ -252,8 +258,9 @@ int pccl_hip_graph_read_trace(void *graph, void *stream, unsigned long long *rec
 /* How the executor treats each dependency of the graph (no counterpart in the reference):
  * one byte per dependency, ops in uid order and each op's dependencies in list order;
  * 1 = met part by part (part p of the op waits only for part p of that predecessor, see
- * pccl_op_layout.h), 0 = the op waits for the whole predecessor.  Copies up to `capacity`
- * bytes and reports the number of dependencies in *n_deps.  graph_rebind may change it. */
+ * pccl_op_layout.h), 0 = the op waits for the whole predecessor (also reported for a dependency
+ * from or on a signal op that rides on a data op: the data op does that waiting).  Copies up to
+ * `capacity` bytes and reports the number of dependencies in *n_deps.  graph_rebind may change it. */
 int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capacity, long *n_deps);
 
 /* The rule behind that, on its own: given the ops and the number of parts each is cut into

@@ -30,6 +30,9 @@
 //   * an op that follows one op alone, which nothing else needs, queues no entries: the
 //     workgroup that ran part p of the one goes on with part p of the other (plan_chains
 //     below), and where the value can stay in registers the whole chain is one pass;
+//   * a NOTIFY behind one data op alone, and a GET_NOTIFIED in front of one data op alone, queue no
+//     entries either: the op's last part stores the one word, every part of the op polls the other
+//     (fuse_signals below);
 //   * when there are no more entries than workgroups, workgroup b simply takes entry b
 //     (no tickets; the mode word beside the queue lengths says so);
 //   * data moves between workgroups (possibly on different XCDs, whose L2s are not
@@ -115,6 +118,13 @@ struct Graph {
   std::vector<int> n_succ;                 // per op: ops that depend on it
   std::vector<unsigned char> order_touch;  // per op: takes part in a NOTIFY -> GET_NOTIFIED ordering edge
   std::vector<int> chain_words;            // kChainWords ints per op, as uploaded
+  // signal ops carried by data ops (fuse_signals): what build_graph works on
+  std::vector<pccl_op_desc> eff;           // descs with the dependency lists rewritten; deps point into eff_deps
+  std::vector<int> eff_deps;
+  std::vector<int> fused_into;             // per op: the data op that carries this signal op, or -1
+  std::vector<int> wait_of, notify_of;     // per op: the GET_NOTIFIED / NOTIFY it carries, or -1
+  std::vector<long> user_dep_to_eff;       // per dependency as the caller listed them: its place among eff's, or -1
+  size_t fuse_table_off = 0;               // arena offset of the carried signals' table (behind the chain table)
   std::vector<int> fixed_parts;            // build_graph: cut the ops like this instead of choosing (a rebuild in place:
                                            // the arena's layout, and with it its size, follows from the part counts)
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
@@ -344,6 +354,118 @@ bool plan_launches(const std::vector<pccl_op_desc> &ops, std::vector<pccl_op_des
   return take;
 }
 
+// ---- signal ops carried by data ops ------------------------------------------------
+// A ring written the way ranks on different devices write it is, per step, GET_NOTIFIED -> data op ->
+// NOTIFY, each a queue entry of its own with a hand-over through the arrival words between them (about
+// 2.5 us each: a ring all-reduce over 8 resident ranks x 1 MiB took 106 us with signals against 18 us
+// with plain dependencies).  Where the shape allows, the data op carries its neighbours instead:
+//   * a NOTIFY that depends on one data op alone is stored by whoever completes that op (its last
+//     part), and whatever depended on the NOTIFY depends on the data op;
+//   * a GET_NOTIFIED that one data op alone depends on is polled by every part of that op before it
+//     starts, and the op takes over the GET_NOTIFIED's own dependencies.
+// A carried signal op queues no entry and is complete when its data op is.  One of each kind per data
+// op; anything else stays an op of its own.  The plan depends on the ops' kinds and dependency lists
+// only, never on addresses, so a rebind cannot change it.  PCCL_HIP_FUSE_SIGNALS=0 switches it off.
+void fuse_signals(Graph *G) {
+  const std::vector<pccl_op_desc> &user = G->descs;
+  const int n = (int)user.size();
+  G->fused_into.assign(n, -1);
+  G->wait_of.assign(n, -1);
+  G->notify_of.assign(n, -1);
+  bool on = true;
+  if (const char *env = getenv("PCCL_HIP_FUSE_SIGNALS")) on = env[0] != '0';
+  std::vector<std::vector<int>> deps(n);
+  bool sane = true;
+  for (int i = 0; i < n && sane; ++i) {
+    const pccl_op_desc &o = user[i];
+    sane = o.n_deps >= 0 && (o.n_deps == 0 || o.deps) && o.primitive <= PCCL_GET_NOTIFIED;
+    for (int d = 0; sane && d < o.n_deps; ++d) {
+      sane = o.deps[d] >= 0 && o.deps[d] < n && o.deps[d] != i;
+      if (sane) deps[i].push_back(o.deps[d]);
+    }
+  }
+  auto is_data = [&](int i) { return user[i].primitive == PCCL_COPY || user[i].primitive == PCCL_REDUCE; };
+  if (on && sane) {
+    std::vector<int> n_succ(n, 0);
+    for (int i = 0; i < n; ++i)
+      for (int d : deps[i]) ++n_succ[d];
+    // NOTIFYs first: what depended on a carried NOTIFY then depends on its data op
+    std::vector<int> stands_for(n);
+    for (int i = 0; i < n; ++i) stands_for[i] = i;
+    for (int v = 0; v < n; ++v) {
+      if (user[v].primitive != PCCL_NOTIFY || deps[v].size() != 1) continue;
+      const int a = deps[v][0];
+      if (!is_data(a) || G->notify_of[a] >= 0 || n_succ[a] - 1 + n_succ[v] > 255) continue;
+      G->notify_of[a] = v;
+      G->fused_into[v] = a;
+      stands_for[v] = a;
+      n_succ[a] += n_succ[v] - 1;
+      n_succ[v] = 0;
+      deps[v].clear();
+    }
+    for (int i = 0; i < n; ++i) {
+      for (int &d : deps[i]) d = stands_for[d];
+      std::sort(deps[i].begin(), deps[i].end());
+      deps[i].erase(std::unique(deps[i].begin(), deps[i].end()), deps[i].end());
+    }
+    // GET_NOTIFIEDs that one data op alone waits for
+    std::vector<int> only_succ(n, -1), succ_count(n, 0);
+    for (int i = 0; i < n; ++i)
+      for (int d : deps[i]) {
+        ++succ_count[d];
+        only_succ[d] = i;
+      }
+    for (int v = 0; v < n; ++v) {
+      if (user[v].primitive != PCCL_GET_NOTIFIED || succ_count[v] != 1) continue;
+      const int b = only_succ[v];
+      if (!is_data(b) || G->wait_of[b] >= 0) continue;
+      std::vector<int> merged;
+      for (int d : deps[b])
+        if (d != v) merged.push_back(d);
+      merged.insert(merged.end(), deps[v].begin(), deps[v].end());
+      std::sort(merged.begin(), merged.end());
+      merged.erase(std::unique(merged.begin(), merged.end()), merged.end());
+      if (merged.size() > 255) continue;
+      G->wait_of[b] = v;
+      G->fused_into[v] = b;
+      deps[b].swap(merged);
+      deps[v].clear();
+    }
+  }
+  // the ops with the rewritten lists, and for every dependency the caller listed its place among them
+  G->eff = user;
+  G->eff_deps.clear();
+  G->user_dep_to_eff.clear();
+  if (!sane) return;  // (build_graph reports what is wrong with the lists, from the ops as they came)
+  std::vector<size_t> start(n + 1, 0);
+  for (int i = 0; i < n; ++i) {
+    start[i] = G->eff_deps.size();
+    G->eff_deps.insert(G->eff_deps.end(), deps[i].begin(), deps[i].end());
+  }
+  start[n] = G->eff_deps.size();
+  for (int i = 0; i < n; ++i) {
+    G->eff[i].n_deps = (int)(start[i + 1] - start[i]);
+    G->eff[i].deps = G->eff[i].n_deps > 0 ? G->eff_deps.data() + start[i] : nullptr;
+    for (int d = 0; d < user[i].n_deps; ++d) {
+      long place = -1;
+      if (G->fused_into[i] < 0 && G->fused_into[user[i].deps[d]] < 0)
+        for (size_t k = start[i]; k < start[i + 1]; ++k)
+          if (G->eff_deps[k] == user[i].deps[d]) place = (long)k;
+      G->user_dep_to_eff.push_back(place);
+    }
+  }
+}
+
+// G->eff with the operands of `moved` (the same ops at other addresses)
+std::vector<pccl_op_desc> effective_of(const Graph *G, const std::vector<pccl_op_desc> &moved) {
+  std::vector<pccl_op_desc> e = G->eff;
+  for (size_t i = 0; i < e.size(); ++i) {
+    memcpy(e[i].ins, moved[i].ins, sizeof(e[i].ins));
+    memcpy(e[i].outs, moved[i].outs, sizeof(e[i].outs));
+  }
+  return e;
+}
+
 // ---- chains -------------------------------------------------------------------
 // B follows A in a chain when B depends on A alone, A is needed by B alone, both are cut alike and
 // part p of B may start as soon as part p of A is complete (single-part ops: always; otherwise the
@@ -483,6 +605,36 @@ void fill_chain_table(const std::vector<int> &words, int n_ops, const char *payl
   }
 }
 
+// plan_chains for a graph's ops, and in the length word of every op the signal ops it carries: a
+// workgroup that completes the op counts those complete with it (such an op is in no chain, so the
+// word would otherwise say 1).
+std::vector<int> plan_chains_of(const Graph *G, const std::vector<pccl_op_desc> &ops, const std::vector<int> &parts,
+                                const std::vector<unsigned char> &part_edge, int forward_elem_bytes) {
+  std::vector<int> words = plan_chains(ops, parts, part_edge, G->n_succ, G->order_touch, forward_elem_bytes);
+  for (size_t i = 0; i < ops.size(); ++i)
+    words[(size_t)kChainWords * i + kChainLength] += (G->wait_of[i] >= 0) + (G->notify_of[i] >= 0);
+  return words;
+}
+
+// Rows of GraphControl::fuse: per data op the signal word and value it waits for before every part and
+// the ones it stores when its last part is complete (addresses as they stand in `ops`).
+void fill_fuse_table(const Graph *G, const std::vector<pccl_op_desc> &ops, SignalFuse *rows) {
+  for (size_t i = 0; i < ops.size(); ++i) {
+    SignalFuse f = {0ull, 0ull, 0u, 0u};
+    if (G->wait_of[i] >= 0) {
+      const pccl_op_desc &w = ops[G->wait_of[i]];
+      f.wait_word = (unsigned long long)(uintptr_t)w.ins[0];
+      f.wait_value = (unsigned int)w.count;
+    }
+    if (G->notify_of[i] >= 0) {
+      const pccl_op_desc &v = ops[G->notify_of[i]];
+      f.notify_word = (unsigned long long)(uintptr_t)v.outs[0];
+      f.notify_value = (unsigned int)v.count;
+    }
+    rows[i] = f;
+  }
+}
+
 // What pccl_hip_reduce_copy would refuse about a planned launch's operands, found at creation time.
 int check_launch(const pccl_op_desc &o) {
   const int es = elem_bytes(o.dtype);
@@ -504,8 +656,10 @@ struct FixedArena {
 
 int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t reuse_bytes = 0,
                 const FixedArena *fixed = nullptr) {
-  const pccl_op_desc *ops = G->descs.data();
-  const int n_ops = (int)G->descs.size();
+  fuse_signals(G);  // from here on the ops are G->eff: the caller's, with signal ops folded into data ops where that is possible
+  const pccl_op_desc *ops = G->eff.data();
+  const int n_ops = (int)G->eff.size();
+  auto carrier = [&](int i) { return G->fused_into[i] >= 0 ? G->fused_into[i] : i; };
   long tile_bytes = G->tile_bytes;
   const bool default_tile = tile_bytes == 0;  // parts are then sized per dependency level, below
   if (!default_tile) tile_bytes = std::max<long>(tile_bytes, 1024);
@@ -569,6 +723,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     n_edges += (size_t)o.n_deps;
     op_bytes[i] = is_signal ? 0 : o.count * es;
   }
+  // An op that carries a NOTIFY has one more place in its successor list: kSuccNotify, behind the ops
+  // (what completes the op walks that list anyway, and an op with a successor waits for its stores).
+  for (int i = 0; i < n_ops; ++i)
+    if (G->notify_of[i] >= 0) {
+      ++n_succ[i];
+      ++n_edges;
+    }
   for (int i = 0; i < n_ops; ++i)
     if (n_succ[i] > 255) return fail(PCCL_ERR_GRAPH, "op %d: %d successors exceed num_next_ops_ (unsigned char)", i, n_succ[i]);
   // copy-only graphs: the kernel instance of the first op's dtype (a chain of copies of that element
@@ -587,8 +748,12 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // of them runs is settled once the chains are known, below; the launch width must hold for both.  A
   // rebuild in place keeps the instance: launches that a stream capture has recorded carry it.)
   const DrainKernel plain_kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute, false);
-  const DrainKernel forward_kernel = mixed ? nullptr : drain_for(g_dtype, g_compute, true);
-  const int forward_elem_bytes = (G->fixed_kernel ? G->forward_capable : !mixed) ? elem_bytes(g_dtype) : 0;
+  // (the instance with the one-pass code has no registers to spare for carried signal ops: a graph with
+  // such ops runs the plain one, its chains through memory)
+  bool carries = false;
+  for (int i = 0; i < n_ops; ++i) carries = carries || G->fused_into[i] >= 0;
+  const DrainKernel forward_kernel = (mixed || carries) ? nullptr : drain_for(g_dtype, g_compute, true);
+  const int forward_elem_bytes = (G->fixed_kernel ? G->forward_capable : (!mixed && !carries)) ? elem_bytes(g_dtype) : 0;
   int occ = 8;
   for (DrainKernel k : {plain_kernel, forward_kernel}) {
     if (!k) continue;
@@ -603,7 +768,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // ---- acyclicity (Kahn) -----------------------------------------------------
   std::vector<int> succ_start(n_ops + 1, 0);
   for (int i = 0; i < n_ops; ++i) succ_start[i + 1] = succ_start[i] + n_succ[i];
-  std::vector<int> succ(n_edges ? n_edges : 1), fill(n_ops, 0);
+  std::vector<int> succ(n_edges ? n_edges : 1, kSuccNotify), fill(n_ops, 0);  // (the places no op fills are the carried NOTIFYs')
   for (int i = 0; i < n_ops; ++i)
     for (int d = 0; d < ops[i].n_deps; ++d) {
       const int u = ops[i].deps[d];
@@ -633,7 +798,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
         stack.pop_back();
         if (u == to) return true;
         for (int e = succ_start[u]; e < succ_start[u + 1]; ++e)
-          if (!seen[succ[e]]) { seen[succ[e]] = 1; stack.push_back(succ[e]); }
+          if (succ[e] >= 0 && !seen[succ[e]]) { seen[succ[e]] = 1; stack.push_back(succ[e]); }
         for (int v : order_succ[u])
           if (!seen[v]) { seen[v] = 1; stack.push_back(v); }
       }
@@ -647,9 +812,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       for (int a : it->second)
         if (ops[a].count >= ops[b].count && (best < 0 || ops[a].count < ops[best].count)) best = a;
       if (best < 0) continue;
-      if (ops[best].count != ops[b].count && reaches(b, best)) continue;
-      order_succ[best].push_back(b);
-      ++order_pred[b];
+      // (carried signal ops stand where their data ops stand)
+      const int from = carrier(best), to = carrier(b);
+      if (from == to) continue;
+      if (ops[best].count != ops[b].count && reaches(to, from)) continue;
+      if (std::find(order_succ[from].begin(), order_succ[from].end(), to) != order_succ[from].end()) continue;
+      order_succ[from].push_back(to);
+      ++order_pred[to];
     }
   }
   // level[i] = length of the longest dependency chain ending in op i
@@ -672,7 +841,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       stack.pop_back();
       G->topo.push_back(u);
       ++seen;
-      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) relax(u, succ[e]);
+      for (int e = succ_start[u]; e < succ_start[u + 1]; ++e)
+        if (succ[e] >= 0) relax(u, succ[e]);
       for (int v : order_succ[u]) relax(u, v);
     }
     if (seen != n_ops) return fail(PCCL_ERR_GRAPH, "dependency graph has a cycle (%d of %d ops reachable)", seen, n_ops);
@@ -743,7 +913,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
                        [&](int a, int b) { return last_pred_at[a] < last_pred_at[b]; });
       for (int at = lo; at < hi; ++at) {
         const int u = by_level[at];
-        for (int e = succ_start[u]; e < succ_start[u + 1]; ++e) last_pred_at[succ[e]] = std::max(last_pred_at[succ[e]], at);
+        for (int e = succ_start[u]; e < succ_start[u + 1]; ++e)
+          if (succ[e] >= 0) last_pred_at[succ[e]] = std::max(last_pred_at[succ[e]], at);
         for (int v : order_succ[u]) last_pred_at[v] = std::max(last_pred_at[v], at);
       }
       lo = hi;
@@ -767,12 +938,14 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // graphs of more than 4 Mi entries (a 256 MiB array) keep every dependency whole-op.
   G->parts = parts;
   G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
-  G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
+  G->part_edge = classify_dependencies(G->eff, parts, G->topo, &G->part_eligible);
   // ---- chains (plan_chains) ------------------------------------------------------
   G->n_succ = n_succ;
   G->order_touch.assign(n_ops, 0);
-  for (int i = 0; i < n_ops; ++i) G->order_touch[i] = order_pred[i] != 0 || !order_succ[i].empty();
-  G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, forward_elem_bytes);
+  // (an op that carries a signal op polls or stores a word around its parts: not inside a chain)
+  for (int i = 0; i < n_ops; ++i)
+    G->order_touch[i] = order_pred[i] != 0 || !order_succ[i].empty() || G->fused_into[i] >= 0 || G->wait_of[i] >= 0 || G->notify_of[i] >= 0;
+  G->chain_words = plan_chains_of(G, G->eff, parts, G->part_edge, forward_elem_bytes);
   std::vector<int> chain_prev(n_ops, -1), chain_tail(n_ops, 0);
   auto link_chains = [&] {
     std::fill(chain_prev.begin(), chain_prev.end(), -1);
@@ -854,12 +1027,12 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       }
       G->parts = parts;
       G->part_eligible.assign(n_ops, tiles <= kMaxPartWordEntries);
-      G->part_edge = classify_dependencies(G->descs, parts, G->topo, &G->part_eligible);
-      G->chain_words = plan_chains(G->descs, parts, G->part_edge, G->n_succ, G->order_touch, forward_elem_bytes);
+      G->part_edge = classify_dependencies(G->eff, parts, G->topo, &G->part_eligible);
+      G->chain_words = plan_chains_of(G, G->eff, parts, G->part_edge, forward_elem_bytes);
       link_chains();
     }
   }
-  auto queued = [&](int i) { return chain_prev[i] < 0; };  // has entries of its own
+  auto queued = [&](int i) { return chain_prev[i] < 0 && G->fused_into[i] < 0; };  // has entries of its own
   long long live_tiles = 0;
   for (int i = 0; i < n_ops; ++i)
     if (queued(i)) live_tiles += parts[i];
@@ -890,7 +1063,9 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   const size_t off_hdr = off;     off = align_up(off + sizeof(pccl_operation_layout_header) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_payload = off; off = align_up(off + kPayloadStride * (size_t)std::max(n_ops, 1), 256);
   // (the chain table follows the payloads directly: graph_rebind uploads the two as one block)
-  const size_t off_chain_table = off; off = align_up(off + sizeof(ForwardStep) * (size_t)std::max(n_ops, 1), 256);
+  const size_t off_chain_table = off; off = off + sizeof(ForwardStep) * (size_t)std::max(n_ops, 1);
+  // (... and the table of carried signals directly behind that one, for the same reason)
+  const size_t off_fuse = off;        off = align_up(off + sizeof(SignalFuse) * (size_t)std::max(n_ops, 1), 256);
   const size_t off_succ = off;    off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_succ_part = off; off = align_up(off + sizeof(int) * std::max<size_t>(n_edges, 1), 256);
   const size_t off_hot = off;     off = align_up(off + sizeof(HotWord) * kHotWords, 256);
@@ -992,6 +1167,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   C->chain = (const int *)(dev + off_chain);
   C->chain_table = (const ForwardStep *)(dev + off_chain_table);
   G->chain_table_off = off_chain_table;
+  G->fuse_table_off = off_fuse;
+  C->fuse = (const SignalFuse *)(dev + off_fuse);
   memcpy(img + off_chain, G->chain_words.data(), sizeof(int) * G->chain_words.size());
   hot[kHotCompleted].value = 0;
   hot[kHotTotal].value = (unsigned int)n_ops;
@@ -1011,7 +1188,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
           if (!queued(i)) continue;  // runs behind its chain's head
           for (int p = first; p < std::min(first + block, parts[i]); ++p, ++t)
             qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32) |
-                                      (G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 ? kEntryChainHead : 0ull));
+                                      ((G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 || G->wait_of[i] >= 0 || G->notify_of[i] >= 0) ? kEntryChainHead : 0ull) |
+                                      (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull));
         }
       lo = hi;
     }
@@ -1069,6 +1247,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
   }
   fill_chain_table(G->chain_words, n_ops, img + off_payload, (ForwardStep *)(img + off_chain_table));
+  fill_fuse_table(G, G->eff, (SignalFuse *)(img + off_fuse));
   if (n_edges) memcpy(img + off_succ, succ.data(), sizeof(int) * n_edges);
   if (n_edges) memcpy(img + off_succ_part, succ_part_base.data(), sizeof(int) * n_edges);
   // never more workgroups than entries
@@ -1324,8 +1503,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // addresses, and launches recorded by stream capture point at it); earlier runs on `stream`
   // finish first.  Only a failed upload can leave the graph unusable.
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
-  const std::vector<unsigned char> edges_after = classify_dependencies(next, G->parts, G->topo, &G->part_eligible);
-  if (edges_after != G->part_edge || plan_chains(next, G->parts, edges_after, G->n_succ, G->order_touch, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
+  const std::vector<pccl_op_desc> eff_next = effective_of(G, next);
+  const std::vector<unsigned char> edges_after = classify_dependencies(eff_next, G->parts, G->topo, &G->part_eligible);
+  if (edges_after != G->part_edge || plan_chains_of(G, eff_next, G->parts, edges_after, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
     Graph fresh;
     fresh.descs.swap(next);
@@ -1369,10 +1549,21 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->n_succ.swap(fresh.n_succ);
     G->order_touch.swap(fresh.order_touch);
     G->chain_words.swap(fresh.chain_words);
+    G->eff.swap(fresh.eff);
+    G->eff_deps.swap(fresh.eff_deps);
+    G->fused_into.swap(fresh.fused_into);
+    G->wait_of.swap(fresh.wait_of);
+    G->notify_of.swap(fresh.notify_of);
+    G->user_dep_to_eff.swap(fresh.user_dep_to_eff);
+    G->fuse_table_off = fresh.fuse_table_off;
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
   G->descs.swap(next);
+  for (size_t i = 0; i < G->eff.size(); ++i) {  // (the same ops: the dependency lists stay, the operands move)
+    memcpy(G->eff[i].ins, eff_next[i].ins, sizeof(G->eff[i].ins));
+    memcpy(G->eff[i].outs, eff_next[i].outs, sizeof(G->eff[i].outs));
+  }
   char *payloads = G->image.data() + G->payload_off;
   for (int i = 0; i < G->n_ops; ++i) {
     pccl_op_payload *pl = (pccl_op_payload *)(payloads + kPayloadStride * (size_t)i);
@@ -1382,8 +1573,9 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // ordered after earlier runs on `stream`; the source is pageable host memory,
   // so the call returns once the bytes are staged
   fill_chain_table(G->chain_words, G->n_ops, payloads, (ForwardStep *)(G->image.data() + G->chain_table_off));
+  fill_fuse_table(G, G->eff, (SignalFuse *)(G->image.data() + G->fuse_table_off));
   PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->payload_off, payloads,
-                                G->chain_table_off + sizeof(ForwardStep) * (size_t)G->n_ops - G->payload_off,
+                                G->fuse_table_off + sizeof(SignalFuse) * (size_t)G->n_ops - G->payload_off,
                                 hipMemcpyHostToDevice, (hipStream_t)stream));
   return PCCL_OK;
 }
@@ -1456,10 +1648,14 @@ int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capa
   if (!G || !n_deps) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: null argument");
   if (capacity < 0 || (capacity > 0 && !kinds)) return fail(PCCL_ERR_INVALID_ARG, "graph_dependency_kinds: bad buffer");
   std::lock_guard<std::mutex> lock(G->mu);
-  if (G->as_launches && G->part_edge.empty()) G->part_edge.assign(G->deps_store.size(), 0);  // stream order: whole-op
-  *n_deps = (long)G->part_edge.size();
+  // per dependency as the caller listed them; one that a carried signal op took part in is met by the
+  // data op's own waiting and reports whole-op; a graph run as launches: stream order, whole-op
+  *n_deps = (long)G->deps_store.size();
   const long n = std::min<long>(capacity, *n_deps);
-  if (n > 0) memcpy(kinds, G->part_edge.data(), (size_t)n);
+  for (long k = 0; k < n; ++k) {
+    const long place = (!G->as_launches && (size_t)k < G->user_dep_to_eff.size()) ? G->user_dep_to_eff[(size_t)k] : -1;
+    kinds[k] = place >= 0 ? G->part_edge[(size_t)place] : 0;
+  }
   return PCCL_OK;
 }
 

@@ -48,6 +48,7 @@ struct GraphControl {
   const int *succ_part_base;              // beside succ: entry index of part 0 of a successor released part by part
   const int *chain;                       // per op, kChainWords ints: see kChain* below
   const struct ForwardStep *chain_table;  // one row per op of every forward chain, chain after chain
+  const struct SignalFuse *fuse;          // per op: the signal ops it carries
   int *queue_head[kQueues];               // &layout.ready_queues[q]->head_
   const unsigned long long *queue_entries[kQueues];
   const int *queue_count;                 // entries on each queue, then the mode word (1: no more entries than workgroups,
@@ -80,6 +81,12 @@ constexpr int kMaxForwardSteps = 16;
 // load of its op's chain words.
 constexpr int kMaxParts = 1 << 19;
 constexpr unsigned long long kEntryChainHead = 1ull << 51;
+// ... | (every part polls a signal word first) << 52: the op carries a GET_NOTIFIED (GraphControl::fuse; such an
+// entry has the chain flag too, for the count of ops it stands for).
+constexpr unsigned long long kEntryWaitsSignal = 1ull << 52;
+constexpr unsigned long long kEntryFlags = kEntryChainHead | kEntryWaitsSignal;
+// In a successor list: not an op, but "store the signal word of the NOTIFY this op carries".
+constexpr int kSuccNotify = -1;
 
 // indices into GraphControl::hot
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
@@ -289,6 +296,15 @@ struct ForwardStep {
 };
 static_assert(sizeof(ForwardStep) == 32, "two 16-byte loads per row");
 
+// The signal ops a data op carries (graph_queue.hip, fuse_signals): values are the ops' own, the run's
+// signal base is added by the kernel.
+struct SignalFuse {
+  unsigned long long wait_word;    // 0: none
+  unsigned long long notify_word;  // 0: none
+  unsigned int wait_value, notify_value;
+};
+static_assert(sizeof(SignalFuse) == 24, "three 8-byte words per row");
+
 __device__ __forceinline__ unsigned long long uniform64(unsigned long long v) {  // the same in every lane: into scalar registers
   const unsigned int lo = __builtin_amdgcn_readfirstlane((unsigned int)v), hi = __builtin_amdgcn_readfirstlane((unsigned int)(v >> 32));
   return ((unsigned long long)hi << 32) | lo;
@@ -448,10 +464,11 @@ __device__ __forceinline__ bool bounded_wait(unsigned int *abort_flag, unsigned 
 // function has to wait for (the two then travel together), or, when nothing is counted
 // (single-part op), after the successors have been told, so that their release is not held up
 // behind the ticket (memory operations of a wavefront return in order).
-template <class DrawTicket>
+// `notify` stores the signal word of the NOTIFY the op carries (a successor list can end in kSuccNotify).
+template <class DrawTicket, class Notify>
 __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operation_layout_header *h,
                                             const OpFacts &op, int uid, int part, unsigned int *done_ops, int chain_ops,
-                                            DrawTicket draw_ticket) {
+                                            DrawTicket draw_ticket, Notify notify) {
   const int parts = op.parts;
   // successors that need only this part of the op (they come first in the successor list):
   // part `part` of each is told right away
@@ -494,8 +511,11 @@ __device__ __forceinline__ void finish_part(const GraphControl &g, pccl_operatio
     __hip_atomic_store(&g.ready[uid].value, 0u, __ATOMIC_RELAXED, AGENT);
   const int n_next = op.num_next_ops();
   const int *next = g.succ + op.succ_start;
-  for (int s = n_part_next; s < n_next; ++s)
-    __hip_atomic_fetch_add(&g.ready[next[s]].value, 1u, __ATOMIC_RELAXED, AGENT);
+  for (int s = n_part_next; s < n_next; ++s) {
+    const int to = next[s];
+    if (to == kSuccNotify) notify(uid);  // (every part waited for its stores: the op has a successor)
+    else __hip_atomic_fetch_add(&g.ready[to].value, 1u, __ATOMIC_RELAXED, AGENT);
+  }
   // (an op that heads a chain stands for all the chain's ops: they ran behind it, part by part)
   *done_ops += (unsigned int)chain_ops;  // (the workgroup reports its count when it leaves)
   if (!drawn) draw_ticket();
@@ -609,9 +629,23 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         if (first_q >= 0) first_t = __hip_atomic_fetch_add(g.queue_head[first_q], 1, __ATOMIC_RELAXED, AGENT);
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       };
+      auto base_of_run = [&] {
+        if (!have_signal_base) {
+          signal_base = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT) << 16;
+          have_signal_base = true;
+        }
+        return signal_base;
+      };
+      // (graphs whose data ops carry signal ops run the plain instance: this one has no registers to spare)
+      auto notify = [&](int uid) {
+        if constexpr (!FORWARD) {
+          const SignalFuse *f = &g.fuse[uid];
+          __hip_atomic_store((unsigned int *)f->notify_word, base_of_run() + f->notify_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+      };
       if (h) {
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, h, cur_op, cur_uid, cur_part, &s_done, cur_chain_ops, draw_ticket);
+        finish_part(g, h, cur_op, cur_uid, cur_part, &s_done, cur_chain_ops, draw_ticket, notify);
       } else {
         draw_ticket();
       }
@@ -650,7 +684,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
             go = 1;
             if (g.trace) {
               cur_trace = g.trace + entry_index * kTraceWords;
-              cur_trace[kTraceWhat] = (e & ~kEntryChainHead) | ((unsigned long long)blockIdx.x << 52);
+              cur_trace[kTraceWhat] = (e & ~kEntryFlags) | ((unsigned long long)blockIdx.x << 52);
               cur_trace[kTraceClaimed] = wall_clock64();
             }
             if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
@@ -669,7 +703,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         // that word's only reader and clears it for the next run.
         const unsigned int w12 = *word12(hc);
         const unsigned int arrived = __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT);
-        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + ((size_t)(g.entry_base[uid] + (int)((e & ~kEntryChainHead) >> 32)) << g.part_shift) : nullptr;
+        unsigned int *part_word = g.part_arrivals ? g.part_arrivals + ((size_t)(g.entry_base[uid] + (int)((e & ~kEntryFlags) >> 32)) << g.part_shift) : nullptr;
         const unsigned int part_arrived = part_word ? __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) : 0u;
         const int prim = sc->payload.primitive_;
         const unsigned int part_preds = sc->payload.part_preds_;
@@ -698,14 +732,23 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           }
           __hip_atomic_store(part_word, 0u, __ATOMIC_RELAXED, AGENT);
         }
+        // the GET_NOTIFIED the op carries: every part polls the word before it starts
+        if (!FORWARD && (e & kEntryWaitsSignal)) {
+          const SignalFuse *f = &g.fuse[uid];
+          unsigned int *word = (unsigned int *)f->wait_word;
+          const unsigned int want = base_of_run() + f->wait_value;
+          if ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) < 0 &&
+              !bounded_wait(abort_flag, spin_limit, [&] {
+                return (int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
+              })) {
+            go = 0;
+            break;
+          }
+        }
         if (cur_trace) cur_trace[kTraceReady] = wall_clock64();
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
-        if (!have_signal_base) {
-          signal_base = __hip_atomic_load(&hot[kHotRun].value, __ATOMIC_RELAXED, AGENT) << 16;
-          have_signal_base = true;
-        }
-        const unsigned int want = signal_base + (unsigned int)sc->payload.chunks_[0].num_elems_;
+        const unsigned int want = base_of_run() + (unsigned int)sc->payload.chunks_[0].num_elems_;
         if (prim == PCCL_NOTIFY) {
           // everything this op depends on is already at the point of coherence
           __hip_atomic_store(sig, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -716,7 +759,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, hc, OpFacts::of(sc), uid, 0, &s_done, 1, [] {});
+        finish_part(g, hc, OpFacts::of(sc), uid, 0, &s_done, 1, [] {}, notify);
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
@@ -728,7 +771,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
     __syncthreads();
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
     const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
-    const int part = __builtin_amdgcn_readfirstlane((int)((s_entry & ~kEntryChainHead) >> 32));
+    const int part = __builtin_amdgcn_readfirstlane((int)((s_entry & ~kEntryFlags) >> 32));
     cur_uid = uid;
     cur_part = part;
     h = &g.headers[uid];

@@ -66,6 +66,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAINS");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_OWN_ENTRIES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAIN_BALANCE");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_FUSE_SIGNALS");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;

@@ -869,3 +869,117 @@ def test_get_notified_is_released_by_a_notify_of_a_larger_value(hip, oracle):
     H.assert_bits_equal(dt.download(), a, "copy released from outside")
     assert int(sig[1].item()) == base + 5
     g.destroy()
+
+
+# ---- signal ops carried by data ops -----------------------------------------------------------
+
+def _signal_ring_run(torch, hip, oracle, world, size, tile):
+    per = world * size
+    d_in = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    d_out = [H.DevBuf(torch, "bf16", per, 0) for _ in range(world)]
+    signals = torch.zeros(64, dtype=torch.int32, device="cuda")
+    ops, sym = _signal_ring_ops(world, size, signals.data_ptr(), d_in, d_out)
+    g = hip.Graph(ops, tile_bytes=tile)
+    ins = [H.gen("bf16", per, 930, r) for r in range(world)]
+    outs = [np.zeros(per, dtype=np.uint16) for _ in range(world)]
+    bufs = {"in": ins, "out": outs}
+    for i in sorted(sym):
+        o = sym[i]
+        oracle.reduce_copy("bf16", "sum", [bufs[b][r][e:e + size] for (b, r, e) in o["ins"]],
+                           [bufs[b][r][e:e + size] for (b, r, e) in o["outs"]])
+    for it in range(2):
+        for r in range(world):
+            d_in[r].upload(ins[r])
+            d_out[r].view().fill_(0xFF)
+        base = g.next_signal_base()
+        g.run(_stream(torch))
+        assert g.status(_stream(torch)) == (len(ops), len(ops))
+        for r in range(world):
+            H.assert_bits_equal(d_out[r].download(), outs[r], "run %d rank %d" % (it, r))
+        assert signals[:world].cpu().tolist() == [base + 2 * world - 2] * world
+    info = g.info()
+    g.destroy()
+    return info["n_tiles"], len(ops), len(sym)
+
+
+def test_signal_ops_are_carried_by_their_data_ops(hip, oracle, monkeypatch):
+    """A ring whose ranks are linked by signal words only: every GET_NOTIFIED is polled by the parts of
+    the one data op behind it and every NOTIFY is stored by whoever completes the one data op in front
+    of it, so only the data ops queue entries; every op still counts as complete, the signal words end
+    at the run's last value, the results are the checker's.  Switched off, every signal op queues an
+    entry of its own and the results are the same."""
+    import torch
+    world, size = 8, 3001
+    entries, n_ops, n_data = _signal_ring_run(torch, hip, oracle, world, size, 4096)
+    parts = -(-size * 2 // 4096)
+    assert entries == n_data * parts, "only the data ops queue entries"
+    monkeypatch.setenv("PCCL_HIP_FUSE_SIGNALS", "0")
+    entries_off, _, _ = _signal_ring_run(torch, hip, oracle, world, size, 4096)
+    assert entries_off == n_data * parts + (n_ops - n_data)
+
+
+def test_signal_ops_that_stay_ops_of_their_own(hip, oracle):
+    """Shapes in which a signal op cannot ride on a data op: a NOTIFY behind two ops, a GET_NOTIFIED that two
+    ops wait for, a second NOTIFY behind the same op (the first is carried), a NOTIFY behind a GET_NOTIFIED,
+    a GET_NOTIFIED in front of a NOTIFY.  All of them still do what they say."""
+    import torch
+    n = 50_001
+    a, b = H.gen("f32", n, 940, 0), H.gen("f32", n, 940, 1)
+    da, db = H.DevBuf(torch, "f32", n, 0, src=a), H.DevBuf(torch, "f32", n, 0, src=b)
+    dt, du, dv, dw = (H.DevBuf(torch, "f32", n, 0) for _ in range(4))
+    sig = torch.zeros(16, dtype=torch.int32, device="cuda")
+    word = lambda k: sig.data_ptr() + 4 * k
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=n, deps=[]),      # 0
+           dict(dtype="f32", compute="max", ins=[da.ptr, db.ptr], outs=[du.ptr], count=n, deps=[]),      # 1
+           dict(primitive=2, signal=word(0), value=3, deps=[0, 1]),                                      # 2: two predecessors
+           dict(primitive=2, signal=word(1), value=4, deps=[0]),                                         # 3: carried by op 0
+           dict(primitive=2, signal=word(2), value=5, deps=[0]),                                         # 4: op 0 carries one already
+           dict(primitive=3, signal=word(0), value=3, deps=[]),                                          # 5: two ops wait for it
+           dict(dtype="f32", compute="sum", ins=[dt.ptr], outs=[dv.ptr], count=n, deps=[5]),             # 6
+           dict(dtype="f32", compute="sum", ins=[du.ptr], outs=[dw.ptr], count=n, deps=[5]),             # 7
+           dict(primitive=3, signal=word(2), value=5, deps=[]),                                          # 8: followed by a NOTIFY
+           dict(primitive=2, signal=word(3), value=6, deps=[8])]                                         # 9: behind a GET_NOTIFIED
+    g = hip.Graph(ops, tile_bytes=32768)
+    parts = -(-n * 4 // 32768)
+    assert g.info()["n_tiles"] == 4 * parts + 5, "ops 2, 4, 5, 8 and 9 keep their entries; op 3 rides on op 0"
+    for it in range(3):
+        for buf in (dt, du, dv, dw):
+            buf.view().fill_(0xFF)
+        base = g.next_signal_base()
+        torch.cuda.synchronize()
+        g.run(_stream(torch))
+        assert g.status(_stream(torch)) == (len(ops), len(ops))
+        H.assert_bits_equal(dv.download(), oracle.reduce("f32", "sum", [a, b]), "v, run %d" % it)
+        H.assert_bits_equal(dw.download(), oracle.reduce("f32", "max", [a, b]), "w, run %d" % it)
+        assert sig[:4].cpu().tolist() == [base + 3, base + 4, base + 5, base + 6]
+    g.destroy()
+
+
+def test_carried_signal_words_move_with_a_rebind(hip, oracle):
+    """The words of carried signal ops are operands like any other: a rebind of the range that holds them
+    moves the word a data op polls and the word it stores."""
+    import torch
+    n = 20_000
+    a = H.gen("f32", n, 950, 0)
+    da, dt = H.DevBuf(torch, "f32", n, 0, src=a), H.DevBuf(torch, "f32", n, 0)
+    sig1 = torch.zeros(16, dtype=torch.int32, device="cuda")
+    sig2 = torch.zeros(16, dtype=torch.int32, device="cuda")
+    ops = [dict(primitive=3, signal=sig1.data_ptr(), value=2, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[da.ptr], outs=[dt.ptr], count=n, deps=[0]),
+           dict(primitive=2, signal=sig1.data_ptr() + 4, value=9, deps=[1])]
+    g = hip.Graph(ops)
+    assert g.info()["n_tiles"] == g.info()["n_workgroups"], "one entry per part of the copy, none for the signal ops"
+    stream = _stream(torch)
+    for sig in (sig1, sig2):
+        if sig is sig2:
+            g.rebind(sig1.data_ptr(), sig2.data_ptr(), 64, stream)
+        base = g.next_signal_base()
+        sig[0] = base + 2
+        dt.view().fill_(0xFF)
+        torch.cuda.synchronize()
+        g.run(stream)
+        assert g.status(stream) == (3, 3)
+        H.assert_bits_equal(dt.download(), a, "copy released through the word")
+        assert int(sig[1].item()) == base + 9
+    assert int(sig1[1].item()) != int(sig2[1].item())
+    g.destroy()
