@@ -539,6 +539,25 @@ def main():
                                                               queue_entries=g.info()["n_tiles"],
                                                               dependencies_part_by_part="%d of %d" % (sum(kinds), len(kinds)))
                 g.destroy()
+                # The same all-reduce written the way ranks on different devices write it: dependency
+                # edges inside a rank only, the hand-over between neighbours NOTIFY -> signal word ->
+                # GET_NOTIFIED (328 ops).  Nothing can stay in registers across such a hand-over.
+                if per_rank_mib <= 8:
+                    irs, _ = lang.ring_allreduce_signalled(8, (per_rank_mib << 20) // 2 // 8, dtype="bf16")
+                    lows = irs.lower()
+                    words = torch.zeros(64, dtype=torch.int32, device="cuda")
+                    first = rb["out"][0].clone()
+                    for r in range(8):
+                        rb["out"][r].zero_()
+                    gs = hip.Graph(lang.bind(lows, lambda b, r, e: rb[b][r].data_ptr() + 2 * e, signals=words.data_ptr()))
+                    ts = event_times_us(torch, lambda: gs.run(stream), 20, 3)
+                    done, total = gs.status(stream)
+                    assert done == total == len(lows)
+                    for r in range(8):
+                        assert torch.equal(rb["out"][r], first), "the ring linked by signal words differs from the ring linked by dependencies"
+                    full["8_ranks_x_%d_MiB" % per_rank_mib]["linked_by_signal_words_only"] = dict(
+                        stats(ts), ops=len(lows), queue_entries=gs.info()["n_tiles"])
+                    gs.destroy()
                 del rb
             full["note"] = ("GBps_median counts the algorithmic bytes of the 112 ops; the 14 ops of a chunk run as one chain that keeps "
                             "the value in registers and stores only what the chain does not overwrite itself: bytes_moved / GBps_moved_median")
