@@ -280,6 +280,12 @@ int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int
  * executor's operand table.  Touches no device. */
 int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, int forward_elem_bytes, int *words);
 
+/* Which signal ops of a graph ride on data ops (no counterpart in the reference; touches no device):
+ * carrier[i] = the COPY / REDUCE op that stores NOTIFY i when it completes, or whose parts poll
+ * GET_NOTIFIED i before they start; -1 for every other op.  The rule is stated at
+ * pccl_hip_graph_create; it looks at kinds and dependency lists only. */
+int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier);
+
 /* Device address of the GraphBufferLayout and launch facts, for inspection: n_tiles = queue entries
  * (parts of the ops that queue entries; ops that run behind another op in a chain queue none), or the
  * number of launches for a graph that runs as plain launches; n_workgroups = width of the launch. */

@@ -1642,6 +1642,23 @@ int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, i
   return PCCL_OK;
 }
 
+int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier) {
+  pccl_host::clear_error();
+  if (n_ops < 0 || (n_ops > 0 && (!ops || !carrier))) return fail(PCCL_ERR_INVALID_ARG, "plan_signals: bad arguments");
+  for (int i = 0; i < n_ops; ++i) {
+    const pccl_op_desc &o = ops[i];
+    if (o.primitive > PCCL_GET_NOTIFIED) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown primitive code %d", i, o.primitive);
+    if (o.n_deps < 0 || (o.n_deps > 0 && !o.deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
+    for (int d = 0; d < o.n_deps; ++d)
+      if (o.deps[d] < 0 || o.deps[d] >= n_ops || o.deps[d] == i) return fail(PCCL_ERR_GRAPH, "op %d: dependency %d is not another op", i, o.deps[d]);
+  }
+  Graph G;
+  G.descs.assign(ops, ops + n_ops);
+  fuse_signals(&G);
+  for (int i = 0; i < n_ops; ++i) carrier[i] = G.fused_into[i];
+  return PCCL_OK;
+}
+
 int pccl_hip_graph_dependency_kinds(void *graph, unsigned char *kinds, long capacity, long *n_deps) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;

@@ -88,6 +88,7 @@ def lib():
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.pccl_hip_classify_dependencies.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), vp]
         L.pccl_hip_plan_chains.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ci, ctypes.POINTER(ci)]
+        L.pccl_hip_plan_signals.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci)]
         L.pccl_hip_graph_dependency_kinds.argtypes = [vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_trace.argtypes = [vp, ci]
         L.pccl_hip_graph_read_trace.argtypes = [vp, vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
@@ -264,6 +265,15 @@ def plan_chains(ops, parts, forward_elem_bytes):
     words = (ctypes.c_int * max(4 * len(ops), 1))()
     _check(lib().pccl_hip_plan_chains(arr, len(ops), pa, forward_elem_bytes, words))
     return [tuple(words[4 * i:4 * i + 4]) for i in range(len(ops))]
+
+
+def plan_signals(ops):
+    """Which signal ops ride on data ops (host only): per op the index of the COPY / REDUCE that carries
+    it, or -1."""
+    arr, keep = _op_descs(ops)
+    carrier = (ctypes.c_int * max(len(ops), 1))()
+    _check(lib().pccl_hip_plan_signals(arr, len(ops), carrier))
+    return list(carrier[:len(ops)])
 
 
 STATIC_ARENA_BYTES = 8 << 20

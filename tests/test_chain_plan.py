@@ -141,3 +141,54 @@ def test_bad_arguments_are_refused():
         hip.plan_chains([op([a, b], [t], [5])], [1], ES)      # dependency on an op that does not exist
     with pytest.raises(hip.PcclError):
         hip.plan_chains([op([a, b], [t], [])], [0], ES)       # no parts
+
+
+# ---- which signal ops ride on data ops (pccl_hip_plan_signals, host only) --------------------
+
+def notify(word, value, deps):
+    return dict(primitive=2, signal=word, value=value, deps=list(deps))
+
+
+def get_notified(word, value, deps):
+    return dict(primitive=3, signal=word, value=value, deps=list(deps))
+
+
+def test_a_ring_step_carries_its_wait_and_its_notify():
+    a, b, t, u = (buf(k) for k in range(4))
+    sig = 0x900000
+    # rank-style sequence: GET -> data -> NOTIFY -> GET -> data -> NOTIFY
+    ops = [get_notified(sig, 1, []), op([a, b], [t], [0]), notify(sig + 4, 1, [1]),
+           get_notified(sig, 2, [2]), op([t], [u], [3]), notify(sig + 4, 2, [4])]
+    assert hip.plan_signals(ops) == [1, -1, 1, 4, -1, 4]
+    # the plan looks at kinds and dependency lists only: other addresses, same plan
+    moved = [dict(o) for o in ops]
+    moved[1] = op([b, a], [u], [0])
+    assert hip.plan_signals(moved) == [1, -1, 1, 4, -1, 4]
+
+
+def test_signal_ops_that_stay_ops_of_their_own():
+    a, b, t, u, v, w = (buf(k) for k in range(6))
+    sig = 0x900000
+    ops = [op([a, b], [t], []),                 # 0
+           op([a, b], [u], []),                 # 1
+           notify(sig, 3, [0, 1]),              # 2: behind two ops
+           notify(sig + 4, 4, [0]),             # 3: rides on op 0
+           notify(sig + 8, 5, [0]),             # 4: op 0 carries one already
+           get_notified(sig, 3, []),            # 5: two ops wait for it
+           op([t], [v], [5]),                   # 6
+           op([u], [w], [5]),                   # 7
+           get_notified(sig + 8, 5, []),        # 8: in front of a NOTIFY, not of a data op
+           notify(sig + 12, 6, [8]),            # 9: behind a GET_NOTIFIED, not a data op
+           get_notified(sig + 12, 6, [])]       # 10: nothing waits for it
+    assert hip.plan_signals(ops) == [-1, -1, -1, 0, -1, -1, -1, -1, -1, -1, -1]
+    # one data op can carry a wait and a notify at once, but not two waits
+    ops = [get_notified(sig, 1, []), get_notified(sig + 4, 1, []), op([a], [t], [0, 1]), notify(sig + 8, 1, [2])]
+    assert hip.plan_signals(ops) == [2, -1, -1, 2]
+
+
+def test_plan_signals_refuses_bad_lists():
+    a, t = buf(0), buf(1)
+    with pytest.raises(hip.PcclError) as e:
+        hip.plan_signals([op([a], [t], [3])])
+    assert e.value.code == hip.ERR_GRAPH
+    assert hip.plan_signals([]) == []
