@@ -190,3 +190,50 @@ def test_random_programs_over_one_pool_match_sequential_execution(hip, oracle):
         g.destroy()
     # the sweep met both kinds of dependency often
     assert min(kinds_seen) >= 20, kinds_seen
+
+
+def test_random_programs_with_dependencies_replaced_by_signal_words(hip, oracle):
+    """The same kind of program with about half of its dependency edges u -> v replaced by
+    NOTIFY(behind u) -> signal word -> GET_NOTIFIED(in front of v), a word per replaced edge: some of
+    those signal ops ride on their data op, some (a second NOTIFY behind the same op, a second wait in
+    front of it) queue entries of their own.  The pool must equal sequential execution, run after run."""
+    import torch
+    pool_elems = 1_000_000
+    stream = torch.cuda.current_stream().cuda_stream
+    carried_seen, own_seen = 0, 0
+    for seed in range(5 * SCALE):
+        rng = np.random.default_rng(8000 + seed + SEED_SHIFT)
+        prog = S.random_pool_program(rng, pool_elems, int(rng.integers(6, 40)))
+        host = H.gen("f32", pool_elems, 977 + seed, 0, kind="uniform", lo=-1.0, hi=1.0)
+        dev = H.DevBuf(torch, "f32", pool_elems, 0, src=host)
+        words = torch.zeros(1024, dtype=torch.int32, device="cuda")
+        ops, new_index, n_words = [], {}, 0
+        for i, o in enumerate(prog):
+            deps = []
+            for u in o["deps"]:
+                if rng.random() < 0.5 and n_words < 1000:
+                    word = words.data_ptr() + 4 * n_words
+                    n_words += 1
+                    ops.append(dict(primitive=2, signal=word, value=1, deps=[new_index[u]]))
+                    ops.append(dict(primitive=3, signal=word, value=1, deps=[]))
+                    deps.append(len(ops) - 1)
+                else:
+                    deps.append(new_index[u])
+            new_index[i] = len(ops)
+            ops.append(dict(dtype="f32", compute=o["compute"], count=o["count"], deps=deps,
+                            ins=[dev.ptr + 4 * r for r in o["ins"]], outs=[dev.ptr + 4 * r for r in o["outs"]]))
+        carrier = hip.plan_signals(ops)
+        carried_seen += sum(1 for c in carrier if c >= 0)
+        own_seen += sum(1 for k, c in enumerate(carrier) if c < 0 and ops[k].get("primitive", 0) >= 2)
+        g = hip.Graph(ops, tile_bytes=[0, 16384, 65536][seed % 3])
+        for run in range(3):
+            for o in prog:
+                n = o["count"]
+                oracle.reduce_copy("f32", o["compute"], [host[r:r + n].copy() for r in o["ins"]], [host[r:r + n] for r in o["outs"]])
+            g.run(stream)
+            done, total = g.status(stream)
+            assert done == total == len(ops)
+            H.assert_bits_equal(dev.download(), host, "seed %d run %d (%d ops, %d words)" % (seed, run, len(ops), n_words))
+        assert dev.guards_intact()
+        g.destroy()
+    assert carried_seen >= 20 and own_seen >= 20, (carried_seen, own_seen)
