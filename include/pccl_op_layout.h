@@ -103,7 +103,10 @@ typedef struct pccl_op_payload {
  * start as soon as A's part p is complete (and all of B's other dependencies are), which is
  * what lets a chain of large ops stream instead of draining between ops.  The same must hold
  * for every op still possibly in flight behind A through such edges; otherwise the
- * dependency stays whole-op.  The observable result is that of whole-op dependencies. */
+ * dependency stays whole-op.  (A and B sharing no bytes at all, a dependency that only orders
+ * them, counts as "every overlap lines up".)  The observable result is that of whole-op
+ * dependencies: memory ends as if the ops had run one after the other, B is complete only
+ * after A is, and so is every NOTIFY behind B. */
 
 /* Ready-queue entry: which op, which of its required_executors_ parts. */
 typedef struct pccl_queue_entry {

@@ -137,9 +137,13 @@ struct Graph {
 // number of parts, same bytes per part and in all) and every pair of operands through which
 // they conflict (A writes what B reads or writes, or A reads what B writes) starts at the
 // same address: then part p of either op touches the same bytes of that pair.  A pair that
-// overlaps at different addresses makes some other part of A matter, and no conflicting pair
-// at all means that the dependency orders something this code cannot see; both keep the
-// dependency whole-op.
+// overlaps at different addresses makes some other part of A matter and keeps the dependency
+// whole-op.  No conflicting pair at all (the caller orders two ops that share no bytes) is met
+// part by part as well: what a dependency promises here is that B is complete only after A is,
+// and that everything B's parts touch is as A and A's own predecessors left it; both hold
+// (every part of B waits for a part of A, and the rule below looks at what can still be in
+// flight behind A), and who reads a NOTIFY behind B still knows A complete.  PCCL_HIP_ORDER_EDGES=0
+// keeps such dependencies whole-op.
 enum Conflict { kNoConflict, kSameAddress, kOtherAddress };
 constexpr long long kMaxPartWordEntries = 1ll << 22;
 
@@ -192,6 +196,8 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
   std::vector<unsigned char> flags(dep_start[n_ops], 0);
   if (const char *env = getenv("PCCL_HIP_PART_DEPS"))
     if (env[0] == '0') return flags;  // every dependency whole-op
+  bool order_edges_by_part = true;
+  if (const char *env = getenv("PCCL_HIP_ORDER_EDGES")) order_edges_by_part = env[0] != '0';
   std::vector<std::vector<int>> behind(n_ops);
   auto is_data = [&](const pccl_op_desc &o) { return o.primitive != PCCL_NOTIFY && o.primitive != PCCL_GET_NOTIFIED; };
   auto bytes_of = [&](const pccl_op_desc &o) { return (uintptr_t)o.count * (uintptr_t)elem_bytes(o.dtype); };
@@ -206,7 +212,8 @@ std::vector<unsigned char> classify_dependencies(const std::vector<pccl_op_desc>
       if (!is_data(A) || parts[a] != parts[b] || bytes_of(A) != bytes ||
           (uintptr_t)part_elems(A.count, parts[a]) * (uintptr_t)elem_bytes(A.dtype) != per)
         continue;
-      if (conflict_of(A, B, bytes) != kSameAddress) continue;
+      const Conflict how = conflict_of(A, B, bytes);
+      if (how == kOtherAddress || (how == kNoConflict && !order_edges_by_part)) continue;
       bool ok = behind[a].size() + behind[b].size() + 1 <= kMaxBehind;
       for (size_t k = 0; ok && k < behind[a].size(); ++k)
         ok = conflict_of(ops[behind[a][k]], B, bytes) != kOtherAddress;

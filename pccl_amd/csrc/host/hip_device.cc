@@ -67,6 +67,7 @@ struct HipPluginRegistration {
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_OWN_ENTRIES");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_CHAIN_BALANCE");
     utils::LaunchEnvironments::registerOpt("PCCL_HIP_FUSE_SIGNALS");
+    utils::LaunchEnvironments::registerOpt("PCCL_HIP_ORDER_EDGES");
   }
 };
 static HipPluginRegistration g_hip_plugin_registration;
