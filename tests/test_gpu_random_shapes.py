@@ -237,3 +237,40 @@ def test_random_programs_with_dependencies_replaced_by_signal_words(hip, oracle)
         assert dev.guards_intact()
         g.destroy()
     assert carried_seen >= 20 and own_seen >= 5, (carried_seen, own_seen)
+
+
+def test_random_programs_with_dependencies_between_ops_that_share_no_bytes(hip, oracle):
+    """The same kind of program with extra dependencies that it does not need (to any earlier op): those
+    between ops cut alike are met part by part, and the ops reached through them must still be looked at
+    when a later op touches their bytes at another address.  The pool must equal sequential execution."""
+    import torch
+    pool_elems = 1_500_000
+    stream = torch.cuda.current_stream().cuda_stream
+    extra, part_wise = 0, 0
+    for seed in range(6 * SCALE):
+        rng = np.random.default_rng(6100 + seed + SEED_SHIFT)
+        prog = S.random_pool_program(rng, pool_elems, int(rng.integers(8, 50)))
+        for i, o in enumerate(prog):
+            for _ in range(2):
+                if i and rng.random() < 0.4:
+                    j = int(rng.integers(0, i))
+                    if j not in o["deps"]:
+                        o["deps"].append(j)
+                        extra += 1
+        host = H.gen("f32", pool_elems, 877 + seed, 0, kind="uniform", lo=-1.0, hi=1.0)
+        dev = H.DevBuf(torch, "f32", pool_elems, 0, src=host)
+        g = hip.Graph([dict(dtype="f32", compute=o["compute"], count=o["count"], deps=o["deps"],
+                            ins=[dev.ptr + 4 * r for r in o["ins"]], outs=[dev.ptr + 4 * r for r in o["outs"]])
+                       for o in prog], tile_bytes=[0, 16384, 65536][seed % 3])
+        part_wise += g.dependency_kinds().count(1)
+        for run in range(2):
+            for o in prog:
+                n = o["count"]
+                oracle.reduce_copy("f32", o["compute"], [host[r:r + n].copy() for r in o["ins"]], [host[r:r + n] for r in o["outs"]])
+            g.run(stream)
+            done, total = g.status(stream)
+            assert done == total == len(prog)
+            H.assert_bits_equal(dev.download(), host, "seed %d run %d (%d ops)" % (seed, run, len(prog)))
+        assert dev.guards_intact()
+        g.destroy()
+    assert extra >= 50 and part_wise >= 20, (extra, part_wise)
