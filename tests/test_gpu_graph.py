@@ -983,3 +983,47 @@ def test_carried_signal_words_move_with_a_rebind(hip, oracle):
         assert int(sig[1].item()) == base + 9
     assert int(sig1[1].item()) != int(sig2[1].item())
     g.destroy()
+
+
+@pytest.mark.parametrize("tile_bytes", [4096, 0])
+def test_ops_without_elements_still_order_and_signal(hip, oracle, tile_bytes):
+    """An op of zero elements moves nothing but is an op like any other: it completes behind its
+    dependencies, releases what depends on it, may stand in a chain, and carries a GET_NOTIFIED and a
+    NOTIFY (null operands are allowed for it)."""
+    import torch
+    n = 30_011
+    a, b = H.gen("f32", n, 960, 0), H.gen("f32", n, 960, 1)
+    da, db = H.DevBuf(torch, "f32", n, 0, src=a), H.DevBuf(torch, "f32", n, 0, src=b)
+    dt, du, dv = (H.DevBuf(torch, "f32", n, 0) for _ in range(3))
+    sig = torch.zeros(16, dtype=torch.int32, device="cuda")
+    word = lambda k: sig.data_ptr() + 4 * k
+    ops = [dict(dtype="f32", compute="sum", ins=[da.ptr, db.ptr], outs=[dt.ptr], count=n, deps=[]),      # 0
+           dict(dtype="f32", compute="sum", ins=[dt.ptr, da.ptr], outs=[du.ptr], count=0, deps=[0]),     # 1: empty, between two ops
+           dict(dtype="f32", compute="sum", ins=[dt.ptr, db.ptr], outs=[du.ptr], count=n, deps=[1]),     # 2
+           dict(primitive=2, signal=word(0), value=7, deps=[2]),                                         # 3: rides on op 2
+           dict(primitive=3, signal=word(0), value=7, deps=[]),                                          # 4: rides on op 5
+           dict(dtype="f32", compute="sum", ins=[0], outs=[0], count=0, deps=[4]),                       # 5: empty carrier, null operands
+           dict(primitive=2, signal=word(1), value=8, deps=[5]),                                         # 6: rides on op 5
+           dict(primitive=3, signal=word(1), value=8, deps=[]),                                          # 7: rides on op 8
+           dict(dtype="f32", compute="max", ins=[du.ptr, da.ptr], outs=[dv.ptr], count=n, deps=[7])]     # 8
+    assert hip.plan_signals(ops) == [-1, -1, -1, 2, 5, -1, 5, 8, -1]
+    g = hip.Graph(ops, tile_bytes=tile_bytes)
+    t = oracle.reduce("f32", "sum", [a, b])
+    u = oracle.reduce("f32", "sum", [t, b])
+    for it in range(2):
+        for buf in (dt, du, dv):
+            buf.view().fill_(0xFF)
+        base = g.next_signal_base()
+        torch.cuda.synchronize()
+        g.run(_stream(torch))
+        assert g.status(_stream(torch)) == (len(ops), len(ops))
+        H.assert_bits_equal(du.download(), u, "u, run %d" % it)
+        H.assert_bits_equal(dv.download(), oracle.reduce("f32", "max", [u, a]), "v, run %d" % it)
+        assert sig[:2].cpu().tolist() == [base + 7, base + 8]
+    g.destroy()
+    # a graph of empty ops alone
+    g = hip.Graph([dict(dtype="bf16", compute="sum", ins=[0, 0], outs=[0], count=0, deps=[]),
+                   dict(dtype="bf16", compute="sum", ins=[0], outs=[0], count=0, deps=[0])], tile_bytes=tile_bytes)
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (2, 2)
+    g.destroy()
