@@ -192,3 +192,60 @@ def test_plan_signals_refuses_bad_lists():
         hip.plan_signals([op([a], [t], [3])])
     assert e.value.code == hip.ERR_GRAPH
     assert hip.plan_signals([]) == []
+
+
+def _model_plan_signals(ops):
+    """The documented rule, restated: NOTIFYs first, in op order (one data op behind it alone, which
+    carries none yet); what depended on a carried NOTIFY then depends on its data op; then
+    GET_NOTIFIEDs in op order (one data op alone depends on it, which carries no wait yet)."""
+    n = len(ops)
+    kind = [o.get("primitive", 0) for o in ops]
+    deps = [list(o["deps"]) for o in ops]
+    data = lambda i: kind[i] < 2
+    carrier = [-1] * n
+    has_notify, has_wait = set(), set()
+    stands_for = list(range(n))
+    for v in range(n):
+        if kind[v] == 2 and len(deps[v]) == 1 and data(deps[v][0]) and deps[v][0] not in has_notify:
+            a = deps[v][0]
+            has_notify.add(a)
+            carrier[v] = a
+            stands_for[v] = a
+            deps[v] = []
+    deps = [sorted(set(stands_for[d] for d in ds)) for ds in deps]
+    succ = [[] for _ in range(n)]
+    for i in range(n):
+        for d in deps[i]:
+            succ[d].append(i)
+    for v in range(n):
+        if kind[v] == 3 and len(succ[v]) == 1 and data(succ[v][0]) and succ[v][0] not in has_wait:
+            b = succ[v][0]
+            has_wait.add(b)
+            carrier[v] = b
+    return carrier
+
+
+def test_plan_signals_follows_the_documented_rule_on_random_programs():
+    import random
+    rng = random.Random(31)
+    carried = 0
+    for case in range(400):
+        n = rng.randint(1, 24)
+        ops = []
+        for i in range(n):
+            k = min(i, rng.choice([0, 1, 1, 1, 2, 3]))
+            deps = rng.sample(range(i), k)
+            r = rng.random()
+            if r < 0.5:
+                ops.append(op([buf(2 * i)], [buf(2 * i + 1)], deps))
+            elif r < 0.75:
+                ops.append(notify(0x900000 + 4 * rng.randint(0, 5), rng.randint(1, 9), deps))
+            else:
+                ops.append(get_notified(0x900000 + 4 * rng.randint(0, 5), rng.randint(1, 9), deps))
+        got = hip.plan_signals(ops)
+        assert got == _model_plan_signals(ops), "case %d: %r" % (case, ops)
+        carried += sum(1 for c in got if c >= 0)
+        for v, c in enumerate(got):
+            if c >= 0:
+                assert ops[v].get("primitive", 0) >= 2 and ops[c].get("primitive", 0) < 2
+    assert carried > 300
