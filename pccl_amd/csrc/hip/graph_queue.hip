@@ -176,10 +176,11 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // same dependency level takes its turn (PCCL_HIP_ORDER_BLOCK; 0 = all of them, i.e. op after
 // op).  With op after op the workgroups in flight cover two or three large ops at a time; in
 // blocks they work on every op of the level at once, each through a narrow window.  Measured on
-// 14 independent 32 MiB ring steps (7 reductions 2 -> 2, 7 copies; 256 parts each): op after op
-// 208-210 us, blocks of 8 .. 64 parts 197-198 us (7.1 TB/s), blocks of 128 214 us; ring and direct
-// all-reduces over 8 ranks x 1 .. 64 MiB and the 4096-op schedule (at most 3 parts per op) are
-// unchanged within 1 %.
+// 14 32 MiB ring steps (7 reductions 2 -> 2, 7 copies; 256 parts each): op after op 208-210 us,
+// blocks of 8 .. 64 parts 197-198 us, blocks of 128 214 us.  Most of that gain is the L2: each copy
+// there reads the buffer a reduction reads too, and in blocks the two run side by side; with copies
+// that read buffers of their own it is 212 -> 209 us.  Ring and direct all-reduces over 8 ranks x
+// 1 .. 64 MiB and the 4096-op schedule (at most 3 parts per op) are unchanged within 1 %.
 int order_block() {
   int block = 32;
   if (const char *env = getenv("PCCL_HIP_ORDER_BLOCK")) block = atoi(env);
