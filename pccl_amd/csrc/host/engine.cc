@@ -76,6 +76,9 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
   if (input_bytes < need || output_bytes < need)
     throw std::runtime_error("Engine::exeOp(): '" + name + "' needs " + std::to_string(need) +
                              " bytes per tensor, got " + std::to_string(input_bytes) + " / " + std::to_string(output_bytes));
+  // One graph runs one launch at a time: a run that an earlier call started on another stream ends
+  // before this call rebinds, rebuilds or runs the graph again (same stream: stream order does it).
+  if (op->graph && op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
   if (!op->graph) {
     const DeviceType rocm = TypeRegistry::getTypeId("rocm");
     char *ws = nullptr;
@@ -148,9 +151,6 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
                       (!in_moves || (apart(input, op->bound_in) && apart(input, op->bound_out))) &&
                       (!out_moves || (apart(output, op->bound_out) && apart(output, op->bound_in)));
     if (safe) {
-      // A previous exeOp of this op on another stream may still be reading the operand slots that a
-      // rebind rewrites behind `stream`: it ends first.
-      if (op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
       try {
         if (in_moves) {
           op->executor->rebindGraph(op->graph, op->bound_in, input, need, stream);
@@ -171,8 +171,7 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
         throw;
       }
     } else {
-      // (the graph's device state goes away: every stream it may still be running on ends first)
-      if (op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
+      // (the graph's device state goes away: the stream it may still be running on ends first)
       op->executor->waitGraph(op->graph, stream);
       op->executor->destroyGraph(op->graph);
       op->graph = nullptr;

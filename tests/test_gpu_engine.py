@@ -138,6 +138,36 @@ def test_signalled_ring_schedule(E, eng, oracle, tmp_path):
             H.assert_bits_equal(want[r * per:(r + 1) * per], want[:per], "rank %d equals rank 0" % r)
 
 
+def test_exe_op_on_another_stream_waits_for_the_run_before(E, eng, oracle, tmp_path):
+    """A registered op is one graph on the device and runs one launch at a time: exeOp on a second
+    stream, issued while the run on the first may still be going, starts behind it, and each call's
+    result is the checker's."""
+    import torch
+    p = str(tmp_path / "ring2s.sched")
+    E.write_ring_allreduce(p, "bf16", "sum", 8, 1 << 19)
+    eng.regOp("ring2s", p)
+    info = eng.opInfo("ring2s")
+    n = info["devices"] * info["elems_per_device"]
+    text = open(p).read()
+    inputs = [H.gen("bf16", n, 171 + k, 0) for k in range(3)]
+    wants = [_oracle_replay(oracle, text, a)[1] for a in inputs]
+    d_ins = [_to_dev(torch, a) for a in inputs]
+    d_outs = [torch.zeros(n * 2, dtype=torch.uint8, device="cuda") for _ in inputs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rounds in range(2):
+        for k in range(3):                      # streams alternate; inputs and outputs change every call
+            eng.exeOp("ring2s", d_ins[k], d_outs[k], streams[k % 2].cuda_stream)
+        # the same tensors again on the other stream, without anything in between
+        eng.exeOp("ring2s", d_ins[2], d_outs[2], streams[1].cuda_stream)
+        eng.waitOp("ring2s", streams[1].cuda_stream)
+        torch.cuda.synchronize()
+        for k in range(3):
+            H.assert_bits_equal(d_outs[k].cpu().numpy().view(np.uint16), wants[k], "round %d, call %d" % (rounds, k))
+            d_outs[k].zero_()
+        torch.cuda.synchronize()
+
+
 def test_exe_op_argument_errors(E, eng, tmp_path):
     import torch
     p = str(tmp_path / "r.sched")
