@@ -1,5 +1,6 @@
 #include "hip_device.h"
 
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <stdexcept>
@@ -194,7 +195,12 @@ void *HipExecutor::createGraph(const std::vector<BoundOp> &ops) {
   // the executor's choice: plain launches for the few graphs that run faster that way, else the queue
   long tile_bytes = PCCL_HIP_TILE_AUTO;
   const std::string tb = utils::LaunchEnvironments::getEnv("PCCL_HIP_TILE_BYTES");
-  if (!tb.empty()) tile_bytes = std::stol(tb);
+  if (!tb.empty()) {
+    char *end = nullptr;
+    tile_bytes = strtol(tb.c_str(), &end, 10);
+    if (end == tb.c_str() || *end != '\0')
+      throw std::runtime_error("HipExecutor::createGraph(): PCCL_HIP_TILE_BYTES='" + tb + "' is not a number of bytes");
+  }
   void *graph = nullptr;
   const int rc = pccl_hip_graph_create(descs.data(), (int)descs.size(), tile_bytes, &graph);
   if (rc != PCCL_OK) raise("pccl_hip_graph_create", rc);
