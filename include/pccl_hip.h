@@ -222,7 +222,8 @@ typedef struct pccl_op_desc {
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
 /* Drains the whole DAG with ONE persistent-kernel launch on `stream`; returns
- * without waiting.  The graph re-arms itself, so it can be run again.
+ * without waiting.  The graph re-arms itself, so it can be run again.  The calling thread's current
+ * device must be the one the graph was created on (PCCL_ERR_INVALID_ARG otherwise).
  * Role: Engine::exeOp, include/engine.h:19. */
 int pccl_hip_graph_run(void *graph, void *stream);
 

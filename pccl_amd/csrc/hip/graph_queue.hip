@@ -1363,6 +1363,10 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_run: graph is null");
+  // (a launch goes to the calling thread's current device, the graph's memory lives on the one it was created on)
+  int current = -1;
+  if (hipGetDevice(&current) != hipSuccess || current != G->device)
+    return fail(PCCL_ERR_INVALID_ARG, "graph_run: the graph was created on device %d, the current device is %d", G->device, current);
   if (G->as_launches) {
     std::vector<pccl_op_desc> launches;
     {
