@@ -78,7 +78,15 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
                              " bytes per tensor, got " + std::to_string(input_bytes) + " / " + std::to_string(output_bytes));
   // One graph runs one launch at a time: a run that an earlier call started on another stream ends
   // before this call rebinds, rebuilds or runs the graph again (same stream: stream order does it).
-  if (op->graph && op->last_stream_known && op->last_stream != stream) op->executor->waitGraph(op->graph, op->last_stream);
+  if (op->graph && op->last_stream_known && op->last_stream != stream) {
+    try {
+      op->executor->waitGraph(op->graph, op->last_stream);
+    } catch (...) {
+      // reported once (that run gave up, or its stream no longer exists); the op stays usable
+      op->last_stream_known = false;
+      throw;
+    }
+  }
   if (!op->graph) {
     const DeviceType rocm = TypeRegistry::getTypeId("rocm");
     char *ws = nullptr;
