@@ -99,7 +99,7 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
     const ComputeType compute = TypeRegistry::getTypeId(s.compute);
     const PrimitiveType copy = TypeRegistry::getTypeId("copy"), reduce = TypeRegistry::getTypeId("reduce");
     // "ws" operands live in per-device regions of the workspace, each as large as the schedule needs,
-    // laid out by the executor (the hip executor places them by the memory-channel rule of its allocator)
+    // laid out by the executor (back to back, each on a 256-byte boundary)
     long ws_need = 0;
     for (const ScheduleOp &o : s.ops) {
       if (o.isSignal()) continue;

@@ -45,7 +45,7 @@ public:
   // Byte offsets of n regions of nbytes_each inside [base, base + capacity): how the executor wants a
   // workspace divided among the devices of a schedule (the role of BufferManager::assignBuffer,
   // include/base/chunk.h:48-53).  Throws std::runtime_error when they do not fit.
-  // Default: back to back.
+  // Default: back to back, each region on a 256-byte boundary.
   virtual std::vector<long> carveWorkspace(const void *base, long capacity, int n, long nbytes_each);
 };
 

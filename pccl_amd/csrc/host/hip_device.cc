@@ -101,11 +101,12 @@ std::shared_ptr<ExecutorBase> getExecutor(ExecutorType type) {
 }
 
 std::vector<long> ExecutorBase::carveWorkspace(const void *, long capacity, int n, long nbytes_each) {
-  if (n < 1 || nbytes_each <= 0 || (long)n * nbytes_each > capacity)
+  const long stride = (nbytes_each + 255) / 256 * 256;  // every region starts on a 256-byte boundary of the workspace
+  if (n < 1 || nbytes_each <= 0 || (long)(n - 1) * stride + nbytes_each > capacity)
     throw std::runtime_error("carveWorkspace(): " + std::to_string(n) + " regions of " + std::to_string(nbytes_each) +
                              " bytes do not fit " + std::to_string(capacity) + " bytes");
   std::vector<long> offsets((size_t)n);
-  for (int k = 0; k < n; ++k) offsets[(size_t)k] = (long)k * nbytes_each;
+  for (int k = 0; k < n; ++k) offsets[(size_t)k] = (long)k * stride;
   return offsets;
 }
 
@@ -229,13 +230,6 @@ const GraphBufferLayout *HipExecutor::deviceLayout(void *graph) {
   const int rc = pccl_hip_graph_info(graph, &lay, nullptr, nullptr);
   if (rc != PCCL_OK) raise("pccl_hip_graph_info", rc);
   return static_cast<const GraphBufferLayout *>(lay);
-}
-
-std::vector<long> HipExecutor::carveWorkspace(const void *base, long capacity, int n, long nbytes_each) {
-  std::vector<long> offsets((size_t)std::max(n, 0));
-  const int rc = pccl_hip_carve(base, capacity, n, nbytes_each, offsets.data());
-  if (rc != PCCL_OK) raise("pccl_hip_carve", rc);
-  return offsets;
 }
 
 void HipExecutor::destroyGraph(void *graph) {

@@ -31,8 +31,6 @@ public:
   void rebindGraph(void *graph, const void *old_base, const void *new_base, long nbytes, void *stream) override;
   const GraphBufferLayout *deviceLayout(void *graph) override;
   void destroyGraph(void *graph) override;
-  // regions placed by the memory-channel rule of the plugin's allocator (pccl_hip_carve)
-  std::vector<long> carveWorkspace(const void *base, long capacity, int n, long nbytes_each) override;
 };
 
 // Registry id -> code of include/pccl_hip.h; throws std::runtime_error for an id

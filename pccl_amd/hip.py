@@ -67,11 +67,6 @@ def lib():
         L.pccl_hip_device_info.argtypes = [ctypes.POINTER(ci), ctypes.POINTER(cl), ctypes.c_char_p, ci]
         L.pccl_hip_alloc.argtypes = [ctypes.POINTER(vp), cl]
         L.pccl_hip_free.argtypes = [vp]
-        L.pccl_hip_alloc_group.argtypes = [ctypes.POINTER(vp), ci, cl, cl]
-        L.pccl_hip_carve.argtypes = [vp, cl, ci, cl, ctypes.POINTER(cl)]
-        L.pccl_hip_placement_start.argtypes = [ctypes.c_ulonglong, cl, cl, ctypes.POINTER(ctypes.c_ulonglong),
-                                               ctypes.POINTER(cl), ci, ctypes.POINTER(ctypes.c_ulonglong),
-                                               ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_accumulate.argtypes = [ci, ci, vp, ctypes.POINTER(vp), ci, cl, vp]
         L.pccl_hip_set_tuning.argtypes = [ci, ci]
@@ -140,32 +135,8 @@ def alloc(nbytes):
     return p.value
 
 
-def alloc_group(n, nbytes_each, pad_bytes=-1):
-    """n buffers out of one allocation, staggered by pad_bytes; free the group with free(ptrs[0])."""
-    arr = (ctypes.c_void_p * n)()
-    _check(lib().pccl_hip_alloc_group(arr, n, nbytes_each, pad_bytes))
-    return [arr[k] for k in range(n)]
-
-
 def free(ptr):
     _check(lib().pccl_hip_free(ctypes.c_void_p(ptr)))
-
-
-def carve(base, capacity, n, nbytes_each):
-    """Byte offsets of n placed buffers inside memory the caller holds (pccl_hip_carve)."""
-    offs = (ctypes.c_long * n)()
-    _check(lib().pccl_hip_carve(ctypes.c_void_p(_addr(base)), capacity, n, nbytes_each, offs))
-    return list(offs)
-
-
-def placement_start(extent, nbytes, slack, before=()):
-    """(start, channel group of the start) the allocator's placing rule picks; touches no device."""
-    n = len(before)
-    addrs = (ctypes.c_ulonglong * max(n, 1))(*[a for a, _ in before])
-    sizes = (ctypes.c_long * max(n, 1))(*[b for _, b in before])
-    start, code = ctypes.c_ulonglong(0), ctypes.c_uint(0)
-    _check(lib().pccl_hip_placement_start(extent, nbytes, slack, addrs, sizes, n, ctypes.byref(start), ctypes.byref(code)))
-    return start.value, code.value
 
 
 def set_rotation(rotate=-1):

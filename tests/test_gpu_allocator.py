@@ -1,4 +1,5 @@
-"""The plugin's allocator on the GPU: extents of a few large blocks, placed starts, reuse after free."""
+"""The plugin's allocator on the GPU: 2 MiB-rounded allocations tracked by pointer (the role of
+csrc/plugins/cuda_executor/device.cc:59-144)."""
 import numpy as np
 import pytest
 
@@ -24,32 +25,41 @@ def _fill_and_check(torch, hip, ptrs, nbytes):
         assert torch.equal(back, srcs[k]), "buffer %d was overwritten" % k
 
 
-def test_allocations_are_disjoint_aligned_and_reused(hip):
+def test_allocations_are_disjoint_aligned_and_tracked(hip):
     import torch
     sizes = [100, 3 * MIB + 5, 16 * MIB, 40 * MIB, 16 * MIB, 2 * MIB]
     ptrs = [hip.alloc(n) for n in sizes]
     assert all(p % 4096 == 0 for p in ptrs)
-    spans = sorted((p, p + n) for p, n in zip(ptrs, sizes))
+    # every allocation has its size rounded up to 2 MiB to itself
+    spans = sorted((p, p + (n + 2 * MIB - 1) // (2 * MIB) * (2 * MIB)) for p, n in zip(ptrs, sizes))
     assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
     _fill_and_check(torch, hip, ptrs, 100)
-    # freeing the middle ones and asking again for what fits there stays inside the same memory
-    lo, hi = spans[0][0], spans[-1][1]
+    # the last bytes of a rounded allocation are usable
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.arange(256, dtype=torch.uint8, device="cuda")
+    end = ptrs[1] + 4 * MIB - 256
+    hip.reduce_copy("f8e4m3", "sum", [src], [end], 256, stream)
+    back = torch.empty_like(src)
+    hip.reduce_copy("f8e4m3", "sum", [end], [back], 256, stream)
+    torch.cuda.synchronize()
+    assert torch.equal(back, src)
     hip.free(ptrs[2])
     hip.free(ptrs[3])
     again = hip.alloc(50 * MIB)
-    assert lo <= again < hi, "a freed extent was not reused"
+    _fill_and_check(torch, hip, [ptrs[0], ptrs[1], ptrs[4], ptrs[5], again], 100)
     for p in (ptrs[0], ptrs[1], ptrs[4], ptrs[5], again):
         hip.free(p)
     with pytest.raises(hip.PcclError):
         hip.free(ptrs[0])          # already gone
     with pytest.raises(hip.PcclError):
+        hip.free(again + 4096)     # not the start of an allocation
+    with pytest.raises(hip.PcclError):
         hip.alloc(0)
+    hip.free(0)                    # (a null pointer is fine, as for hipFree)
 
 
-def test_large_buffers_allocated_one_by_one_differ_in_their_channel_groups(hip, oracle):
-    """Nine 64 MiB buffers from nine calls: their starts, seen as offsets inside the allocator's block,
-    follow the placing rule (checked on the CPU in test_placement.py); here: they hold data independently
-    and a fold over them is bit-exact."""
+def test_large_buffers_allocated_one_by_one_hold_operands(hip, oracle):
+    """Nine 64 MiB buffers from nine calls hold data independently and a fold over them is bit-exact."""
     import torch
     n, count = 9, 32 * MIB          # bf16 elements: 64 MiB per buffer
     ptrs = [hip.alloc(2 * count) for _ in range(n)]
@@ -63,30 +73,6 @@ def test_large_buffers_allocated_one_by_one_differ_in_their_channel_groups(hip, 
     got = torch.empty(count, dtype=torch.int16, device="cuda")
     hip.reduce_copy("bf16", "sum", [ptrs[n - 1]], [got], count, stream)
     torch.cuda.synchronize()
-    H.assert_bits_equal(got.cpu().numpy().view(np.uint16), oracle.reduce("bf16", "sum", ins), "fold over placed buffers")
+    H.assert_bits_equal(got.cpu().numpy().view(np.uint16), oracle.reduce("bf16", "sum", ins), "fold over plugin-allocated buffers")
     for p in ptrs:
         hip.free(p)
-
-
-def test_a_request_beyond_half_a_block_gets_its_own(hip):
-    import torch
-    big = hip.alloc(3 << 30)
-    small = hip.alloc(MIB)
-    assert not (big <= small < big + (3 << 30))
-    stream = torch.cuda.current_stream().cuda_stream
-    src = torch.arange(1 << 20, dtype=torch.int32, device="cuda")
-    hip.reduce_copy("i32", "sum", [src], [big + (3 << 30) - (4 << 20)], 1 << 20, stream)   # its last 4 MiB are there
-    back = torch.empty_like(src)
-    hip.reduce_copy("i32", "sum", [big + (3 << 30) - (4 << 20)], [back], 1 << 20, stream)
-    torch.cuda.synchronize()
-    assert torch.equal(back, src)
-    hip.free(big)
-    hip.free(small)
-
-
-def test_carve_inside_an_allocation(hip):
-    base = hip.alloc(256 * MIB)
-    offs = hip.carve(base, 256 * MIB, 8, 30 * MIB)
-    assert all(o % 256 == 0 for o in offs) and offs[-1] + 30 * MIB <= 256 * MIB
-    assert all(b - a >= 30 * MIB for a, b in zip(offs, offs[1:]))
-    hip.free(base)

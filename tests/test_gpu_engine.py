@@ -247,9 +247,9 @@ def test_python_emitted_collectives(E, eng, oracle, tmp_path, which):
 
 def test_schedule_staging_through_the_workspace(E, eng, oracle, tmp_path):
     """Operands named "ws" live in per-device regions of the engine's workspace, laid out by the
-    executor (placed by the allocator's memory-channel rule): ws[r] = in[r] + in[r+1]; out[r] = ws[r]."""
+    executor (back to back, each on a 256-byte boundary): ws[r] = in[r] + in[r+1]; out[r] = ws[r]."""
     import torch
-    W, n = 4, 3 * 1000 * 1000 + 7      # 12 MB per region: large enough for the regions to be placed
+    W, n = 4, 3 * 1000 * 1000 + 7      # 12 MB per region, a ragged size: the regions' starts are rounded to 256 bytes
     lines = ["pccl-schedule 1", "name staged", "dtype f32", "compute sum", "devices %d" % W,
              "elems_per_device %d" % n, "ops %d" % (2 * W)]
     for r in range(W):

@@ -316,35 +316,6 @@ def test_operands_longer_than_one_launch_covers(hip, oracle):
         hip.set_slice_bytes(0)
 
 
-def test_group_allocation(hip, oracle):
-    """pccl_hip_alloc_group: n buffers out of one allocation at the stated stride, usable as
-    operands, freed through the first one."""
-    import torch
-    n, nbytes = 5, (3 << 20) + 100
-    ptrs = hip.alloc_group(n, nbytes, 8192)
-    stride = (nbytes + 255) // 256 * 256 + 8192
-    assert [p - ptrs[0] for p in ptrs] == [k * stride for k in range(n)] and ptrs[0] % 256 == 0
-    count = nbytes // 4
-    ins = [H.gen("f32", count, 55, k) for k in range(n - 1)]
-    stream = torch.cuda.current_stream().cuda_stream
-    for a, p in zip(ins, ptrs):
-        t = torch.from_numpy(a).cuda()
-        hip.reduce_copy("f32", "sum", [t], [p], count, stream)
-    hip.reduce_copy("f32", "sum", ptrs[:n - 1], [ptrs[n - 1]], count, stream)
-    got = torch.empty(count, dtype=torch.float32, device="cuda")
-    hip.reduce_copy("f32", "sum", [ptrs[n - 1]], [got], count, stream)
-    torch.cuda.synchronize()
-    H.assert_bits_equal(got.cpu().numpy(), oracle.reduce("f32", "sum", ins), "operands from a group allocation")
-    hip.free(ptrs[0])
-    with pytest.raises(hip.PcclError):
-        hip.free(ptrs[1])           # only the first buffer names the group
-    d = hip.alloc_group(2, 1 << 20)  # built-in stagger
-    assert d[1] - d[0] > (1 << 20)
-    hip.free(d[0])
-    with pytest.raises(hip.PcclError):
-        hip.alloc_group(0, 16)
-
-
 # ---- the fold rounds to binary32 at every step, then once to the element type ----------------
 
 def _tie_tuples(oracle, dtype, compute, n_in, want, seed):
