@@ -74,6 +74,13 @@ int pccl_hip_device_count(int *n);
  * reporting; the reference has no counterpart because it has no launches). */
 int pccl_hip_device_info(int *compute_units, long *hbm_bytes, char *name, int name_len);
 
+/* The id under which the host's TypeRegistry registered this executor (registerExecutorType,
+ * include/base/registry.h:37; ids come from one run-time counter, :79).  The plugin writes it into
+ * RingBuffer::producer_ / consumer_ (include/base/operator.h:8-9) and
+ * OperationLayoutHeader::executor_type_ (:24) of every graph created afterwards; a caller of the bare
+ * C ABI that never sets it gets 0 there.  0..255. */
+int pccl_hip_set_executor_id(int id);
+
 /* Device memory, tracked until freed: one hipMalloc per call, the size rounded up to 2 MiB, in a
  * pointer-keyed map under a mutex.  nbytes <= 0 yields PCCL_ERR_INVALID_ARG and *p == NULL.
  * Role: CudaDevice::allocate / deallocate, csrc/plugins/cuda_executor/device.cc:59-144 (2 MiB
@@ -282,23 +289,25 @@ int pccl_hip_graph_next_signal_base(void *graph, unsigned int *base);
  * was recorded with). */
 int pccl_hip_graph_set_spin_limit(void *graph, unsigned int microseconds);
 
-/* pccl_hip_graph_create + pccl_hip_graph_run in one call that allocates NO device memory: the
- * graph's device state (headers, payloads, counters, ready queues: what graph_create puts into a
- * hipMalloc'ed arena) goes into a fixed array inside the library's code object, of which every GPU
- * holds one copy of PCCL_HIP_STATIC_ARENA_BYTES until the process ends.  No counterpart in the
- * reference; it is for callers that cannot allocate: tight serving loops and harnesses that forbid
- * hipMalloc.  The call uploads the state behind earlier work on `stream` and launches the drain kernel
- * there.  A call with the very same ops as the last one on this GPU skips the upload (the state re-arms
- * itself).  A graph that needs more than the array holds (about 4,500 ops of three parts each) is
- * refused with PCCL_ERR_NOMEM and nothing is launched.  completed / total both NULL: returns without
- * waiting.  Otherwise waits for `stream` and reports the two counters of operator.h:32-33
- * (PCCL_ERR_GRAPH if the drain gave up; the next call then uploads the state afresh).  A caller that
- * always passes NULL for both never learns that a wait gave up: later calls with the same ops launch
- * onto the abandoned state, where every workgroup leaves at once.  Graphs that wait for peers on signal
- * words should read the counters at least now and then.  All calls on one GPU share the one array: a call waits for
- * the previous one's stream before it rewrites the state, and calls issued at the same time from
- * several threads or onto streams that overlap race.  Not meant to be recorded by stream capture (the
- * upload reads host memory). */
+/* pccl_hip_graph_create + pccl_hip_graph_run in one call that allocates NO device memory.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate: tight serving loops and harnesses
+ * that forbid hipMalloc.  The graph's device state (headers, payloads, counters, ready queues: what
+ * graph_create puts into a hipMalloc'ed arena) goes into a fixed array inside the library's code object,
+ * of which every GPU holds one copy of PCCL_HIP_STATIC_ARENA_BYTES until the process ends.  (Host memory:
+ * the library's own vectors, which stop growing once they have held the largest graph.)
+ * All calls on one GPU share the one array, so a call first waits for the previous call's run to end,
+ * whichever stream that went to, and looks at its abort word: if a wait inside that run gave up, this call
+ * returns PCCL_ERR_GRAPH, launches nothing, and the call after it uploads the state afresh (a caller that
+ * passes no counters learns of a failed run this way, one call late).  Then the call uploads the state
+ * behind earlier work on `stream` and launches the drain kernel there; a call with the very same ops as
+ * the last one on this GPU skips the upload (the state re-arms itself).  A graph that needs more than the
+ * array holds (about 4,500 ops of three parts each) is refused with PCCL_ERR_NOMEM and nothing is launched.
+ * completed / total both NULL: returns without waiting for the run it launched.  Otherwise waits for
+ * `stream` and reports the graph's two progress counters (PCCL_ERR_GRAPH if the drain gave up; the next
+ * call then uploads the state afresh).  Calls issued at the same time from several threads are
+ * serialised by the library; work of the caller's own on other streams that touches the operands is the
+ * caller's to order.  Not meant to be recorded by stream capture (the upload reads host memory and the
+ * call waits for a stream). */
 #define PCCL_HIP_STATIC_ARENA_BYTES (8u << 20)
 int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_bytes, void *stream,
                               unsigned int *completed, unsigned int *total);

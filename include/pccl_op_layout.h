@@ -33,7 +33,9 @@ typedef struct pccl_chunk_meta {
  * tail_ counts entries published, head_ counts entries claimed; both only grow
  * during a run and the run's last workgroup rewinds them.  producer_buffer_ and
  * consumer_buffer_ name the same device array when producer and consumer are
- * the same executor, which is the only case on one GPU. */
+ * the same executor, which is the only case on one GPU.  producer_ and consumer_
+ * carry the registry id given to pccl_hip_set_executor_id (the host layer passes
+ * the id of "hip"; 0 if the C ABI is used without it). */
 typedef struct pccl_ring_buffer {
   pccl_general_type producer_; /* @0  ExecutorType */
   pccl_general_type consumer_; /* @1  ExecutorType */
@@ -54,6 +56,8 @@ typedef struct pccl_ring_buffer {
  *                        word of its own per op (outside this struct, alone on a
  *                        cache line) and runs the op when that count equals
  *                        this field;
+ *   executor_type_       registry id of the executor that runs the op (see
+ *                        pccl_ring_buffer::producer_);
  *   op_buffer_/op_size_  payload: pccl_op_payload, at most 255 bytes;
  *   next_op_uids_head_   num_next_ops_ successor uids. */
 typedef struct pccl_operation_layout_header {

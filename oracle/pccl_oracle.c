@@ -394,12 +394,13 @@ void pccl_oracle_fill_uniform_f32(float *dst, long n, uint64_t seed, uint64_t st
   }
 }
 
-void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64_t stream,
-                             double mean, double sigma) {
+void pccl_oracle_fill_normal_at(void *dst, int dtype, long first, long n, uint64_t seed, uint64_t stream,
+                                double mean, double sigma) {
   const double two_pi = 6.283185307179586476925286766559;
   for (long i = 0; i < n; ++i) {
-    uint64_t a = pccl_oracle_rng_u64(seed, stream, 2 * (uint64_t)i);
-    uint64_t b = pccl_oracle_rng_u64(seed, stream, 2 * (uint64_t)i + 1);
+    const uint64_t at = (uint64_t)(first + i);
+    uint64_t a = pccl_oracle_rng_u64(seed, stream, 2 * at);
+    uint64_t b = pccl_oracle_rng_u64(seed, stream, 2 * at + 1);
     double u1 = ((double)(a >> 11) + 1.0) * (1.0 / 9007199254740992.0); /* (0, 1] */
     double u2 = (double)(b >> 11) * (1.0 / 9007199254740992.0);         /* [0, 1) */
     const double zd = mean + sigma * sqrt(-2.0 * log(u1)) * cos(two_pi * u2);
@@ -414,6 +415,11 @@ void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64
       default: return;
     }
   }
+}
+
+void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64_t stream,
+                             double mean, double sigma) {
+  pccl_oracle_fill_normal_at(dst, dtype, 0, n, seed, stream, mean, sigma);
 }
 
 void pccl_oracle_fill_int32(int32_t *dst, long n, uint64_t seed, uint64_t stream,

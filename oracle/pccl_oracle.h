@@ -132,6 +132,10 @@ void pccl_oracle_fill_uniform_f32(float *dst, long n, uint64_t seed, uint64_t st
  * (F32, BF16, F16, F8E4M3, F8E5M2) with round-to-nearest-even. */
 void pccl_oracle_fill_normal(void *dst, int dtype, long n, uint64_t seed, uint64_t stream,
                              double mean, double sigma);
+/* Values first .. first + n - 1 of the same stream into dst[0 .. n): slices of one buffer can be
+ * filled by several threads. */
+void pccl_oracle_fill_normal_at(void *dst, int dtype, long first, long n, uint64_t seed, uint64_t stream,
+                                double mean, double sigma);
 /* uniform integers in [lo, hi] */
 void pccl_oracle_fill_int32(int32_t *dst, long n, uint64_t seed, uint64_t stream,
                             int32_t lo, int32_t hi);

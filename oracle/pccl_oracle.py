@@ -68,6 +68,8 @@ def lib():
         L.pccl_oracle_fill_uniform_f32.restype = None
         L.pccl_oracle_fill_normal.argtypes = [vp, ci, cl, u64, u64, ctypes.c_double, ctypes.c_double]
         L.pccl_oracle_fill_normal.restype = None
+        L.pccl_oracle_fill_normal_at.argtypes = [vp, ci, cl, cl, u64, u64, ctypes.c_double, ctypes.c_double]
+        L.pccl_oracle_fill_normal_at.restype = None
         L.pccl_oracle_fill_int32.argtypes = [vp, cl, u64, u64, ctypes.c_int32, ctypes.c_int32]
         L.pccl_oracle_fill_int32.restype = None
         _lib = L
@@ -172,10 +174,22 @@ def fill_uniform_f32(n, seed, stream, lo, hi):
     return a
 
 
-def fill_normal(dtype, n, seed, stream, mean=0.0, sigma=1.0):
+def fill_normal(dtype, n, seed, stream, mean=0.0, sigma=1.0, nthreads=1):
+    """N(mean, sigma) values 0 .. n-1 of the stream; nthreads > 1 fills contiguous slices in parallel
+    (the generator is counter-based: the same bytes either way)."""
     dt = _code(DTYPES, dtype)
     a = np.empty(n, dtype=NP_STORAGE[dt])
-    lib().pccl_oracle_fill_normal(a.ctypes.data, dt, n, seed, stream, mean, sigma)
+    if nthreads <= 1 or n < (1 << 16):
+        lib().pccl_oracle_fill_normal(a.ctypes.data, dt, n, seed, stream, mean, sigma)
+        return a
+    from concurrent.futures import ThreadPoolExecutor
+    per = (n + nthreads - 1) // nthreads
+    fill = lib().pccl_oracle_fill_normal_at   # (ctypes releases the interpreter lock during the call)
+    with ThreadPoolExecutor(nthreads) as pool:
+        jobs = [pool.submit(fill, a.ctypes.data + lo * a.itemsize, dt, lo, min(per, n - lo), seed, stream, mean, sigma)
+                for lo in range(0, n, per)]
+        for j in jobs:
+            j.result()
     return a
 
 

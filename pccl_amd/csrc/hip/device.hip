@@ -62,6 +62,11 @@ Tuning tuning() {
                 g_tune_rotate.load(std::memory_order_relaxed)};
 }
 
+// The id under which the host's TypeRegistry knows this executor (ids are handed out at run time from
+// one shared counter, include/base/registry.h:79); written into the executor fields of the device image.
+static std::atomic<int> g_executor_id{0};
+int executor_id() { return g_executor_id.load(std::memory_order_relaxed); }
+
 // A grid times its 256 lanes must fit 32 bits, so a launch with one workgroup per 4 KiB of every stream
 // reaches just under 64 GiB per stream; operands are cut into slices of half that.
 static std::atomic<long> g_slice_bytes{32l << 30};
@@ -164,6 +169,13 @@ int pccl_hip_free(void *p) {
     mem_map()[p] = b;
     return fail(PCCL_ERR_HIP, "pccl_hip_free: hipFree(%p): %s (the buffer is still allocated)", p, hipGetErrorString(e));
   }
+  return PCCL_OK;
+}
+
+int pccl_hip_set_executor_id(int id) {
+  clear_error();
+  if (id < 0 || id > 255) return fail(PCCL_ERR_INVALID_ARG, "executor id %d does not fit the registry's unsigned char", id);
+  g_executor_id.store(id, std::memory_order_relaxed);
   return PCCL_OK;
 }
 

@@ -83,6 +83,17 @@ DrainKernel drain_for(int dtype, int compute, bool forward) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// How long a wait inside the kernel may last for a graph created from now on: two seconds, or
+// PCCL_HIP_SPIN_LIMIT_US (at least 64; read at every creation).  pccl_hip_graph_set_spin_limit changes
+// it for one graph; pccl_hip_graph_run_static, which hands out no graph, only has this.
+unsigned int default_spin_limit() {
+  if (const char *env = getenv("PCCL_HIP_SPIN_LIMIT_US")) {
+    const long v = atol(env);
+    if (v > 0) return (unsigned int)std::min<long>(std::max<long>(v, 64), 0x7fffffffl);
+  }
+  return kDefaultSpinLimit;
+}
+
 int elem_bytes(int dtype) { return pccl_host::pccl_dtype_bytes(dtype); }
 
 struct Graph {
@@ -1210,8 +1221,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       C->queue_head[q] = &((pccl_ring_buffer *)(dev + off_ring + 256 * (size_t)q))->head_;
       C->queue_entries[q] = (const unsigned long long *)(dev + pos);
       ((int *)(img + off_qcount))[q] = (int)qe[q].size();
-      R->producer_ = 0;  // executor ids are the host layer's; one executor fills and drains
-      R->consumer_ = 0;
+      R->producer_ = (pccl_general_type)pccl_host::executor_id();  // one executor fills and drains
+      R->consumer_ = (pccl_general_type)pccl_host::executor_id();
       R->elem_size_ = (int)sizeof(pccl_queue_entry);
       R->max_num_elems_ = (int)qe[q].size();
       R->max_flush_time_ = 0;  // producer and consumer share one address space: nothing to flush
@@ -1232,7 +1243,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     h->required_executors_ = parts[i];
     h->remaining_executors_ = parts[i] > kGroupThreshold ? kPartGroups : parts[i];
     h->pre_dependencies_ = (unsigned char)n_pred[i];
-    h->executor_type_ = 0;
+    h->executor_type_ = (pccl_general_type)pccl_host::executor_id();
     h->op_size_ = (unsigned char)(8 + sizeof(pccl_chunk_meta) * (size_t)(o.n_in + o.n_out));
     h->num_next_ops_ = (unsigned char)n_succ[i];
     h->op_buffer_ = dev + off_payload + kPayloadStride * (size_t)i;
@@ -1262,16 +1273,25 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
   G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
   {
-    // entries without tickets (graph_queue_device.h): when they are few per workgroup; beyond one
-    // each the mapping of entries to workgroups needs every queue to have the same number of workgroups.
-    // With one entry each a workgroup only ever waits for workgroups that were started before it; with
-    // more (PCCL_HIP_OWN_ENTRIES > 1, not the default) a workgroup's second entry can wait for the first
-    // entry of a workgroup that has no compute unit yet, which is only safe while nothing else keeps
-    // the launch from being resident as a whole.
+    // Entries without tickets (graph_queue_device.h): when there is at most one per workgroup
+    // (PCCL_HIP_OWN_ENTRIES=k: up to k; the mapping of entries to workgroups then needs every queue to
+    // have the same number of workgroups) AND no queued entry waits for another entry of this graph.
+    // An entry that belongs to a workgroup by number can belong to one that has no compute unit yet;
+    // whoever waits for it then waits for the dispatcher, which hands out a launch's workgroups in
+    // order per XCD but shares the compute units with whatever else runs: beside a second graph of
+    // this kind (or any kernel that does not end by itself) the two can hold each other's compute
+    // units while the entries they wait for sit with workgroups that cannot start.  Tickets have no
+    // such case (only a running workgroup ever holds an entry), so graphs whose entries depend on
+    // each other draw tickets; chains' heads, independent ops and waits for signals from outside the
+    // graph depend on no other entry.
     long long rounds = 1;
     if (const char *env = getenv("PCCL_HIP_OWN_ENTRIES")) rounds = atoll(env);
-    const bool own = rounds > 0 && (live_tiles <= (long long)G->n_wg ||
-                                    (G->n_wg % kQueues == 0 && live_tiles <= rounds * (long long)G->n_wg));
+    bool entries_wait = false;
+    for (int i = 0; i < n_ops && !entries_wait; ++i)
+      entries_wait = queued(i) && (n_pred[i] > 0 || order_pred[i] > 0);
+    const bool own = rounds > 0 && !entries_wait &&
+                     (live_tiles <= (long long)G->n_wg ||
+                      (G->n_wg % kQueues == 0 && live_tiles <= rounds * (long long)G->n_wg));
     ((int *)(img + off_qcount))[kQueues] = own ? 1 : 0;
   }
 
@@ -1297,8 +1317,10 @@ struct StaticArena {
   Graph *graph = nullptr;       // host side of what the array holds now
   bool valid = false;           // ... and it is complete and was not left behind by an aborted run
   bool used = false;
+  bool launched = false;        // a drain kernel has run on the state the array holds now
   hipStream_t last_stream = nullptr;
   unsigned int runs = 0;        // launches on this array so far (signal values go on from here)
+  std::vector<int> deps;        // the call's dependency lists, back to back (kept between calls: no host allocation once it has grown)
 };
 std::mutex g_static_mutex;
 StaticArena g_static[kMaxStaticDevices];
@@ -1320,6 +1342,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   // own copy of the ops and their dependency lists
   Graph *G = new Graph();
   G->tile_bytes = tile_bytes;
+  G->spin_limit = default_spin_limit();
   G->descs.assign(ops, ops + n_ops);
   size_t n_deps = 0;
   for (int i = 0; i < n_ops; ++i) {
@@ -1539,6 +1562,14 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
       const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
       PCCL_HIP_CHECK(hipMemcpy(&run_word, G->dev + off_hot + sizeof(HotWord) * kHotRun, sizeof(run_word),
                                hipMemcpyDeviceToHost));
+      // A run that gave up and that nobody has asked about yet: the new state would bury its abort
+      // word.  Nothing is changed; pccl_hip_graph_status reports that run and restores the graph.
+      unsigned int gave_up = 0;
+      PCCL_HIP_CHECK(hipMemcpy(&gave_up, G->dev + off_hot + sizeof(HotWord) * kHotAbort, sizeof(gave_up),
+                               hipMemcpyDeviceToHost));
+      if (gave_up)
+        return fail(PCCL_ERR_GRAPH, "graph_rebind: the graph's last run gave up and has not been reported yet; "
+                                    "call pccl_hip_graph_status first (it restores the graph), then rebind");
     }
     const int rc = build_graph(&fresh, run_word, G->dev, G->arena_bytes);
     if (rc != PCCL_OK) return rc;
@@ -1735,12 +1766,33 @@ int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_byte
     if (ops[i].n_deps < 0 || (ops[i].n_deps > 0 && !ops[i].deps)) return fail(PCCL_ERR_GRAPH, "op %d: bad dependency list", i);
     n_deps += (size_t)ops[i].n_deps;
   }
-  std::vector<int> deps;
+  std::vector<int> &deps = S.deps;
+  deps.clear();
   deps.reserve(n_deps);
   for (int i = 0; i < n_ops; ++i) deps.insert(deps.end(), ops[i].deps, ops[i].deps + ops[i].n_deps);
   Graph *G = S.graph;
+  // Every call on this GPU shares the one array, so the previous call's run ends first, whatever stream
+  // it went to and whether or not this call brings the same ops: two drains on the one state would race,
+  // and a new upload would pull the state from under a running one.  With the run over, its abort word
+  // says whether a wait inside it gave up.  A caller that passed no counters has not heard of that; it
+  // hears now, nothing is launched on the abandoned state (every workgroup would leave at once and the
+  // outputs would stay as they are), and the call after this one uploads the state afresh.
+  if (S.used) PCCL_HIP_CHECK(hipStreamSynchronize(S.last_stream));
+  if (S.valid && S.launched) {
+    const size_t off_hot = (size_t)((const char *)((const GraphControl *)G->image.data())->hot - G->dev);
+    unsigned int gave_up = 0;
+    PCCL_HIP_CHECK(hipMemcpy(&gave_up, G->dev + off_hot + sizeof(HotWord) * kHotAbort, sizeof(gave_up), hipMemcpyDeviceToHost));
+    if (gave_up) {
+      S.valid = false;
+      S.launched = false;
+      return fail(PCCL_ERR_GRAPH, "graph_run_static: the previous run on this GPU gave up (an op's dependencies or a signal "
+                                  "were not satisfied within the spin limit); nothing was launched, the next call uploads fresh state");
+    }
+  }
   auto same_ops = [&] {
-    if (!S.valid || (int)G->descs.size() != n_ops || G->tile_bytes != tile_bytes || G->deps_store != deps) return false;
+    if (!S.valid || (int)G->descs.size() != n_ops || G->tile_bytes != tile_bytes || G->deps_store != deps ||
+        G->spin_limit != default_spin_limit())
+      return false;
     for (int i = 0; i < n_ops; ++i) {
       const pccl_op_desc &a = G->descs[i], &b = ops[i];
       if (a.op_uid != b.op_uid || a.primitive != b.primitive || a.dtype != b.dtype || a.compute != b.compute ||
@@ -1751,11 +1803,10 @@ int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_byte
     return true;
   };
   if (!same_ops()) {
-    // The array still serves the previous call, and the host image that call was uploaded from is
-    // about to be rewritten: that call's work ends first.
-    if (S.used) PCCL_HIP_CHECK(hipStreamSynchronize(S.last_stream));
     S.valid = false;
+    S.launched = false;
     G->tile_bytes = tile_bytes;
+    G->spin_limit = default_spin_limit();
     G->descs.assign(ops, ops + n_ops);
     G->deps_store.swap(deps);
     for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) G->descs[i].deps = G->deps_store.data() + at;
@@ -1773,6 +1824,7 @@ int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_byte
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run_static launch failed: %s", hipGetErrorString(e));
     ++S.runs;
+    S.launched = true;
   }
   if (!completed && !total) return PCCL_OK;
   PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
@@ -1784,6 +1836,7 @@ int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_byte
   if (total) *total = hot[kHotTotal].value;
   if (hot[kHotAbort].value) {
     S.valid = false;  // the next call uploads a fresh image
+    S.launched = false;
     return fail(PCCL_ERR_GRAPH, "drain gave up: an op's dependencies were not satisfied within the spin limit "
                                 "(%u of %u ops had completed)", hot[kHotCompleted].value, hot[kHotTotal].value);
   }

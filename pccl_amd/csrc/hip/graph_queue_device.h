@@ -543,10 +543,9 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   // workgroups; entry b / kQueues + k * W / kQueues of its home queue) and leaves when its home queue
   // has no more.  No ticket is drawn, and no workgroup goes round the eight queues at the end to find
   // each of them empty (eight returning atomics, one after the other: 14.9 -> 11 us for a graph of one
-  // 64 KiB op).  The host asks for it (mode word) when the entries are few per workgroup.
-  // Dependencies point backwards in the global order, a workgroup takes its entries in that order
-  // and workgroups are started in order, so the owner of the lowest-numbered unfinished entry is
-  // always at that entry and never waits for one that has not started.
+  // 64 KiB op).  The host asks for it (mode word) when the entries are few per workgroup and none of
+  // them waits for another entry of the graph: an entry then never waits for a workgroup that the
+  // dispatcher has not started yet.
   // The mode word sits behind the queue lengths in memory, not in the kernel arguments: a rebind can
   // change the number of entries (see GraphControl::queue_count).  Thread 0 reads it before its first
   // claim, together with the entry that would be its own (a load from inside the queue's room even

@@ -24,6 +24,9 @@ inline int pccl_dtype_bytes(int dtype) {
 // Compute units of the current device (cached per device index).
 int compute_units();
 
+// What pccl_hip_set_executor_id was given (0 before any call).
+int executor_id();
+
 struct Tuning {
   int workgroups_per_cu;  // 0 = built-in choice
   int cache_treatment;        // -1 = built-in choice, else 0 cacheable / 1 streaming / 2 streaming loads + write-through stores

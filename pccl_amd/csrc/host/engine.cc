@@ -1,6 +1,7 @@
 #include "engine.h"
 
 #include <algorithm>
+#include <exception>
 #include <stdexcept>
 
 #include "device_plugin.h"
@@ -158,6 +159,7 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
     const bool safe = apart(op->bound_in, op->bound_out) && apart(input, output) &&
                       (!in_moves || (apart(input, op->bound_in) && apart(input, op->bound_out))) &&
                       (!out_moves || (apart(output, op->bound_out) && apart(output, op->bound_in)));
+    bool rebuild = !safe;
     if (safe) {
       try {
         if (in_moves) {
@@ -168,21 +170,25 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
           op->executor->rebindGraph(op->graph, op->bound_out, output, need, stream);
           op->bound_out = output;
         }
-      } catch (...) {
-        // half-moved operands are not worth tracking: the next exeOp builds the graph again
-        try {
-          op->executor->waitGraph(op->graph, stream);
-        } catch (...) {
-        }
-        op->executor->destroyGraph(op->graph);
-        op->graph = nullptr;
-        throw;
+      } catch (const std::exception &e) {
+        // (the executor cannot move this graph's operands, or moved only half of them: build it again)
+        PCCL_LOG_WARN("Engine::exeOp(): '%s' is built again for its new tensors: %s", name.c_str(), e.what());
+        rebuild = true;
       }
-    } else {
-      // (the graph's device state goes away: the stream it may still be running on ends first)
-      op->executor->waitGraph(op->graph, stream);
+    }
+    if (rebuild) {
+      // The graph's device state goes away: the stream it may still be running on ends first.  If that
+      // run gave up, this call reports it (once); the graph is gone either way and the next call builds it.
+      std::exception_ptr gave_up;
+      try {
+        op->executor->waitGraph(op->graph, stream);
+      } catch (...) {
+        gave_up = std::current_exception();
+      }
       op->executor->destroyGraph(op->graph);
       op->graph = nullptr;
+      op->last_stream_known = false;
+      if (gave_up) std::rethrow_exception(gave_up);
       exeOp(name, input, output, input_bytes, output_bytes, stream);
       return;
     }

@@ -36,6 +36,7 @@ struct HipPluginRegistration {
     regDev(device, std::make_shared<HipDevice>());
     CodeTable &t = codes();
     t.executor = TypeRegistry::registerExecutorType("hip");
+    (void)pccl_hip_set_executor_id((int)t.executor);  // what the device image's executor fields carry
     const char *prims[] = {"copy", "reduce", "notify", "get_notified"};
     const int prim_codes[] = {PCCL_COPY, PCCL_REDUCE, PCCL_NOTIFY, PCCL_GET_NOTIFIED};
     for (int i = 0; i < 4; ++i) {

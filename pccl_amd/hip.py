@@ -65,6 +65,7 @@ def lib():
         vp, ci, cl = ctypes.c_void_p, ctypes.c_int, ctypes.c_long
         L.pccl_hip_device_count.argtypes = [ctypes.POINTER(ci)]
         L.pccl_hip_device_info.argtypes = [ctypes.POINTER(ci), ctypes.POINTER(cl), ctypes.c_char_p, ci]
+        L.pccl_hip_set_executor_id.argtypes = [ci]
         L.pccl_hip_alloc.argtypes = [ctypes.POINTER(vp), cl]
         L.pccl_hip_free.argtypes = [vp]
         L.pccl_hip_reduce_copy.argtypes = [ci, ci, ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, cl, vp]
@@ -127,6 +128,11 @@ def device_info():
     name = ctypes.create_string_buffer(256)
     _check(lib().pccl_hip_device_info(ctypes.byref(cus), ctypes.byref(mem), name, 256))
     return {"compute_units": cus.value, "hbm_bytes": mem.value, "name": name.value.decode()}
+
+
+def set_executor_id(ident):
+    """The registry id the device image's executor fields carry (pccl_hip_set_executor_id)."""
+    _check(lib().pccl_hip_set_executor_id(ident))
 
 
 def alloc(nbytes):

@@ -148,6 +148,73 @@ def test_config3_eight_input_reduce_full_size(hip, oracle, dtype, n_out, count):
     assert torch.equal(acc.to(ins[0].dtype), outs[0][:1 << 22])
 
 
+def _normal_on_device(torch, oracle, dtype, count, seed, stream, sigma):
+    """True N(0, sigma) input from the CPU checker's Box-Muller generator (threaded on the host, uploaded): the
+    values the configurations name, tails included, where _dev_random's "normal" is a bounded uniform."""
+    host = oracle.fill_normal(dtype, count, seed, stream, 0.0, sigma, nthreads=THREADS)
+    return host, torch.from_numpy(host.view(np.int16)).cuda()
+
+
+def test_config3_true_normal_inputs_full_size(hip, oracle):
+    """Configuration 3 on the inputs it names: 8 x bf16 N(0, 1) from seed 2, 64 Mi elements (128 MiB) each -> 1
+    output, and the f16 form with two outputs on a quarter of that."""
+    import torch
+    for dtype, n_out, count in (("bf16", 1, 1 << 26), ("f16", 2, 1 << 24)):
+        pairs = [_normal_on_device(torch, oracle, dtype, count, 2, k, 1.0) for k in range(8)]
+        h_ins, d_ins = [p[0] for p in pairs], [p[1] for p in pairs]
+        assert max(float(np.abs(oracle.widen(dtype, a[:1 << 22])).max()) for a in h_ins) > 4.5, "no tails: not a normal sample"
+        outs = [torch.zeros(count, dtype=torch.int16, device="cuda") for _ in range(n_out)]
+        hip.reduce_copy(dtype, "sum", d_ins, outs, count, _stream(torch))
+        torch.cuda.synchronize()
+        want = _expect(oracle, dtype, "sum", h_ins)
+        for j, o in enumerate(outs):
+            H.assert_bits_equal(o.cpu().numpy().view(np.uint16), want, "%s 8->%d output %d on N(0,1) inputs" % (dtype, n_out, j))
+        del pairs, h_ins, d_ins, outs
+
+
+def test_config2_true_normal_inputs_full_size(hip, oracle):
+    """Configuration 2 on the inputs it names: bf16 N(0, 1e-2) from seed 1, one rank's 14 ring steps over
+    32 MiB chunks, as 14 launches and as one launch of the queue executor; both against the CPU checker."""
+    import torch
+    W, ce = 8, 1 << 24
+    h_grad, grad = _normal_on_device(torch, oracle, "bf16", W * ce, 1, 0, 1e-2)
+    peers = [_normal_on_device(torch, oracle, "bf16", ce, 1, 1 + s, 1e-2) for s in range(W - 1)]
+    h_peers, d_peers = [p[0] for p in peers], [p[1] for p in peers]
+    h_result = np.zeros(W * ce, dtype=np.uint16)
+    h_send = None
+    for s in range(W - 1):
+        c = (W - 1 - s) % W
+        h_send = _expect(oracle, "bf16", "sum", [h_peers[s], h_grad[c * ce:(c + 1) * ce]])
+        h_result[c * ce:(c + 1) * ce] = h_send
+    for s in range(W - 1):
+        c = (W - s) % W
+        h_result[c * ce:(c + 1) * ce] = h_peers[s]
+    result = torch.zeros(W * ce, dtype=torch.int16, device="cuda")
+    send = torch.zeros(ce, dtype=torch.int16, device="cuda")
+    ops = []
+    for s in range(W - 1):
+        c = (W - 1 - s) % W
+        ops.append(dict(dtype="bf16", compute="sum", ins=[d_peers[s], grad[c * ce:(c + 1) * ce]],
+                        outs=[result[c * ce:(c + 1) * ce], send], count=ce, deps=[len(ops) - 1] if ops else []))
+    for s in range(W - 1):
+        c = (W - s) % W
+        ops.append(dict(dtype="bf16", compute="sum", ins=[d_peers[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce,
+                        deps=[s - 1] if s else []))
+    for o in ops:
+        hip.reduce_copy("bf16", "sum", o["ins"], o["outs"], ce, _stream(torch))
+    torch.cuda.synchronize()
+    H.assert_bits_equal(result.cpu().numpy().view(np.uint16), h_result, "14 launches, assembled 256 MiB result")
+    H.assert_bits_equal(send.cpu().numpy().view(np.uint16), h_send, "14 launches, send buffer")
+    result.zero_()
+    send.zero_()
+    g = hip.Graph(ops)
+    g.run(_stream(torch))
+    assert g.status(_stream(torch)) == (14, 14)
+    H.assert_bits_equal(result.cpu().numpy().view(np.uint16), h_result, "one queue launch, assembled 256 MiB result")
+    H.assert_bits_equal(send.cpu().numpy().view(np.uint16), h_send, "one queue launch, send buffer")
+    g.destroy()
+
+
 # forced members of the count list plus a log-uniform draw from [1, 2^28] (seed 3)
 FORCED = [1, 2, 3, 5, 7, 31, 127, 8191, 131071, 524287, (1 << 20) + 7, (1 << 24) - 3, (1 << 28) - 57, 1 << 28]
 

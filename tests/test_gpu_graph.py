@@ -219,6 +219,44 @@ def test_bounded_wait_aborts_cleanly(hip, oracle):
     g.destroy()
 
 
+def test_device_image_carries_the_executor_id(hip):
+    """RingBuffer::producer_ / consumer_ (include/base/operator.h:8-9) and OperationLayoutHeader::executor_type_
+    (:24), read back through the reference's offsets, hold the id given to pccl_hip_set_executor_id (the host
+    layer passes the registry id of "hip")."""
+    import ctypes as C
+    import torch
+    hipmemcpy = C.CDLL("libamdhip64.so").hipMemcpy
+    hipmemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+
+    def read(addr, n):
+        host = torch.empty(n, dtype=torch.uint8)
+        assert hipmemcpy(host.data_ptr(), addr, n, 2) == 0
+        return host.numpy()
+
+    x, y = H.DevBuf(torch, "f32", 4096, 0), H.DevBuf(torch, "f32", 4096, 0)
+    ops = [dict(dtype="f32", compute="sum", ins=[x.ptr], outs=[y.ptr], count=4096, deps=[])]
+    try:
+        from pccl_amd import engine
+        for ident in (0, 37, engine.type_id("hip")):
+            hip.set_executor_id(ident)
+            g = hip.Graph(ops)
+            layout = read(g.info()["device_layout"], 48)
+            operators = int(layout[16:24].view(np.uint64)[0])
+            queues = int(layout[32:40].view(np.uint64)[0])
+            assert int(layout[24:28].view(np.uint32)[0]) == 1 and int(layout[40:44].view(np.uint32)[0]) == 8
+            header = read(int(read(operators, 8).view(np.uint64)[0]), 32)
+            assert header[13] == ident, "executor_type_"
+            ring = read(int(read(queues, 8).view(np.uint64)[0]), 40)
+            assert ring[0] == ident and ring[1] == ident, "producer_ / consumer_"
+            g.destroy()
+        with pytest.raises(hip.PcclError):
+            hip.set_executor_id(256)
+    finally:
+        # what the host layer sets when it registers its executor (loading it does that)
+        from pccl_amd import engine
+        hip.set_executor_id(engine.type_id("hip"))
+
+
 # ---- signal ops: NOTIFY / GET_NOTIFIED ---------------------------------------------------------
 
 def _signal_ring_ops(world, size, signals_ptr, dev_in, dev_out, es=2, dtype="bf16"):
@@ -263,8 +301,8 @@ def _signal_ring_ops(world, size, signals_ptr, dev_in, dev_out, es=2, dtype="bf1
 
 @pytest.mark.parametrize("size,tile,own_rounds", [(3001, 0, None), (30001, 8192, "16"), (30001, 8192, "0")])
 def test_ring_allreduce_over_signal_words(hip, oracle, monkeypatch, size, tile, own_rounds):
-    """(Second and third case: more entries than workgroups, taken without tickets in several rounds
-    per workgroup, and by ticket.)"""
+    """(Second and third case: more entries than workgroups.  The entries of this graph wait for each other,
+    so they are drawn by ticket whatever PCCL_HIP_OWN_ENTRIES allows.)"""
     import torch
     if own_rounds is not None:
         monkeypatch.setenv("PCCL_HIP_OWN_ENTRIES", own_rounds)
@@ -684,13 +722,42 @@ def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, 
     g.destroy()
 
 
+@pytest.mark.parametrize("own_rounds", [None, "16", "0"])
+def test_independent_ops_taken_without_tickets(hip, oracle, monkeypatch, own_rounds):
+    """Entries that wait for no other entry of the graph are taken by workgroup number where they are few per
+    workgroup: one each (built-in), several rounds (PCCL_HIP_OWN_ENTRIES=16), or by ticket (=0).  Same bytes."""
+    import torch
+    if own_rounds is not None:
+        monkeypatch.setenv("PCCL_HIP_OWN_ENTRIES", own_rounds)
+    rng = np.random.default_rng(77)
+    n_ops = 700 if own_rounds is None else 3000
+    counts = [int(c) for c in rng.integers(1, 4000, size=n_ops)]   # at most 8 KB: one part each
+    total = sum(counts)
+    a, b = H.gen("bf16", total, 78, 0), H.gen("bf16", total, 78, 1)
+    da, db = H.DevBuf(torch, "bf16", total, 0, src=a), H.DevBuf(torch, "bf16", total, 0, src=b)
+    dz = H.DevBuf(torch, "bf16", total, 0)
+    ops, at = [], 0
+    for c in counts:
+        ops.append(dict(dtype="bf16", compute="sum", ins=[da.ptr + 2 * at, db.ptr + 2 * at], outs=[dz.ptr + 2 * at], count=c, deps=[]))
+        at += c
+    g = hip.Graph(ops)
+    info = g.info()
+    assert info["n_tiles"] == n_ops and (own_rounds is not None) == (info["n_tiles"] > info["n_workgroups"])
+    for _ in range(2):
+        dz.view().fill_(0xFF)
+        _run_and_check(torch, hip, g, n_ops)
+        H.assert_bits_equal(dz.download(), oracle.reduce("bf16", "sum", [a, b]), "independent ops, PCCL_HIP_OWN_ENTRIES=%s" % own_rounds)
+    assert dz.guards_intact()
+    g.destroy()
+
+
 @pytest.mark.parametrize("chains,size", [("0", 30_001), ("1", 30_001), ("0", 3_000_001)])
 def test_graph_beside_a_kernel_that_occupies_the_gpu(hip, oracle, monkeypatch, chains, size):
     """The drain's workgroups wait for each other inside one launch, so it needs its queues' workgroups
     resident.  With another stream's long elementwise kernels holding compute units at the same time the
     run must still complete every op (no bounded wait may give up), bit-exact: with every op queueing
-    its own entries (112 ops that wait for each other through the queue; one workgroup per entry at
-    the small size, tickets at the large one) and with the ring's steps chained."""
+    its own entries (112 ops that wait for each other through the queue, drawn by ticket) and with the
+    ring's steps chained (one workgroup per entry, by number: the chains' heads wait for nothing)."""
     import torch
     from pccl_amd import lang
     monkeypatch.setenv("PCCL_HIP_CHAINS", chains)

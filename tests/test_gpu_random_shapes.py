@@ -156,21 +156,19 @@ def test_accumulate_random(hip, oracle, restore_knobs):
 
 # ---- random programs over one pool of memory ------------------------------------------------
 
-def test_random_programs_over_one_pool_match_sequential_execution(hip, oracle):
-    """Programs whose ops alias each other's operands in every way the dependency analysis of
-    the queue executor distinguishes: the pool after the run must equal, bit for bit, the pool
-    after running the ops one by one on the CPU.  Each program runs twice (the second run
-    starts from the first one's results and re-uses the re-armed graph)."""
+def _run_pool_programs(hip, oracle, seeds, tile_auto=False):
+    """Bytes only: the pool after every run equals sequential execution on the CPU.  Returns how many
+    dependencies of each kind (whole-op, part by part) the executor reported."""
     import torch
     pool_elems = 2_000_000
     stream = torch.cuda.current_stream().cuda_stream
     kinds_seen = [0, 0]
-    for seed in range(6 * SCALE):
+    for seed in seeds:
         rng = np.random.default_rng(5000 + seed + SEED_SHIFT)
         prog = S.random_pool_program(rng, pool_elems, int(rng.integers(8, 60)))
         host = H.gen("f32", pool_elems, 777 + seed, 0, kind="uniform", lo=-1.0, hi=1.0)
         dev = H.DevBuf(torch, "f32", pool_elems, 0, src=host)
-        tile = [0, 0, 16384, 65536][seed % 4]
+        tile = hip.TILE_AUTO if tile_auto else [0, 0, 16384, 65536][seed % 4]
         g = hip.Graph([dict(dtype="f32", compute=o["compute"], count=o["count"], deps=o["deps"],
                             ins=[dev.ptr + 4 * r for r in o["ins"]], outs=[dev.ptr + 4 * r for r in o["outs"]])
                        for o in prog], tile_bytes=tile)
@@ -188,20 +186,26 @@ def test_random_programs_over_one_pool_match_sequential_execution(hip, oracle):
             H.assert_bits_equal(dev.download(), host, "seed %d run %d (%d ops, tile %d)" % (seed, run, len(prog), tile))
         assert dev.guards_intact()
         g.destroy()
-    # the sweep met both kinds of dependency often
+    return kinds_seen
+
+
+def test_random_programs_over_one_pool_match_sequential_execution(hip, oracle):
+    """Programs whose ops alias each other's operands in every way the dependency analysis of
+    the queue executor distinguishes: the pool after the run must equal, bit for bit, the pool
+    after running the ops one by one on the CPU.  Each program runs twice (the second run
+    starts from the first one's results and re-uses the re-armed graph)."""
+    kinds_seen = _run_pool_programs(hip, oracle, range(6 * SCALE))
+    # (plan shape, built-in settings only) the sweep met both kinds of dependency often
     assert min(kinds_seen) >= 20, kinds_seen
 
 
-def test_random_programs_with_dependencies_replaced_by_signal_words(hip, oracle):
-    """The same kind of program with about half of its dependency edges u -> v replaced by
-    NOTIFY(behind u) -> signal word -> GET_NOTIFIED(in front of v), a word per replaced edge: some of
-    those signal ops ride on their data op, some (a second NOTIFY behind the same op, a second wait in
-    front of it) queue entries of their own.  The pool must equal sequential execution, run after run."""
+def _run_signal_programs(hip, oracle, seeds):
+    """Bytes only.  Returns (signal ops carried by data ops, signal ops with entries of their own)."""
     import torch
     pool_elems = 1_000_000
     stream = torch.cuda.current_stream().cuda_stream
     carried_seen, own_seen = 0, 0
-    for seed in range(8 * SCALE):
+    for seed in seeds:
         rng = np.random.default_rng(8000 + seed + SEED_SHIFT)
         prog = S.random_pool_program(rng, pool_elems, int(rng.integers(6, 40)))
         host = H.gen("f32", pool_elems, 977 + seed, 0, kind="uniform", lo=-1.0, hi=1.0)
@@ -236,18 +240,25 @@ def test_random_programs_with_dependencies_replaced_by_signal_words(hip, oracle)
             H.assert_bits_equal(dev.download(), host, "seed %d run %d (%d ops, %d words)" % (seed, run, len(ops), n_words))
         assert dev.guards_intact()
         g.destroy()
-    assert carried_seen >= 20 and own_seen >= 5, (carried_seen, own_seen)
+    return carried_seen, own_seen
 
 
-def test_random_programs_with_dependencies_between_ops_that_share_no_bytes(hip, oracle):
-    """The same kind of program with extra dependencies that it does not need (to any earlier op): those
-    between ops cut alike are met part by part, and the ops reached through them must still be looked at
-    when a later op touches their bytes at another address.  The pool must equal sequential execution."""
+def test_random_programs_with_dependencies_replaced_by_signal_words(hip, oracle):
+    """The same kind of program with about half of its dependency edges u -> v replaced by
+    NOTIFY(behind u) -> signal word -> GET_NOTIFIED(in front of v), a word per replaced edge: some of
+    those signal ops ride on their data op, some (a second NOTIFY behind the same op, a second wait in
+    front of it) queue entries of their own.  The pool must equal sequential execution, run after run."""
+    carried_seen, own_seen = _run_signal_programs(hip, oracle, range(8 * SCALE))
+    assert carried_seen >= 20 and own_seen >= 5, (carried_seen, own_seen)   # (plan shape, built-in settings only)
+
+
+def _run_extra_edge_programs(hip, oracle, seeds):
+    """Bytes only.  Returns (extra dependencies added, dependencies the executor meets part by part)."""
     import torch
     pool_elems = 1_500_000
     stream = torch.cuda.current_stream().cuda_stream
     extra, part_wise = 0, 0
-    for seed in range(6 * SCALE):
+    for seed in seeds:
         rng = np.random.default_rng(6100 + seed + SEED_SHIFT)
         prog = S.random_pool_program(rng, pool_elems, int(rng.integers(8, 50)))
         for i, o in enumerate(prog):
@@ -273,4 +284,62 @@ def test_random_programs_with_dependencies_between_ops_that_share_no_bytes(hip, 
             H.assert_bits_equal(dev.download(), host, "seed %d run %d (%d ops)" % (seed, run, len(prog)))
         assert dev.guards_intact()
         g.destroy()
-    assert extra >= 50 and part_wise >= 20, (extra, part_wise)
+    return extra, part_wise
+
+
+def test_random_programs_with_dependencies_between_ops_that_share_no_bytes(hip, oracle):
+    """The same kind of program with extra dependencies that it does not need (to any earlier op): those
+    between ops cut alike are met part by part, and the ops reached through them must still be looked at
+    when a later op touches their bytes at another address.  The pool must equal sequential execution."""
+    extra, part_wise = _run_extra_edge_programs(hip, oracle, range(6 * SCALE))
+    assert extra >= 50 and part_wise >= 20, (extra, part_wise)   # (plan shape, built-in settings only)
+
+
+# ---- the same sweeps under every documented switch of the executor: bytes only ---------------------
+
+def _ring_through_the_queue(hip, oracle, world, size, seed, tile_auto=False):
+    """Ring all-reduce over resident ranks as one graph (its chunks run as chains where chains are on)."""
+    import torch
+    from pccl_amd import lang
+    stream = torch.cuda.current_stream().cuda_stream
+    ir, per_rank = lang.ring_allreduce(world, size, dtype="bf16")
+    low = ir.lower()
+    host_in = [H.gen("bf16", per_rank, seed, r) for r in range(world)]
+    bufs = {"in": [H.DevBuf(torch, "bf16", per_rank, 0, src=a) for a in host_in],
+            "out": [H.DevBuf(torch, "bf16", per_rank, 0) for _ in range(world)]}
+    outs = [np.zeros(per_rank, dtype=np.uint16) for _ in range(world)]
+    hb = {"in": host_in, "out": outs}
+    for o in low:
+        n = o["count"]
+        oracle.reduce_copy("bf16", "sum", [hb[b][r][e:e + n] for (b, r, e) in o["ins"]], [hb[b][r][e:e + n] for (b, r, e) in o["outs"]])
+    g = hip.Graph(lang.bind(low, lambda b, r, e: bufs[b][r].ptr + 2 * e), tile_bytes=hip.TILE_AUTO if tile_auto else 0)
+    for run in range(2):
+        for r in range(world):
+            bufs["out"][r].view().fill_(0xFF)
+        g.run(stream)
+        assert g.status(stream) == (len(low), len(low))
+        for r in range(world):
+            H.assert_bits_equal(bufs["out"][r].download(), outs[r], "ring %d x %d, run %d, rank %d" % (world, size, run, r))
+            assert bufs["out"][r].guards_intact()
+    g.destroy()
+
+
+KNOBS = [("PCCL_HIP_PLAN_LAUNCHES", "0"), ("PCCL_HIP_ORDER_EDGES", "0"), ("PCCL_HIP_CHAINS", "0"), ("PCCL_HIP_CHAINS", "1m"),
+         ("PCCL_HIP_CHAIN_BALANCE", "0"), ("PCCL_HIP_PART_DEPS", "0"), ("PCCL_HIP_FUSE_SIGNALS", "0"),
+         ("PCCL_HIP_OWN_ENTRIES", "0"), ("PCCL_HIP_OWN_ENTRIES", "16"), ("PCCL_HIP_ORDER_BLOCK", "0"), ("PCCL_HIP_ORDER_BLOCK", "1")]
+
+
+@pytest.mark.parametrize("name,value", KNOBS, ids=["%s=%s" % kv for kv in KNOBS])
+def test_random_programs_under_each_executor_switch(hip, oracle, monkeypatch, name, value):
+    """Every documented switch of the queue executor changes HOW a graph runs, never what it leaves in
+    memory: a short form of the three random-program sweeps, a ring all-reduce whose chunks chain, one of
+    uneven chunks, and graphs handed over with PCCL_HIP_TILE_AUTO, under each switch.  Bytes only; what the
+    plan looks like under a switch is nobody's business here."""
+    monkeypatch.setenv(name, value)
+    _run_pool_programs(hip, oracle, range(3))
+    _run_pool_programs(hip, oracle, range(3, 5), tile_auto=True)
+    _run_signal_programs(hip, oracle, range(3))
+    _run_extra_edge_programs(hip, oracle, range(3))
+    _ring_through_the_queue(hip, oracle, 8, 20_011, 3100)
+    _ring_through_the_queue(hip, oracle, 4, 300_007, 3101)
+    _ring_through_the_queue(hip, oracle, 4, 1_501, 3102, tile_auto=True)

@@ -319,3 +319,22 @@ def test_f64_fold_order_and_width(oracle):
                        ([np.float64(1e8), one, np.float64(-1e8)], one)):
         ins = [np.full(3, v, dtype=np.float64) for v in vals]
         H.assert_bits_equal(oracle.reduce("f64", "sum", ins), np.full(3, want, dtype=np.float64), "f64 %s" % (vals,))
+
+
+def test_normal_generator_threaded_form_and_shape(oracle):
+    """fill_normal over several threads gives the bytes of the scalar loop (the generator is counter-based), and
+    what it gives is a normal sample: mean, standard deviation, and tails at the rate the distribution has
+    (a bounded stand-in such as a scaled uniform has none beyond 1.74 sigma)."""
+    n = 1 << 20
+    for dtype, sigma in (("f32", 1.0), ("bf16", 1e-2), ("f16", 1.0)):
+        one = oracle.fill_normal(dtype, n, 9, 4, 0.0, sigma)
+        many = oracle.fill_normal(dtype, n, 9, 4, 0.0, sigma, nthreads=5)
+        assert np.array_equal(one, many)
+        z = (oracle.widen(dtype, one) if dtype != "f32" else one).astype(np.float64) / sigma
+        assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3
+        for k, rate in ((2.0, 4.55e-2), (3.0, 2.70e-3), (4.0, 6.33e-5)):
+            seen = float((np.abs(z) > k).mean())
+            assert 0.7 * rate < seen < 1.3 * rate, "%s: P(|z| > %g) = %g, a normal has %g" % (dtype, k, seen, rate)
+    # another stream, another seed: other values
+    assert not np.array_equal(oracle.fill_normal("f32", 64, 9, 4), oracle.fill_normal("f32", 64, 9, 5))
+    assert not np.array_equal(oracle.fill_normal("f32", 64, 9, 4), oracle.fill_normal("f32", 64, 10, 4))

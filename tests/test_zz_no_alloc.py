@@ -78,3 +78,60 @@ def test_static_arena_refuses_a_graph_beyond_its_size_and_works_afterwards(hip, 
     assert hip.graph_run_static([dict(dtype="f32", compute="sum", ins=[x.ptr], outs=[y.ptr], count=n)], stream) == (1, 1)
     H.assert_bits_equal(y.download(), x.download(), "copy through the fixed array after a refused call")
     assert hip.graph_run_static([], stream) == (0, 0)
+
+
+def test_a_run_that_gave_up_is_reported_by_the_next_call_and_the_one_after_runs_afresh(hip, oracle, monkeypatch):
+    """A caller that passes no counters launches a graph whose GET_NOTIFIED nobody satisfies: the wait gives up
+    inside the kernel (spin limit set from the host, every workgroup leaves normally).  The next call, same ops and
+    again without counters, must not launch onto the abandoned state and return PCCL_OK with the outputs
+    untouched: it reports PCCL_ERR_GRAPH.  The call after that, with the word satisfied, is a correct fresh run."""
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    monkeypatch.setenv("PCCL_HIP_SPIN_LIMIT_US", "20000")
+    n = 50_000
+    src = H.gen("f32", n, 504, 0)
+    x = H.DevBuf(torch, "f32", n, 0, src=src)
+    y = H.DevBuf(torch, "f32", n, 0, fill=0x5A)
+    word = torch.zeros(4, dtype=torch.int32, device="cuda")
+    ops = [dict(primitive=hip.GET_NOTIFIED, signal=word.data_ptr(), value=1, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[x.ptr], outs=[y.ptr], count=n, deps=[0])]
+    assert hip.graph_run_static(ops, stream, wait=False) is None      # gives up after 20 ms, unnoticed
+    with pytest.raises(hip.PcclError) as e:
+        hip.graph_run_static(ops, stream, wait=False)
+    assert e.value.code == hip.ERR_GRAPH and "gave up" in str(e.value)
+    torch.cuda.synchronize()
+    assert bool((y.view() == 0x5A).all()), "nothing may have been copied: the signal never came"
+    word.fill_(0x7fff0000)   # ahead of every run's signal base: the wait is satisfied at once
+    torch.cuda.synchronize()
+    assert hip.graph_run_static(ops, stream) == (2, 2)
+    H.assert_bits_equal(y.download(), src, "fresh run after the abandoned one")
+    assert y.guards_intact(0x5A)
+    # ... and a caller that does pass counters hears of a wait that gave up in the same call
+    word.zero_()
+    torch.cuda.synchronize()
+    with pytest.raises(hip.PcclError) as e:
+        hip.graph_run_static(ops, stream)
+    assert e.value.code == hip.ERR_GRAPH
+    monkeypatch.delenv("PCCL_HIP_SPIN_LIMIT_US")
+    assert hip.graph_run_static([dict(dtype="f32", compute="sum", ins=[x.ptr], outs=[y.ptr], count=n)], stream) == (1, 1)
+
+
+def test_the_same_ops_on_another_stream_wait_for_the_run_before(hip, oracle):
+    """Two calls with the same ops on two streams, nothing between them: the second waits for the first run
+    (they share the one array) and both leave the checker's result."""
+    import torch
+    n = 1 << 22
+    a, b = H.gen("f32", n, 505, 0), H.gen("f32", n, 505, 1)
+    want = oracle.reduce("f32", "sum", [a, b])
+    x, y = H.DevBuf(torch, "f32", n, 0, src=a), H.DevBuf(torch, "f32", n, 0, src=b)
+    z = H.DevBuf(torch, "f32", n, 0, fill=0x5A)
+    w = H.DevBuf(torch, "f32", n, 0, fill=0x5A)
+    ops = [dict(dtype="f32", compute="sum", ins=[x.ptr, y.ptr], outs=[z.ptr], count=n, deps=[]),
+           dict(dtype="f32", compute="sum", ins=[z.ptr], outs=[w.ptr], count=n, deps=[0])]
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert hip.graph_run_static(ops, s1.cuda_stream, wait=False) is None
+    assert hip.graph_run_static(ops, s2.cuda_stream) == (2, 2)
+    torch.cuda.synchronize()
+    H.assert_bits_equal(z.download(), want, "fold")
+    H.assert_bits_equal(w.download(), want, "copy behind it")
