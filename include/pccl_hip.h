@@ -188,7 +188,10 @@ typedef struct pccl_op_desc {
  * as one of at most two inputs; an output that a later op of the same such chain writes again at the
  * same address is then not stored by the earlier op: nothing could read it).  A level of the graph whose entries start such chains is cut by
  * the built-in choice into the smallest parts (from 8 KiB) with which its entries fit the resident
- * workgroups once.  Results, graph_status and graph_rebind are as without chains;
+ * workgroups once.  In a chain that does not run in one pass, a COPY whose input is output 0 of the op before it is not run at
+ * all: that op stores the copy's outputs as further outputs of its own (a slice folded 8 -> 1 and then copied 1 -> 7 is stored
+ * as 8 -> 8), provided they fit one op and overlap none of its operands at another address; PCCL_HIP_FOLD_COPIES=0 runs it.
+ * Results, graph_status and graph_rebind are as without chains;
  * graph_info's n_tiles and the timeline count the entries that are queued.  PCCL_HIP_CHAINS=0
  * switches chains off.
  * Signal ops that stand alone beside one data op ride on it: a NOTIFY whose only dependency is a
@@ -257,7 +260,8 @@ int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int
  * (else 1); for an op that starts a chain 1 if the chain runs in one pass with the value kept in
  * registers, for another op of such a chain the index of the input that is its predecessor's
  * output 0; and, for an op that starts a one-pass chain, the first of the chain's rows in the
- * executor's operand table.  Touches no device. */
+ * executor's operand table.  In a chain that does not run in one pass the third int of a COPY that the op before it stores
+ * (see graph_create) is 2.  Touches no device. */
 int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, int forward_elem_bytes, int *words);
 
 /* Which signal ops of a graph ride on data ops (no counterpart in the reference; touches no device):

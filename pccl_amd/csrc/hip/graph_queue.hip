@@ -508,8 +508,9 @@ std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::ve
   // forward_elem_bytes: element size of the kernel instance's dtype if it has the one-pass code, else 0.
   // A chain of copies may have another element size than the graph's REDUCE ops (a copy moves bytes
   // of its own dtype): such a chain goes through memory, where every op is run by its own rule.
-  bool on = true, forward_on = forward_elem_bytes > 0;
+  bool on = true, forward_on = forward_elem_bytes > 0, fold_copies = true;
   if (const char *env = getenv("PCCL_HIP_CHAINS")) on = env[0] != '0', forward_on = forward_on && (env[0] != '1' || env[1] != 'm');  // "1m": through memory only
+  if (const char *env = getenv("PCCL_HIP_FOLD_COPIES")) fold_copies = env[0] != '0';
   auto is_data = [&](int i) { return ops[i].primitive != PCCL_NOTIFY && ops[i].primitive != PCCL_GET_NOTIFIED; };
   auto bytes_of = [&](int i) { return (uintptr_t)ops[i].count * (uintptr_t)elem_bytes(ops[i].dtype); };
   size_t at = 0;
@@ -582,6 +583,35 @@ std::vector<int> plan_chains(const std::vector<pccl_op_desc> &ops, const std::ve
       words[(size_t)kChainWords * h + kChainRow] = listed;  // first of its rows in the chain table (fill_chain_table)
       listed += (int)steps.size();
       for (size_t s = 1; s < steps.size(); ++s) words[(size_t)kChainWords * steps[s] + kChainForward] = fed[s];
+    } else if (fold_copies) {
+      // A chain that runs through memory: a COPY of the previous op's output 0 is not run at all, the
+      // previous op stores the copy's outputs as further outputs of its own (what the fold of an
+      // all-reduce slice followed by its broadcast copy is: 8 -> 1 then 1 -> 7 becomes 8 -> 8, with no
+      // wait for the stores, barrier and read-back between the two).  The copy's outputs must be new
+      // to the previous op: none of them may overlap one of its operands at another address (the lanes
+      // of a part would write what other lanes still have to read), and together they fit one op.
+      bool prev_folded = false;
+      for (size_t s = 1; s < steps.size(); ++s) {
+        const pccl_op_desc &A = ops[steps[s - 1]], &B = ops[steps[s]];
+        bool fold = !prev_folded && B.n_in == 1 && B.ins[0] == A.outs[0] && A.n_out + B.n_out <= PCCL_MAX_OUTPUTS;
+        for (int k = 0; fold && k < B.n_out; ++k) {
+          const uintptr_t y = (uintptr_t)B.outs[k];
+          for (int j = 0; fold && j < A.n_in; ++j) {
+            const uintptr_t x = (uintptr_t)A.ins[j];
+            if (x != y && x < y + len && y < x + len) fold = false;
+          }
+          for (int j = 0; fold && j < A.n_out; ++j) {
+            const uintptr_t x = (uintptr_t)A.outs[j];
+            if (x != y && x < y + len && y < x + len) fold = false;
+          }
+          for (int j = 0; fold && j < k; ++j) {
+            const uintptr_t x = (uintptr_t)B.outs[j];
+            if (x != y && x < y + len && y < x + len) fold = false;
+          }
+        }
+        if (fold) words[(size_t)kChainWords * steps[s] + kChainForward] = kChainFolded;
+        prev_folded = fold;
+      }
     }
   }
   return words;

@@ -74,7 +74,9 @@ constexpr int kChainNext = 0;     // the op that runs behind this one, or -1
 constexpr int kChainLength = 1;   // for the op a chain starts with: ops in it (1 for an op outside any chain)
 constexpr int kChainForward = 2;  // head: 1 if the whole chain runs in one pass with values handed on in registers
                                   // (run_chain_forward); another op of such a chain: which of its inputs is the
-                                  // previous op's output 0
+                                  // previous op's output 0; an op of a chain that runs through memory: kChainFolded
+                                  // if it is a COPY of the previous op's output 0 whose outputs that op stores itself
+constexpr int kChainFolded = 2;
 constexpr int kChainRow = 3;      // head of a forward chain: its first row in GraphControl::chain_table
 constexpr int kMaxForwardSteps = 16;
 // A queue entry: op uid | part << 32 | (op heads a chain) << 51.  The flag saves every other entry the
@@ -164,10 +166,15 @@ __device__ __forceinline__ void run_part_body(const RcOperands &a, long head, lo
 }
 
 // SLIM: only the variant that tolerates unaligned streams (keeps the any-dtype instance small).
+// `more`: null, or the payload of a COPY that is chained behind this op and whose input is this op's
+// output 0 (kChainFolded): its outputs are stored by this op as further outputs, and the copy itself is
+// not run.  The value goes from registers to every destination; nothing is written, waited for and read
+// back between the two ops.
 template <class D, class Op, int NIN, bool SLIM = false>
-__device__ __forceinline__ void run_part_nin(const pccl_op_payload *pl, long lo, long count) {
+__device__ __forceinline__ void run_part_nin(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
   RcOperands a;
-  a.n_out = pl->n_out_;
+  const int own_out = pl->n_out_;
+  a.n_out = own_out + (more ? more->n_out_ : 0);
   a.out[0] = (char *)pl->chunks_[NIN].addr_ + lo * D::kElemBytes;
   // bits in which some stream's address differs from output 0's
   unsigned long long mis = 0;
@@ -179,7 +186,8 @@ __device__ __forceinline__ void run_part_nin(const pccl_op_payload *pl, long lo,
 #pragma unroll
   for (int j = 1; j < PCCL_MAX_OUTPUTS; ++j)
     if (j < a.n_out) {
-      a.out[j] = (char *)pl->chunks_[NIN + j].addr_ + lo * D::kElemBytes;
+      const void *to = j < own_out ? pl->chunks_[NIN + j].addr_ : more->chunks_[1 + j - own_out].addr_;
+      a.out[j] = (char *)to + lo * D::kElemBytes;
       mis |= (unsigned long long)a.out[j] ^ (unsigned long long)a.out[0];
     }
   // same peel as the direct launch: make output 0 start on 16 bytes; the other
@@ -198,31 +206,31 @@ __device__ __forceinline__ void run_part_nin(const pccl_op_payload *pl, long lo,
 
 // COPY moves bytes, and its element size is its own, not that of the graph's REDUCE ops:
 // it runs as a copy of 1-byte units.
-__device__ __forceinline__ void run_copy_part(const pccl_op_payload *pl, long lo, long count) {
+__device__ __forceinline__ void run_copy_part(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
   const int dt = pl->chunks_[0].dtype_;
   const long units = dt == PCCL_F64 ? 8 : (dt == PCCL_F32 || dt == PCCL_I32 || dt == PCCL_U32) ? 4
                      : (dt == PCCL_BF16 || dt == PCCL_F16) ? 2 : 1;
-  run_part_nin<Dtype<PCCL_F8E4M3>, OpSum, 1>(pl, lo * units, count * units);
+  run_part_nin<Dtype<PCCL_F8E4M3>, OpSum, 1>(pl, more, lo * units, count * units);
 }
 
 template <int DT, class Op, bool SLIM = false>
-__device__ __forceinline__ void run_reduce_part(const pccl_op_payload *pl, long lo, long count) {
+__device__ __forceinline__ void run_reduce_part(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
   typedef Dtype<DT> D;
   switch (pl->n_in_) {
-    case 2: run_part_nin<D, Op, 2, SLIM>(pl, lo, count); break;
-    case 3: run_part_nin<D, Op, 3, SLIM>(pl, lo, count); break;
-    case 4: run_part_nin<D, Op, 4, SLIM>(pl, lo, count); break;
-    case 5: run_part_nin<D, Op, 5, SLIM>(pl, lo, count); break;
-    case 6: run_part_nin<D, Op, 6, SLIM>(pl, lo, count); break;
-    case 7: run_part_nin<D, Op, 7, SLIM>(pl, lo, count); break;
-    default: run_part_nin<D, Op, 8, SLIM>(pl, lo, count); break;
+    case 2: run_part_nin<D, Op, 2, SLIM>(pl, more, lo, count); break;
+    case 3: run_part_nin<D, Op, 3, SLIM>(pl, more, lo, count); break;
+    case 4: run_part_nin<D, Op, 4, SLIM>(pl, more, lo, count); break;
+    case 5: run_part_nin<D, Op, 5, SLIM>(pl, more, lo, count); break;
+    case 6: run_part_nin<D, Op, 6, SLIM>(pl, more, lo, count); break;
+    case 7: run_part_nin<D, Op, 7, SLIM>(pl, more, lo, count); break;
+    default: run_part_nin<D, Op, 8, SLIM>(pl, more, lo, count); break;
   }
 }
 
 template <int DT, class Op>
-__device__ __forceinline__ void run_part(const pccl_op_payload *pl, long lo, long count) {
-  if (pl->n_in_ == 1) run_copy_part(pl, lo, count);
-  else run_reduce_part<DT, Op>(pl, lo, count);
+__device__ __forceinline__ void run_part(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
+  if (pl->n_in_ == 1) run_copy_part(pl, more, lo, count);
+  else run_reduce_part<DT, Op>(pl, more, lo, count);
 }
 
 // A graph whose REDUCE ops do not share one (dtype, compute) pair runs the kernel instance
@@ -234,18 +242,18 @@ constexpr int kAnyDtype = -1;
 // Not inlined: one function per dtype keeps the any-dtype kernel a small caller of eight
 // mid-sized functions (as one flat function its compilation took minutes).
 template <int DT>
-__device__ __attribute__((noinline)) void run_part_any_compute(const pccl_op_payload *pl, long lo, long count) {
+__device__ __attribute__((noinline)) void run_part_any_compute(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
   switch (pl->compute_) {
-    case PCCL_SUM: run_reduce_part<DT, OpSum, true>(pl, lo, count); break;
-    case PCCL_PROD: run_reduce_part<DT, OpProd, true>(pl, lo, count); break;
-    case PCCL_MIN: run_reduce_part<DT, OpMin, true>(pl, lo, count); break;
-    default: run_reduce_part<DT, OpMax, true>(pl, lo, count); break;
+    case PCCL_SUM: run_reduce_part<DT, OpSum, true>(pl, more, lo, count); break;
+    case PCCL_PROD: run_reduce_part<DT, OpProd, true>(pl, more, lo, count); break;
+    case PCCL_MIN: run_reduce_part<DT, OpMin, true>(pl, more, lo, count); break;
+    default: run_reduce_part<DT, OpMax, true>(pl, more, lo, count); break;
   }
 }
 
-__device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, long lo, long count) {
+__device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, const pccl_op_payload *more, long lo, long count) {
   if (pl->n_in_ == 1) {
-    run_copy_part(pl, lo, count);
+    run_copy_part(pl, more, lo, count);
     return;
   }
   const int dt = pl->chunks_[0].dtype_;
@@ -255,14 +263,14 @@ __device__ __forceinline__ void run_part_any(const pccl_op_payload *pl, long lo,
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 0\n\ts_nop 1" ::: "memory");
   }
   switch (dt) {
-    case PCCL_F32: run_part_any_compute<PCCL_F32>(pl, lo, count); break;
-    case PCCL_I32: run_part_any_compute<PCCL_I32>(pl, lo, count); break;
-    case PCCL_BF16: run_part_any_compute<PCCL_BF16>(pl, lo, count); break;
-    case PCCL_F16: run_part_any_compute<PCCL_F16>(pl, lo, count); break;
-    case PCCL_F8E4M3: run_part_any_compute<PCCL_F8E4M3>(pl, lo, count); break;
-    case PCCL_F8E5M2: run_part_any_compute<PCCL_F8E5M2>(pl, lo, count); break;
-    case PCCL_F64: run_part_any_compute<PCCL_F64>(pl, lo, count); break;
-    default: run_part_any_compute<PCCL_U32>(pl, lo, count); break;
+    case PCCL_F32: run_part_any_compute<PCCL_F32>(pl, more, lo, count); break;
+    case PCCL_I32: run_part_any_compute<PCCL_I32>(pl, more, lo, count); break;
+    case PCCL_BF16: run_part_any_compute<PCCL_BF16>(pl, more, lo, count); break;
+    case PCCL_F16: run_part_any_compute<PCCL_F16>(pl, more, lo, count); break;
+    case PCCL_F8E4M3: run_part_any_compute<PCCL_F8E4M3>(pl, more, lo, count); break;
+    case PCCL_F8E5M2: run_part_any_compute<PCCL_F8E5M2>(pl, more, lo, count); break;
+    case PCCL_F64: run_part_any_compute<PCCL_F64>(pl, more, lo, count); break;
+    default: run_part_any_compute<PCCL_U32>(pl, more, lo, count); break;
   }
 }
 
@@ -801,8 +809,14 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         // (One call site for both: a second inlined copy of run_part cost the kernel its registers.)
         const pccl_op_payload *step = pl;
         for (int next = chain_next;;) {
-          if constexpr (DT == kAnyDtype) run_part_any(step, lo, n);
-          else run_part<DT, Op>(step, lo, n);
+          // a COPY of this op's output 0 right behind it: this op stores the copy's outputs too (run_part_nin)
+          const pccl_op_payload *more = nullptr;
+          if (next >= 0 && g.chain[kChainWords * next + kChainForward] == kChainFolded) {
+            more = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
+            next = g.chain[kChainWords * next + kChainNext];
+          }
+          if constexpr (DT == kAnyDtype) run_part_any(step, more, lo, n);
+          else run_part<DT, Op>(step, more, lo, n);
           if (next < 0) break;
           settle_stores();
           __syncthreads();

@@ -86,6 +86,45 @@ def test_one_pass_needs_the_predecessors_output_as_an_input_and_no_other_look_at
     assert hip.plan_chains(ops, [1, 1], ES)[0][2] == 0
 
 
+def test_a_copy_of_the_previous_ops_output_folds_into_that_op_in_a_chain_through_memory():
+    """8 -> 1 followed by the copy 1 -> 7 of its result (a slice of a one-exchange all-reduce): the chain cannot
+    run in one pass (eight inputs), so it goes through memory, and the copy is marked as folded (third word 2):
+    the fold stores the copy's outputs itself.  Not when the outputs would not fit one op, overlap an operand of
+    the fold at a shift, or the copy reads another output than output 0."""
+    ins = [buf(k) for k in range(8)]
+    t = buf(8)
+    outs = [buf(9 + k) for k in range(7)]
+    ops = [op(ins, [t], []), op([t], outs, [0])]
+    plan = hip.plan_chains(ops, [1, 1], ES)
+    assert plan[0][0] == 1 and plan[0][1] == 2 and plan[0][2] == 0 and plan[1][2] == 2
+    # too many outputs for one op (2 + 7 > 8)
+    ops = [op(ins, [t, buf(20)], []), op([t], outs, [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[1][2] == 0
+    # a copy output overlapping an input of the fold 16 elements further on
+    ops = [op(ins, [t], []), op([t], [ins[3] + 16 * ES], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[1][2] == 0
+    # ... at the same address it is the in-place case, pack by pack: folded
+    ops = [op(ins, [t], []), op([t], [ins[3]], [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[1][2] == 2
+    # the copy reads output 1, not output 0
+    ops = [op(ins, [buf(20), t], []), op([t], outs, [0])]
+    assert hip.plan_chains(ops, [1, 1], ES)[1][2] == 0
+    # a second copy behind a folded one runs by itself (its source is not the op before it that runs), a third folds again
+    u, v, w = buf(30), buf(31), buf(32)
+    ops = [op(ins, [t], []), op([t], [u], [0]), op([u], [v], [1]), op([v], [w], [2])]
+    plan = hip.plan_chains(ops, [1, 1, 1, 1], ES)
+    assert [p[0] for p in plan] == [1, 2, 3, -1] and [p[2] for p in plan] == [0, 2, 0, 2]
+    # many parts: folded where part p of the copy needs only part p of the fold
+    n = 100000
+    big = [buf(k, n) for k in range(12)]
+    ops = [op(big[:3], [big[3]], [], count=n), op([big[3]], big[4:6], [0], count=n)]
+    assert hip.plan_chains(ops, [8, 8], ES)[1][2] == 2
+    # (a two-input first op with such a copy behind it runs in one pass instead: nothing to fold)
+    ops = [op(big[:2], [big[3]], [], count=n), op([big[3]], big[4:6], [0], count=n)]
+    plan = hip.plan_chains(ops, [8, 8], ES)
+    assert plan[0][2] == 1 and plan[1][2] == 0
+
+
 def test_outputs_of_a_one_pass_chain_may_coincide_but_not_overlap_at_a_shift():
     a, b, c, t, u = (buf(k) for k in range(5))
     same = [op([a, b], [t], []), op([t, c], [u], [0]), op([u], [t], [1])]          # writes t again, same address

@@ -132,6 +132,42 @@ def test_chain_that_reads_what_it_wrote_earlier_goes_through_memory(hip, oracle)
         g.destroy()
 
 
+@pytest.mark.parametrize("fold", ["1", "0"])
+def test_copy_of_the_previous_ops_output_is_stored_by_that_op(hip, oracle, monkeypatch, fold):
+    """t = fold of 3..8 inputs;  v0..v6 = copy(t);  w = copy(v0);  x = copy(w): the chain goes through memory (more than
+    two inputs), the first copy's outputs are stored by the fold itself, the second copy runs by itself, the third
+    is stored by the second.  Ragged counts, operands off the 16-byte grid, one part and several;
+    PCCL_HIP_FOLD_COPIES=0 runs every op by itself.  Same bytes either way."""
+    import torch
+    monkeypatch.setenv("PCCL_HIP_FOLD_COPIES", fold)
+    for dtype, compute, n_in, n_copy, count, offset, tile in (("bf16", "sum", 8, 7, 300_007, 0, 0), ("f32", "max", 3, 5, 70_001, 4, 16 << 10),
+                                                              ("f16", "prod", 5, 3, 1_000_003, 6, 64 << 10), ("i32", "sum", 8, 7, 4_099, 12, 0),
+                                                              ("f8e5m2", "sum", 4, 4, 250_001, 3, 0), ("f64", "min", 6, 2, 65_537, 8, 0)):
+        pool = Pool(torch, dtype)
+        names_in = ["in%d" % k for k in range(n_in)]
+        for k, n in enumerate(names_in):
+            src = H.gen(dtype, count, 930, k, kind="uniform", lo=0.5, hi=2.0) if compute == "prod" else H.gen(dtype, count, 930, k)
+            pool.add(n, count, offset if k % 2 else 0, src=src)
+        copies = ["v%d" % k for k in range(n_copy)]
+        for k, n in enumerate(["t"] + copies + ["w", "x"]):
+            pool.add(n, count, (offset * (k % 3)) % 64)
+        ops = [dict(compute=compute, ins=names_in, outs=["t"], count=count, deps=[]),
+               dict(compute=compute, ins=["t"], outs=copies, count=count, deps=[0]),
+               dict(compute=compute, ins=["v0"], outs=["w"], count=count, deps=[1]),
+               dict(compute=compute, ins=["w"], outs=["x"], count=count, deps=[2])]
+        oracle.run_ops(pool.ops_for(ops, "host"))
+        bound = pool.ops_for(ops, "dev")
+        plan = hip.plan_chains(bound, [1] * 4, H.ELEM_BYTES[dtype])
+        assert [p[2] for p in plan] == ([0, 2, 0, 2] if fold == "1" else [0, 0, 0, 0])
+        g = hip.Graph(bound, tile_bytes=tile)
+        for run in range(2):
+            for n in ["t", "w", "x"] + copies:
+                pool.dev[n].view().fill_(0xFF)
+            _run(torch, hip, g, 4)
+            pool.check(["t", "w", "x"] + copies, "%s %s %d -> 1 -> %d, count %d, run %d" % (dtype, compute, n_in, n_copy, count, run))
+        g.destroy()
+
+
 def test_mixed_computes_and_more_ops_than_one_pass_holds(hip, oracle):
     """x1 = x0 + a, x2 = max(x1, b), x3 = x2 * c, ... 20 ops in a row: ops that do not share one
     fold run in the kernel instance that picks the fold per op, which takes chains through memory;
