@@ -612,6 +612,23 @@ def main():
                         full["8_ranks_x_%d_MiB" % per_rank_mib]["linked_by_signal_words_only"] = dict(
                             stats(ts), ops=len(lows), queue_entries=gs.info()["n_tiles"])
                         gs.destroy()
+                        # ... and with signals of a word per part of the chunk (schedule format version 2): a rank
+                        # starts on part p of a step as soon as its neighbour has finished part p of the step before
+                        K = 8 if per_rank_mib <= 1 else 32
+                        irp, _ = lang.ring_allreduce_signalled(8, (per_rank_mib << 20) // 2 // 8, dtype="bf16", signal_parts=K)
+                        lowp = irp.lower()
+                        words = torch.zeros(256, dtype=torch.int32, device="cuda")
+                        for r in range(8):
+                            rb["out"][r].zero_()
+                        gp = hip.Graph(lang.bind(lowp, lambda b, r, e: rb[b][r].data_ptr() + 2 * e, signals=words.data_ptr()))
+                        tp = event_times_us(torch, lambda: gp.run(stream), 20, 3)
+                        done, total = gp.status(stream)
+                        assert done == total == len(lowp)
+                        for r in range(8):
+                            assert torch.equal(rb["out"][r], first), "the ring linked by per-part signals differs from the ring linked by dependencies"
+                        full["8_ranks_x_%d_MiB" % per_rank_mib]["linked_by_signal_words_only"]["a_word_per_part"] = dict(
+                            stats(tp), words_per_signal=K, ops=len(lowp), queue_entries=gp.info()["n_tiles"])
+                        gp.destroy()
                     del rb
                 full["note"] = ("GBps_median counts the algorithmic bytes of the 112 ops; the 14 ops of a chunk run as one chain that keeps "
                                 "the value in registers and stores only what the chain does not overwrite itself: bytes_moved / GBps_moved_median")

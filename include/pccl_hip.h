@@ -150,7 +150,17 @@ int pccl_hip_set_rotation(int rotate);
  *   GET_NOTIFIED  n_in 1, n_out 0: ins[0] = signal word, count = value; it completes
  *                 when (int)(word - (signal_base + value)) >= 0 (bounded wait).
  * signal_base = run number << 16 (pccl_hip_graph_next_signal_base), so a word left over
- * from an earlier run never satisfies a wait of a later one. */
+ * from an earlier run never satisfies a wait of a later one.
+ * Signals per part (signal_parts = K >= 2; 0 and 1 mean the one word above): the signal is K consecutive
+ * 32-bit words, word p standing for part p of the data it announces, the data cut into K parts by the
+ * rule that both sides know (part p = elements [p * per, min((p + 1) * per, count)), per =
+ * ceil(count / K) rounded up to 64).  A NOTIFY whose only dependency is one COPY / REDUCE makes the
+ * executor cut that op into exactly K parts, and whoever completes part p stores word p; a GET_NOTIFIED
+ * that one COPY / REDUCE alone depends on makes that op K parts, and its part p polls word p only.  So a
+ * consumer starts on the first part while the producer is still working on the others: a ring whose
+ * ranks are linked by such pairs streams instead of stopping at every step.  (An op that would carry
+ * signals of two different K carries the first; a per-part signal op that stands alone stores, or waits
+ * for, all K words.)  Both ends of a pair must name the same K. */
 typedef struct pccl_op_desc {
   int op_uid;                          /* dense 0..n_ops-1, chunk.py:82-83           */
   unsigned char primitive;             /* enum pccl_primitive                         */
@@ -158,7 +168,8 @@ typedef struct pccl_op_desc {
   unsigned char compute;               /* enum pccl_compute                           */
   unsigned char n_in;                  /* 1..8                                        */
   unsigned char n_out;                 /* 1..8                                        */
-  unsigned char reserved[3];
+  unsigned char reserved;
+  unsigned short signal_parts;         /* NOTIFY / GET_NOTIFIED: words of the signal (see above); else 0 */
   const void *ins[PCCL_MAX_INPUTS];
   void *outs[PCCL_MAX_OUTPUTS];
   long count;                          /* elements per operand                        */
@@ -267,8 +278,10 @@ int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, i
 /* Which signal ops of a graph ride on data ops (no counterpart in the reference; touches no device):
  * carrier[i] = the COPY / REDUCE op that stores NOTIFY i when it completes, or whose parts poll
  * GET_NOTIFIED i before they start; -1 for every other op.  The rule is stated at
- * pccl_hip_graph_create; it looks at kinds and dependency lists only. */
-int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier);
+ * pccl_hip_graph_create; it looks at kinds, dependency lists and signal_parts only.
+ * parts (may be NULL): for a signal op that is carried part by part (signal_parts >= 2, see pccl_op_desc)
+ * its K; for the data op that carries such signals the K it is cut into; 0 for every other op. */
+int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier, int *parts);
 
 /* Device address of the GraphBufferLayout and launch facts, for inspection: n_tiles = queue entries
  * (parts of the ops that queue entries; ops that run behind another op in a chain queue none), or the

@@ -134,6 +134,7 @@ struct Graph {
   std::vector<int> eff_deps;
   std::vector<int> fused_into;             // per op: the data op that carries this signal op, or -1
   std::vector<int> wait_of, notify_of;     // per op: the GET_NOTIFIED / NOTIFY it carries, or -1
+  std::vector<int> signal_cut;             // per op: K if it carries signals of a word per part (it is then cut into K parts), else 0
   std::vector<long> user_dep_to_eff;       // per dependency as the caller listed them: its place among eff's, or -1
   size_t fuse_table_off = 0;               // arena offset of the carried signals' table (behind the chain table)
   std::vector<int> fixed_parts;            // build_graph: cut the ops like this instead of choosing (a rebuild in place:
@@ -391,6 +392,14 @@ void fuse_signals(Graph *G) {
   G->fused_into.assign(n, -1);
   G->wait_of.assign(n, -1);
   G->notify_of.assign(n, -1);
+  G->signal_cut.assign(n, 0);
+  // A signal of a word per part (signal_parts = K >= 2) rides on a data op only if the op can be cut
+  // into exactly K parts: it has no such signal yet, or one of the same K.
+  auto words_of = [&](int v) { return user[v].signal_parts >= 2 ? (int)user[v].signal_parts : 0; };
+  auto cut_allows = [&](int data_op, int v) {
+    const int k = words_of(v);
+    return k == 0 || G->signal_cut[data_op] == 0 || G->signal_cut[data_op] == k;
+  };
   bool on = true;
   if (const char *env = getenv("PCCL_HIP_FUSE_SIGNALS")) on = env[0] != '0';
   std::vector<std::vector<int>> deps(n);
@@ -414,7 +423,8 @@ void fuse_signals(Graph *G) {
     for (int v = 0; v < n; ++v) {
       if (user[v].primitive != PCCL_NOTIFY || deps[v].size() != 1) continue;
       const int a = deps[v][0];
-      if (!is_data(a) || G->notify_of[a] >= 0 || n_succ[a] - 1 + n_succ[v] > 255) continue;
+      if (!is_data(a) || G->notify_of[a] >= 0 || n_succ[a] - 1 + n_succ[v] > 255 || !cut_allows(a, v)) continue;
+      if (words_of(v)) G->signal_cut[a] = words_of(v);
       G->notify_of[a] = v;
       G->fused_into[v] = a;
       stands_for[v] = a;
@@ -437,7 +447,7 @@ void fuse_signals(Graph *G) {
     for (int v = 0; v < n; ++v) {
       if (user[v].primitive != PCCL_GET_NOTIFIED || succ_count[v] != 1) continue;
       const int b = only_succ[v];
-      if (!is_data(b) || G->wait_of[b] >= 0) continue;
+      if (!is_data(b) || G->wait_of[b] >= 0 || !cut_allows(b, v)) continue;
       std::vector<int> merged;
       for (int d : deps[b])
         if (d != v) merged.push_back(d);
@@ -445,6 +455,7 @@ void fuse_signals(Graph *G) {
       std::sort(merged.begin(), merged.end());
       merged.erase(std::unique(merged.begin(), merged.end()), merged.end());
       if (merged.size() > 255) continue;
+      if (words_of(v)) G->signal_cut[b] = words_of(v);
       G->wait_of[b] = v;
       G->fused_into[v] = b;
       deps[b].swap(merged);
@@ -673,12 +684,12 @@ void fill_fuse_table(const Graph *G, const std::vector<pccl_op_desc> &ops, Signa
     if (G->wait_of[i] >= 0) {
       const pccl_op_desc &w = ops[G->wait_of[i]];
       f.wait_word = (unsigned long long)(uintptr_t)w.ins[0];
-      f.wait_value = (unsigned int)w.count;
+      f.wait_value = (unsigned int)w.count | (w.signal_parts >= 2 ? kSignalPerPart : 0u);
     }
     if (G->notify_of[i] >= 0) {
       const pccl_op_desc &v = ops[G->notify_of[i]];
       f.notify_word = (unsigned long long)(uintptr_t)v.outs[0];
-      f.notify_value = (unsigned int)v.count;
+      f.notify_value = (unsigned int)v.count | (v.signal_parts >= 2 ? kSignalPerPart : 0u);
     }
     rows[i] = f;
   }
@@ -737,6 +748,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       if ((uintptr_t)sig % 4) return fail(PCCL_ERR_MISALIGNED, "op %d: signal address not 4-byte aligned", i);
       if (o.count < 0 || o.count > 0xffff)
         return fail(PCCL_ERR_INVALID_ARG, "op %d: signal value %ld outside [0, 65535]", i, o.count);
+      if ((int)o.signal_parts > kMaxParts)
+        return fail(PCCL_ERR_INVALID_ARG, "op %d: a signal of %d words (at most %d)", i, (int)o.signal_parts, kMaxParts);
       signal_ops.push_back(i);
     } else {
       if (o.dtype >= PCCL_NUM_DTYPES) return fail(PCCL_ERR_UNSUPPORTED, "op %d: unknown dtype code %d", i, o.dtype);
@@ -747,6 +760,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       if (o.primitive == PCCL_COPY && o.n_in != 1)
         return fail(PCCL_ERR_INVALID_ARG, "op %d: COPY takes exactly one input", i);
       if (o.count < 0) return fail(PCCL_ERR_INVALID_ARG, "op %d: count %ld < 0", i, o.count);
+      if (o.signal_parts) return fail(PCCL_ERR_INVALID_ARG, "op %d: signal_parts belongs to NOTIFY / GET_NOTIFIED", i);
       es = elem_bytes(o.dtype);
       for (int k = 0; k < o.n_in; ++k) {
         if (!o.ins[k] && o.count) return fail(PCCL_ERR_INVALID_ARG, "op %d: input %d is null", i, k);
@@ -774,8 +788,10 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   }
   // An op that carries a NOTIFY has one more place in its successor list: kSuccNotify, behind the ops
   // (what completes the op walks that list anyway, and an op with a successor waits for its stores).
+  // (a carried NOTIFY of a word per part has no place there: every part stores its own word)
+  auto notifies_by_part = [&](int i) { return G->notify_of[i] >= 0 && ops[G->notify_of[i]].signal_parts >= 2; };
   for (int i = 0; i < n_ops; ++i)
-    if (G->notify_of[i] >= 0) {
+    if (G->notify_of[i] >= 0 && !notifies_by_part(i)) {
       ++n_succ[i];
       ++n_edges;
     }
@@ -936,6 +952,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       };
       parts_by_level[i] = cut(part_bytes);
       parts[i] = cut(even_bytes);  // one size for every level until the chains are known (below): ops of equal length cut alike
+      // an op that carries signals of a word per part is cut into as many parts as the signal has words
+      if (G->signal_cut[i]) parts_by_level[i] = parts[i] = G->signal_cut[i];
       tiles += parts[i];
     }
     if (tiles > (1ll << 30)) return fail(PCCL_ERR_GRAPH, "graph needs %lld queue entries", tiles);
@@ -1238,7 +1256,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
           for (int p = first; p < std::min(first + block, parts[i]); ++p, ++t)
             qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32) |
                                       ((G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 || G->wait_of[i] >= 0 || G->notify_of[i] >= 0) ? kEntryChainHead : 0ull) |
-                                      (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull));
+                                      (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull) | (notifies_by_part(i) ? kEntryNotifiesPart : 0ull));
         }
       lo = hi;
     }
@@ -1294,6 +1312,11 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     // signal ops: the only operand is the signal word, num_elems_ carries the value
     for (int k = 0; k < o.n_in; ++k) pl->chunks_[k] = pccl_chunk_meta{o.dtype, (void *)o.ins[k], o.count};
     for (int k = 0; k < o.n_out; ++k) pl->chunks_[o.n_in + k] = pccl_chunk_meta{o.dtype, o.outs[k], o.count};
+    if (o.primitive == PCCL_NOTIFY || o.primitive == PCCL_GET_NOTIFIED) {
+      // ... and behind it the number of words the signal has (one, or one per part)
+      pl->chunks_[1] = pccl_chunk_meta{o.dtype, nullptr, o.signal_parts >= 2 ? (long)o.signal_parts : 1l};
+      h->op_size_ = (unsigned char)(8 + sizeof(pccl_chunk_meta) * 2);
+    }
   }
   fill_chain_table(G->chain_words, n_ops, img + off_payload, (ForwardStep *)(img + off_chain_table));
   fill_fuse_table(G, G->eff, (SignalFuse *)(img + off_fuse));
@@ -1627,6 +1650,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->fused_into.swap(fresh.fused_into);
     G->wait_of.swap(fresh.wait_of);
     G->notify_of.swap(fresh.notify_of);
+    G->signal_cut.swap(fresh.signal_cut);
     G->user_dep_to_eff.swap(fresh.user_dep_to_eff);
     G->fuse_table_off = fresh.fuse_table_off;
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
@@ -1715,7 +1739,7 @@ int pccl_hip_plan_chains(const pccl_op_desc *ops, int n_ops, const int *parts, i
   return PCCL_OK;
 }
 
-int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier) {
+int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier, int *parts) {
   pccl_host::clear_error();
   if (n_ops < 0 || (n_ops > 0 && (!ops || !carrier))) return fail(PCCL_ERR_INVALID_ARG, "plan_signals: bad arguments");
   for (int i = 0; i < n_ops; ++i) {
@@ -1729,6 +1753,9 @@ int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier) {
   G.descs.assign(ops, ops + n_ops);
   fuse_signals(&G);
   for (int i = 0; i < n_ops; ++i) carrier[i] = G.fused_into[i];
+  if (parts)
+    for (int i = 0; i < n_ops; ++i)
+      parts[i] = G.fused_into[i] >= 0 ? (ops[i].signal_parts >= 2 ? (int)ops[i].signal_parts : 0) : G.signal_cut[i];
   return PCCL_OK;
 }
 
@@ -1826,7 +1853,7 @@ int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_byte
     for (int i = 0; i < n_ops; ++i) {
       const pccl_op_desc &a = G->descs[i], &b = ops[i];
       if (a.op_uid != b.op_uid || a.primitive != b.primitive || a.dtype != b.dtype || a.compute != b.compute ||
-          a.n_in != b.n_in || a.n_out != b.n_out || a.count != b.count || a.n_deps != b.n_deps ||
+          a.n_in != b.n_in || a.n_out != b.n_out || a.count != b.count || a.n_deps != b.n_deps || a.signal_parts != b.signal_parts ||
           memcmp(a.ins, b.ins, sizeof(void *) * b.n_in) || memcmp(a.outs, b.outs, sizeof(void *) * b.n_out))
         return false;
     }

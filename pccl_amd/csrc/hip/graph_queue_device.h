@@ -86,7 +86,9 @@ constexpr unsigned long long kEntryChainHead = 1ull << 51;
 // ... | (every part polls a signal word first) << 52: the op carries a GET_NOTIFIED (GraphControl::fuse; such an
 // entry has the chain flag too, for the count of ops it stands for).
 constexpr unsigned long long kEntryWaitsSignal = 1ull << 52;
-constexpr unsigned long long kEntryFlags = kEntryChainHead | kEntryWaitsSignal;
+// ... | (whoever completes the part stores the part's signal word) << 53: the op carries a NOTIFY of one word per part.
+constexpr unsigned long long kEntryNotifiesPart = 1ull << 53;
+constexpr unsigned long long kEntryFlags = kEntryChainHead | kEntryWaitsSignal | kEntryNotifiesPart;
 // In a successor list: not an op, but "store the signal word of the NOTIFY this op carries".
 constexpr int kSuccNotify = -1;
 
@@ -309,8 +311,10 @@ static_assert(sizeof(ForwardStep) == 32, "two 16-byte loads per row");
 struct SignalFuse {
   unsigned long long wait_word;    // 0: none
   unsigned long long notify_word;  // 0: none
-  unsigned int wait_value, notify_value;
+  unsigned int wait_value, notify_value;  // | kSignalPerPart: the signal is a word per part, part p's is word p
 };
+constexpr unsigned int kSignalPerPart = 1u << 31;
+constexpr unsigned int kSignalValue = 0xffffu;
 static_assert(sizeof(SignalFuse) == 24, "three 8-byte words per row");
 
 __device__ __forceinline__ unsigned long long uniform64(unsigned long long v) {  // the same in every lane: into scalar registers
@@ -575,6 +579,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   int cur_uid = 0, cur_part = 0;  // the entry being executed (uniform)
   OpFacts cur_op = {1, 0, 0};     // ... and its op's facts (uniform)
   int cur_chain_ops = 1;          // ... and how many ops it stands for: the chain it heads, or itself
+  unsigned long long cur_entry = 0;         // the entry itself, flags included (thread 0 only)
   unsigned long long *cur_trace = nullptr;  // its trace record (thread 0 only)
   unsigned int exhausted = 0;  // bit q: queue q has no entries left (thread 0 only)
   // Signal values are offset by (run number << 16).  The run number lives on the device (not
@@ -647,11 +652,17 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       auto notify = [&](int uid) {
         if constexpr (!FORWARD) {
           const SignalFuse *f = &g.fuse[uid];
-          __hip_atomic_store((unsigned int *)f->notify_word, base_of_run() + f->notify_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          __hip_atomic_store((unsigned int *)f->notify_word, base_of_run() + (f->notify_value & kSignalValue), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
       };
       if (h) {
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
+        // the NOTIFY of a word per part that the op carries: this part's word (its stores were waited for)
+        if (!FORWARD && (cur_entry & kEntryNotifiesPart)) {
+          const SignalFuse *f = &g.fuse[cur_uid];
+          __hip_atomic_store((unsigned int *)f->notify_word + cur_part, base_of_run() + (f->notify_value & kSignalValue),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
         finish_part(g, h, cur_op, cur_uid, cur_part, &s_done, cur_chain_ops, draw_ticket, notify);
       } else {
         draw_ticket();
@@ -742,8 +753,10 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         // the GET_NOTIFIED the op carries: every part polls the word before it starts
         if (!FORWARD && (e & kEntryWaitsSignal)) {
           const SignalFuse *f = &g.fuse[uid];
-          unsigned int *word = (unsigned int *)f->wait_word;
-          const unsigned int want = base_of_run() + f->wait_value;
+          const unsigned int value = f->wait_value;
+          // (a word per part: this part's)
+          unsigned int *word = (unsigned int *)f->wait_word + ((value & kSignalPerPart) ? (int)((e & ~kEntryFlags) >> 32) : 0);
+          const unsigned int want = base_of_run() + (value & kSignalValue);
           if ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) < 0 &&
               !bounded_wait(abort_flag, spin_limit, [&] {
                 return (int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
@@ -756,12 +769,20 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         if (prim != PCCL_NOTIFY && prim != PCCL_GET_NOTIFIED) break;
         unsigned int *sig = (unsigned int *)sc->payload.chunks_[0].addr_;
         const unsigned int want = base_of_run() + (unsigned int)sc->payload.chunks_[0].num_elems_;
-        if (prim == PCCL_NOTIFY) {
-          // everything this op depends on is already at the point of coherence
-          __hip_atomic_store(sig, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        } else if (!bounded_wait(abort_flag, spin_limit, [&] {
-                     return (int)(__hip_atomic_load(sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
-                   })) {
+        // (a signal of a word per part that no data op carries: all of its words)
+        const int n_words = (int)sc->payload.chunks_[1].num_elems_;
+        bool gave_up = false;
+        for (int w = 0; w < n_words && !gave_up; ++w) {
+          if (prim == PCCL_NOTIFY) {
+            // everything this op depends on is already at the point of coherence
+            __hip_atomic_store(sig + w, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          } else if (!bounded_wait(abort_flag, spin_limit, [&] {
+                       return (int)(__hip_atomic_load(sig + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
+                     })) {
+            gave_up = true;
+          }
+        }
+        if (gave_up) {
           go = 0;
           break;
         }
@@ -770,6 +791,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
+      cur_entry = e;
       s_go = go;
       s_chain = chain_words;
       s_facts = op_facts;
@@ -779,6 +801,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
     if (!__builtin_amdgcn_readfirstlane(s_go)) break;
     const int uid = __builtin_amdgcn_readfirstlane((int)(s_entry & 0xffffffffu));
     const int part = __builtin_amdgcn_readfirstlane((int)((s_entry & ~kEntryFlags) >> 32));
+    const bool notifies_part = __builtin_amdgcn_readfirstlane((int)((s_entry & kEntryNotifiesPart) >> 53)) != 0;  // (its stores are waited for)
     cur_uid = uid;
     cur_part = part;
     h = &g.headers[uid];
@@ -831,7 +854,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
     // last op, has no successor in the graph) nobody reads the data before the kernel has ended,
     // and the wait is left out: one memory round trip less for the last ops of a graph.
     // The barrier also keeps s_entry / s_go from being rewritten while still being read.
-    if (cur_op.num_next_ops() > 0) settle_stores();
+    if (cur_op.num_next_ops() > 0 || (notifies_part && !FORWARD)) settle_stores();
     __syncthreads();
   }
 

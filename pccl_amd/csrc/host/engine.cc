@@ -130,8 +130,9 @@ void Engine::exeOp(const std::string &name, const void *input, void *output, lon
       const ScheduleOp &o = s.ops[i];
       BoundOp &b = bound[i];
       if (o.isSignal()) {  // the operand is one of the workspace's signal slots, the count its value
-        if (!signals || o.slot >= SLOT)
+        if (!signals || o.slot + o.parts > SLOT)
           throw std::runtime_error("Engine::exeOp(): signal slot " + std::to_string(o.slot) + " is not available");
+        b.signal_parts = o.parts;
         b.primitive = o.kind == ScheduleOp::NOTIFY ? notify : get_notified;
         b.compute = compute;
         b.deps = o.deps;

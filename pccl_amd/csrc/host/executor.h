@@ -22,6 +22,7 @@ struct BoundOp {
   std::vector<ChunkMeta> ins;
   std::vector<ChunkMeta> outs;
   std::vector<int> deps;    // indices of ops that must complete first
+  int signal_parts = 0;     // NOTIFY / GET_NOTIFIED: words of the signal, one per part of the data it announces (0, 1: one word)
 };
 
 class ExecutorBase {

@@ -193,6 +193,12 @@ void *HipExecutor::createGraph(const std::vector<BoundOp> &ops) {
     for (size_t k = 0; k < o.outs.size(); ++k) d.outs[k] = o.outs[k].addr_;
     d.n_deps = (int)o.deps.size();
     d.deps = o.deps.empty() ? nullptr : o.deps.data();
+    if (is_signal) {
+      if (o.signal_parts < 0 || o.signal_parts > 0xffff)
+        throw std::runtime_error("HipExecutor::createGraph(): op " + std::to_string(i) + " names a signal of " +
+                                 std::to_string(o.signal_parts) + " words");
+      d.signal_parts = (unsigned short)o.signal_parts;
+    }
   }
   // the executor's choice: plain launches for the few graphs that run faster that way, else the queue
   long tile_bytes = PCCL_HIP_TILE_AUTO;

@@ -34,6 +34,7 @@ void Schedule::validate() const {
     if (o.count < 0) bad(at + "negative count");
     if (o.isSignal()) {
       if (o.slot < 0 || o.slot >= 256) bad(at + "signal slot outside [0, 256)");
+      if (o.parts < 1 || o.slot + o.parts > 256) bad(at + "a signal of " + std::to_string(o.parts) + " words does not fit the 256 slots");
       if (o.count > 0xffff) bad(at + "signal value outside [0, 65535]");
       if (!o.srcs.empty() || !o.dsts.empty()) bad(at + "a signal op has no data operands");
       if (o.deps.size() > 255) bad(at + "more than 255 dependencies");
@@ -101,7 +102,10 @@ std::vector<int> Schedule::topologicalOrder() const {
 
 std::string Schedule::serialize() const {
   std::ostringstream os;
-  os << "pccl-schedule 1\n";
+  // version 2 where a signal has a word per part (the only thing version 1 cannot say)
+  bool by_part = false;
+  for (const ScheduleOp &o : ops) by_part = by_part || (o.isSignal() && o.parts > 1);
+  os << "pccl-schedule " << (by_part ? 2 : 1) << "\n";
   os << "name " << (name.empty() ? "unnamed" : name) << "\n";
   os << "dtype " << dtype << "\ncompute " << compute << "\n";
   os << "devices " << devices << "\nelems_per_device " << elems_per_device << "\n";
@@ -112,7 +116,9 @@ std::string Schedule::serialize() const {
     os << "op " << i << ' ' << kinds[o.kind] << ' ' << o.count << " deps " << o.deps.size();
     for (int d : o.deps) os << ' ' << d;
     if (o.isSignal()) {
-      os << " slot " << o.slot << "\n";
+      os << " slot " << o.slot;
+      if (by_part) os << " parts " << o.parts;
+      os << "\n";
       continue;
     }
     os << " src " << o.srcs.size();
@@ -159,7 +165,7 @@ Schedule Schedule::parse(const std::string &text) {
   Schedule s;
   expect("pccl-schedule");
   const long version = integer("version");
-  if (version != 1) bad("unsupported format version " + std::to_string(version));
+  if (version != 1 && version != 2) bad("unsupported format version " + std::to_string(version));
   expect("name");
   s.name = word("name");
   expect("dtype");
@@ -193,6 +199,12 @@ Schedule Schedule::parse(const std::string &text) {
     if (o.isSignal()) {
       expect("slot");
       o.slot = (int)integer("slot");
+      if (version >= 2) {
+        expect("parts");
+        const long k = integer("parts");
+        if (k < 1 || k > 256) bad("op " + std::to_string(i) + ": parts out of range");
+        o.parts = (int)k;
+      }
       continue;
     }
     for (int side = 0; side < 2; ++side) {

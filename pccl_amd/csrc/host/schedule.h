@@ -23,6 +23,12 @@
 // 256 slots behind the 256 MiB workspace) and a value in [0, 65535]; NOTIFY publishes the
 // value once its dependencies are complete, GET_NOTIFIED completes when the slot has
 // reached it (pccl/lang/chunk.py:9-10).
+// Version 2 ("pccl-schedule 2"; version 1 files load as before) differs in one thing: a signal
+// op line ends in "parts <K>", and with K >= 2 the signal is K consecutive slots from <index>,
+// slot p standing for part p of the data op it follows (NOTIFY) or precedes (GET_NOTIFIED), the
+// op cut into K parts (part p = elements [p * per, (p + 1) * per), per = ceil(count / K) rounded
+// up to 64).  The executor then lets the consumer start on part p as soon as the producer has
+// finished its part p (pccl_hip.h, pccl_op_desc::signal_parts).
 // Buffers: "in" and "out" are the tensors given to exeOp, laid out as W consecutive
 // per-device regions of elems_per_device elements; "ws" is the device workspace.
 #pragma once
@@ -44,6 +50,7 @@ struct ScheduleOp {
   bool reduce = false;  // kind == REDUCE (kept in step with kind by the parser and generators)
   bool isSignal() const { return kind == NOTIFY || kind == GET_NOTIFIED; }
   int slot = 0;         // signal ops: index of the signal slot; count is the value
+  int parts = 1;        // signal ops: slots the signal takes, one per part of the data (format version 2)
   long count = 0;
   std::vector<int> deps;
   std::vector<ScheduleOperand> srcs;

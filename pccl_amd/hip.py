@@ -41,7 +41,8 @@ class OpDesc(ctypes.Structure):
         ("compute", ctypes.c_ubyte),
         ("n_in", ctypes.c_ubyte),
         ("n_out", ctypes.c_ubyte),
-        ("reserved", ctypes.c_ubyte * 3),
+        ("reserved", ctypes.c_ubyte),
+        ("signal_parts", ctypes.c_ushort),
         ("ins", ctypes.c_void_p * MAX_INPUTS),
         ("outs", ctypes.c_void_p * MAX_OUTPUTS),
         ("count", ctypes.c_long),
@@ -84,7 +85,7 @@ def lib():
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.pccl_hip_classify_dependencies.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), vp]
         L.pccl_hip_plan_chains.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ci, ctypes.POINTER(ci)]
-        L.pccl_hip_plan_signals.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci)]
+        L.pccl_hip_plan_signals.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         L.pccl_hip_graph_dependency_kinds.argtypes = [vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
         L.pccl_hip_graph_trace.argtypes = [vp, ci]
         L.pccl_hip_graph_read_trace.argtypes = [vp, vp, vp, ctypes.c_long, ctypes.POINTER(ctypes.c_long)]
@@ -197,6 +198,7 @@ def _op_descs(ops):
             d.n_in, d.n_out = (0, 1) if prim == NOTIFY else (1, 0)
             (d.outs if prim == NOTIFY else d.ins)[0] = _addr(o["signal"])
             d.count = o["value"]
+            d.signal_parts = o.get("parts", 0)   # >= 2: a signal of that many words, one per part of the data
         else:
             n_in, n_out = len(o["ins"]), len(o["outs"])
             d.primitive = prim if prim is not None else (COPY if n_in == 1 else REDUCE)
@@ -244,12 +246,16 @@ def plan_chains(ops, parts, forward_elem_bytes):
     return [tuple(words[4 * i:4 * i + 4]) for i in range(len(ops))]
 
 
-def plan_signals(ops):
+def plan_signals(ops, with_parts=False):
     """Which signal ops ride on data ops (host only): per op the index of the COPY / REDUCE that carries
-    it, or -1."""
+    it, or -1.  with_parts: also, per op, the K of a signal op carried part by part / of the data op that is
+    cut into K parts for such signals (0 otherwise)."""
     arr, keep = _op_descs(ops)
     carrier = (ctypes.c_int * max(len(ops), 1))()
-    _check(lib().pccl_hip_plan_signals(arr, len(ops), carrier))
+    parts = (ctypes.c_int * max(len(ops), 1))()
+    _check(lib().pccl_hip_plan_signals(arr, len(ops), carrier, parts if with_parts else None))
+    if with_parts:
+        return list(carrier[:len(ops)]), list(parts[:len(ops)])
     return list(carrier[:len(ops)])
 
 

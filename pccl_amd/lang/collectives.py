@@ -167,13 +167,19 @@ def all_to_all(world, chunk_elems, dtype="bf16", name="all_to_all"):
 
 
 def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", name="ring_allreduce_signalled",
-                             first_slot=0):
+                             first_slot=0, signal_parts=1):
     """The same ring all-reduce written the way ranks on different GPUs have to write it:
     dependency edges only between ops of one rank; the hand-over between neighbours goes
     NOTIFY (producer) -> signal slot -> GET_NOTIFIED (consumer).  Link (r-1) -> r uses slot
     first_slot + r, and the value is the step number, so every slot sees its values rise.
+    signal_parts = K >= 2: every signal is K slots, one per part of the chunk it announces (link
+    (r-1) -> r: slots first_slot + r * K ...), so that a rank starts on part p of a step as soon as its
+    neighbour has finished part p of the step before (schedule format version 2).
     Returns (ir, elements_per_rank_used)."""
     W = world
+    K = max(1, int(signal_parts))
+    if first_slot + W * K > 256:
+        raise ValueError("%d links of %d slots each do not fit the 256 signal slots" % (W, K))
     ir = _ring_ir(name, W, dtype, compute)
     last = {}  # rank -> its latest op
     for step in range(1, 2 * W - 1):
@@ -187,7 +193,7 @@ def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", na
                 whole = Chunk(set(), p, chunk_elems, off)
                 deps = [ir.create_operation(PrimitiveOpType.GET_NOTIFIED, src_chunk=whole, tgt_chunk=whole, src_device=p,
                                             tgt_device=r, dependencies=deps,
-                                            metadata={"slot": first_slot + r, "value": step - 1})]
+                                            metadata={"slot": first_slot + r * K, "value": step - 1, "parts": K})]
             if reduce_phase:
                 ranks = {(c + i) % W for i in range(step + 1)}
                 op = ir.create_operation(
@@ -202,7 +208,7 @@ def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", na
             done = Chunk(set(), r, chunk_elems, off)
             last[r] = ir.create_operation(PrimitiveOpType.NOTIFY, src_chunk=done, tgt_chunk=done, src_device=r,
                                           tgt_device=(r + 1) % W, dependencies=[op],
-                                          metadata={"slot": first_slot + (r + 1) % W, "value": step})
+                                          metadata={"slot": first_slot + ((r + 1) % W) * K, "value": step, "parts": K})
     return ir, W * chunk_elems
 
 
@@ -247,7 +253,7 @@ def small_message_allreduce(world=8, n_slices=36, n_extra=64, seed=4, lo_bytes=8
 
 def bind(lowered, resolve, signals=None):
     """Replaces symbolic operands: resolve(buffer, device, element_offset) -> address.
-    Signal ops get "signal" = signals + 4 * slot (signals: address of the int slot array)."""
+    Signal ops get "signal" = signals + 4 * slot (signals: address of the int slot array); "parts" stays."""
     out = []
     for o in lowered:
         d = dict(o)

@@ -146,7 +146,8 @@ class CollectiveIR:
         low = self.lower()
         if elems_per_device is None:
             elems_per_device = max([x[2] + o["count"] for o in low for x in o["ins"] + o["outs"] if x[0] != "ws"] or [0])
-        lines = ["pccl-schedule 1", "name %s" % (self.name.replace(" ", "_") or "unnamed"), "dtype %s" % self.dtype,
+        by_part = any(o["primitive"] >= 2 and o.get("parts", 1) > 1 for o in low)   # only format version 2 can say that
+        lines = ["pccl-schedule %d" % (2 if by_part else 1), "name %s" % (self.name.replace(" ", "_") or "unnamed"), "dtype %s" % self.dtype,
                  "compute %s" % self.compute, "devices %d" % max(len(self.devices), 1),
                  "elems_per_device %d" % elems_per_device, "ops %d" % len(low)]
         kinds = ("COPY", "REDUCE", "NOTIFY", "GET_NOTIFIED")
@@ -154,7 +155,7 @@ class CollectiveIR:
             parts = ["op %d %s %d deps %d" % (i, kinds[o["primitive"]], o["count"], len(o["deps"]))]
             parts += [str(d) for d in o["deps"]]
             if o["primitive"] >= 2:
-                lines.append(" ".join(parts + ["slot %d" % o["slot"]]))
+                lines.append(" ".join(parts + ["slot %d" % o["slot"]] + (["parts %d" % o.get("parts", 1)] if by_part else [])))
                 continue
             for key, ops in (("src", o["ins"]), ("dst", o["outs"])):
                 parts.append("%s %d" % (key, len(ops)))
@@ -171,7 +172,8 @@ class CollectiveIR:
         """Returns a list of dicts (dtype, compute, primitive, ins, outs, count, deps) whose
         operands are symbolic ``(buffer, device, element_offset)`` triples, op ids preserved.
 
-        NOTIFY / GET_NOTIFIED lower to signal ops (``primitive`` 2 / 3, ``slot``, ``value``).
+        NOTIFY / GET_NOTIFIED lower to signal ops (``primitive`` 2 / 3, ``slot``, ``value``, ``parts``: slots the
+        signal takes, one per part of the data it announces; metadata "parts", default 1).
         A COPY reads ``src_chunk`` and writes ``tgt_chunk``.  A REDUCE folds its sources in
         order and writes every destination; without ``metadata["srcs"]`` it is the reference's
         two-operand form "reduce src into tgt": fold(src, tgt) -> tgt."""
@@ -185,7 +187,7 @@ class CollectiveIR:
                     raise ValueError("op %d: NOTIFY / GET_NOTIFIED need metadata 'slot' and 'value'" % op_id)
                 prim = 2 if op.op_type is PrimitiveOpType.NOTIFY else 3
                 out.append(dict(primitive=prim, slot=int(md["slot"]), value=int(md["value"]), ins=[], outs=[],
-                                count=int(md["value"]), deps=list(op.dependencies)))
+                                count=int(md["value"]), deps=list(op.dependencies), parts=int(md.get("parts", 1))))
                 continue
             src = (md.get("src_buffer", "out"), op.src_device, op.src_chunk.offset)
             tgt = (md.get("tgt_buffer", "out"), op.tgt_device, op.tgt_chunk.offset)

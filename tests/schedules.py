@@ -83,8 +83,10 @@ def parse_schedule_text(text):
     def nxt():
         return next(it)
 
-    assert nxt() == "pccl-schedule" and nxt() == "1"
-    hdr = {}
+    assert nxt() == "pccl-schedule"
+    version = int(nxt())
+    assert version in (1, 2)
+    hdr = {"version": version}
     for key in ("name", "dtype", "compute", "devices", "elems_per_device", "ops"):
         assert nxt() == key
         hdr[key] = nxt()
@@ -98,7 +100,11 @@ def parse_schedule_text(text):
         deps = [int(nxt()) for _ in range(int(nxt()))]
         if kind in ("NOTIFY", "GET_NOTIFIED"):
             assert nxt() == "slot"
-            ops.append(dict(signal=kind, slot=int(nxt()), value=count, ins=[], outs=[], count=0, deps=deps))
+            slot, parts = int(nxt()), 1
+            if version >= 2:   # (version 2: the slots the signal takes, one per part of the data)
+                assert nxt() == "parts"
+                parts = int(nxt())
+            ops.append(dict(signal=kind, slot=slot, parts=parts, value=count, ins=[], outs=[], count=0, deps=deps))
             continue
         sides = []
         for key in ("src", "dst"):
@@ -116,10 +122,12 @@ def replay_with_signals(oracle, ops, order, resolve):
     for i in order:
         o = ops[i]
         if o.get("signal") == "NOTIFY":
-            assert slots.get(o["slot"], -1) < o["value"], "slot %d must rise" % o["slot"]
-            slots[o["slot"]] = o["value"]
+            for w in range(o.get("parts", 1)):
+                assert slots.get(o["slot"] + w, -1) < o["value"], "slot %d must rise" % (o["slot"] + w)
+                slots[o["slot"] + w] = o["value"]
         elif o.get("signal") == "GET_NOTIFIED":
-            assert slots.get(o["slot"], -1) >= o["value"], "op %d waits for a value nobody published before it" % i
+            for w in range(o.get("parts", 1)):
+                assert slots.get(o["slot"] + w, -1) >= o["value"], "op %d waits for a value nobody published before it" % i
         else:
             oracle.reduce_copy(o["dtype"], o["compute"], [resolve(*x, o["count"]) for x in o["ins"]],
                                [resolve(*x, o["count"]) for x in o["outs"]])

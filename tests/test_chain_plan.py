@@ -184,12 +184,12 @@ def test_bad_arguments_are_refused():
 
 # ---- which signal ops ride on data ops (pccl_hip_plan_signals, host only) --------------------
 
-def notify(word, value, deps):
-    return dict(primitive=2, signal=word, value=value, deps=list(deps))
+def notify(word, value, deps, parts=0):
+    return dict(primitive=2, signal=word, value=value, deps=list(deps), parts=parts)
 
 
-def get_notified(word, value, deps):
-    return dict(primitive=3, signal=word, value=value, deps=list(deps))
+def get_notified(word, value, deps, parts=0):
+    return dict(primitive=3, signal=word, value=value, deps=list(deps), parts=parts)
 
 
 def test_a_ring_step_carries_its_wait_and_its_notify():
@@ -203,6 +203,28 @@ def test_a_ring_step_carries_its_wait_and_its_notify():
     moved = [dict(o) for o in ops]
     moved[1] = op([b, a], [u], [0])
     assert hip.plan_signals(moved) == [1, -1, 1, 4, -1, 4]
+
+
+def test_signals_of_a_word_per_part_cut_their_data_op():
+    """A NOTIFY / GET_NOTIFIED of K words (one per part of the data) rides on a data op like a one-word one, and the
+    op is then cut into K parts; an op carries such signals of ONE K only."""
+    a, b, t, u = (buf(k) for k in range(4))
+    sig = 0x900000
+    ops = [get_notified(sig, 1, [], parts=8), op([a, b], [t], [0]), notify(sig + 64, 1, [1], parts=8),
+           get_notified(sig, 2, [2], parts=8), op([t], [u], [3]), notify(sig + 64, 2, [4], parts=8)]
+    assert hip.plan_signals(ops, with_parts=True) == ([1, -1, 1, 4, -1, 4], [8, 8, 8, 8, 8, 8])
+    # one word (parts 0 or 1) is the form there always was: carried, the op's cut is the executor's
+    plain = [dict(o, parts=1) if "parts" in o else o for o in ops]
+    assert hip.plan_signals(plain, with_parts=True) == ([1, -1, 1, 4, -1, 4], [0] * 6)
+    # a wait of 8 words and a notify of 4 on one op: the notify comes first in the rule and is carried, the wait stays
+    mixed = [get_notified(sig, 1, [], parts=8), op([a, b], [t], [0]), notify(sig + 64, 1, [1], parts=4)]
+    assert hip.plan_signals(mixed, with_parts=True) == ([-1, -1, 1], [0, 4, 4])
+    # ... a one-word signal beside a per-part one is no conflict
+    mixed = [get_notified(sig, 1, []), op([a, b], [t], [0]), notify(sig + 64, 1, [1], parts=4)]
+    assert hip.plan_signals(mixed, with_parts=True) == ([1, -1, 1], [0, 4, 4])
+    # a per-part signal that no data op can carry (two ops behind it) stays an op of its own
+    alone = [op([a], [t], []), op([b], [u], []), notify(sig, 1, [0, 1], parts=16)]
+    assert hip.plan_signals(alone, with_parts=True) == ([-1, -1, -1], [0, 0, 0])
 
 
 def test_signal_ops_that_stay_ops_of_their_own():

@@ -110,16 +110,18 @@ def test_direct_allreduce_8_inputs(E, eng, oracle, tmp_path):
     H.assert_bits_equal(got[:per], oracle.reduce("f16", "sum", wide), "equals one 8-input fold in rank order")
 
 
-def test_signalled_ring_schedule(E, eng, oracle, tmp_path):
+@pytest.mark.parametrize("parts", [1, 4])
+def test_signalled_ring_schedule(E, eng, oracle, tmp_path, parts):
     """A schedule whose cross-rank hand-over goes through NOTIFY / GET_NOTIFIED on the workspace's
-    signal slots (no dependency edge between ranks), registered from a file and run twice."""
+    signal slots (no dependency edge between ranks), registered from a file and run twice; with one slot per
+    signal (format version 1) and with a slot per part of the chunk (version 2)."""
     import torch
     from pccl_amd import lang
-    ir, per = lang.ring_allreduce_signalled(8, 2500, dtype="bf16", first_slot=16)
+    ir, per = lang.ring_allreduce_signalled(8, 2500, dtype="bf16", first_slot=16, signal_parts=parts)
     p = str(tmp_path / "sig.sched")
     ir.save(p, per)
     text = open(p).read()
-    assert "NOTIFY" in text and "GET_NOTIFIED" in text
+    assert "NOTIFY" in text and "GET_NOTIFIED" in text and text.startswith("pccl-schedule %d\n" % (1 if parts == 1 else 2))
     eng.regOp("sig", p)
     hdr, ops = S.parse_schedule_text(text)
     n = 8 * per
@@ -129,7 +131,7 @@ def test_signalled_ring_schedule(E, eng, oracle, tmp_path):
         bufs = {"in": host_in, "out": want}
         # file order is a valid order (each rank's program order, steps ascending)
         slots = S.replay_with_signals(oracle, ops, range(len(ops)), lambda b, r, e, c: bufs[b][r * per + e:r * per + e + c])
-        assert slots == {16 + r: 14 for r in range(8)}
+        assert slots == {16 + k: 14 for k in range(8 * parts)}
         d_in, d_out = _to_dev(torch, host_in), torch.zeros(n * 2, dtype=torch.uint8, device="cuda")
         eng.exeOp("sig", d_in, d_out)
         eng.waitOp("sig")

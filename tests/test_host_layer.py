@@ -252,7 +252,15 @@ def test_direct_allreduce_schedule_shape(E, tmp_path):
 
 
 @pytest.mark.parametrize("text, why", [
-    ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "version"),
+    ("pccl-schedule 3\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "version"),
+    ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 NOTIFY 4 deps 0 slot 3\n", "expected parts"),
+    ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 NOTIFY 4 deps 0 slot 250 parts 8\n", "does not fit"),
+    ("pccl-schedule 2\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 GET_NOTIFIED 4 deps 0 slot 0 parts 0\n", "parts out of range"),
+    ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
+     "op 0 NOTIFY 4 deps 0 slot 3 parts 2\n", "trailing text"),
     ("pccl-schedule 1\nname x\ndtype q7\ncompute sum\ndevices 1\nelems_per_device 4\nops 0\n", "dtype"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute xor\ndevices 1\nelems_per_device 4\nops 0\n", "compute"),
     ("pccl-schedule 1\nname x\ndtype f32\ncompute sum\ndevices 1\nelems_per_device 4\nops 1\n"
@@ -280,6 +288,32 @@ def test_schedule_parser_rejects(E, text, why):
         eng.regOpText("bad", text)
     assert why.lower() in str(e.value).lower(), str(e.value)
     eng.close()
+
+
+def test_schedule_format_version_2_says_signals_of_a_slot_per_part(E, tmp_path):
+    """A signalled ring whose signals take K slots, one per part of the chunk they announce, is written as
+    "pccl-schedule 2" with "parts K" behind every signal op's slot; the native parser loads it (and version 1
+    files as before), and the same ring with one-slot signals is still written as version 1."""
+    from pccl_amd import lang
+    ir, per = lang.ring_allreduce_signalled(4, 1000, dtype="f32", first_slot=8, signal_parts=4)
+    text = ir.serialize(per)
+    assert text.startswith("pccl-schedule 2\n")
+    hdr, ops = S.parse_schedule_text(text)
+    sig = [o for o in ops if o.get("signal")]
+    assert hdr["version"] == 2 and len(sig) == 44 and all(o["parts"] == 4 for o in sig)
+    assert sorted(set(o["slot"] for o in sig)) == [8, 12, 16, 20]          # link r: slots 8 + 4 r ...
+    p = str(tmp_path / "v2.sched")
+    ir.save(p, per)
+    assert E.inspect_schedule(p, want_order=False)["n_ops"] == len(ops)
+    eng = E.Engine(0, 1)
+    eng.initEngine()
+    eng.regOp("v2", p)
+    assert eng.opInfo("v2")["n_ops"] == len(ops)
+    eng.close()
+    plain, _ = lang.ring_allreduce_signalled(4, 1000, dtype="f32", first_slot=8)
+    assert plain.serialize(per).startswith("pccl-schedule 1\n") and " parts " not in plain.serialize(per)
+    with pytest.raises(ValueError):
+        lang.ring_allreduce_signalled(8, 1000, signal_parts=33)            # 8 links x 33 slots > 256
 
 
 def test_engine_without_gpu_fails_loudly(E, tmp_path):
