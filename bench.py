@@ -146,7 +146,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--extras", default="all", metavar="LIST",
-                    help="comma-separated secondary workloads to run: layout (the headline shape on torch tensors and through Engine::exeOp), nvls, accumulate, ring, plumbing, unaligned, "
+                    help="comma-separated secondary workloads to run: layout (the headline shape on torch tensors and through Engine::exeOp), nvls, accumulate, ring, plumbing, unaligned, footprint, "
                          "op64k, schedule (one persistent launch), schedule_launches (the same ops as 4096 launches), "
                          "or all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -439,7 +439,16 @@ def main():
                 dsts = [randn(torch, c3, "bf16") for _ in range(7)]
                 t = event_times_us(torch, lambda: hip.accumulate("bf16", "sum", src, dsts, c3, stream), 20, 3)
                 extras["accumulate_bf16_1in_7dst_128MiB"] = dict(stats(t), GBps_median=gbps(15 * c3 * 2, t[len(t) // 2]))
-                del src, dsts
+                # what bounds it: the share of writes.  Two walks of the same width for comparison, a broadcast
+                # copy 1 -> 7 (1 read stream, 7 write streams) and a fold 8 -> 7 (8 read streams, 7 write streams,
+                # exactly the accumulate's traffic without its in-place destinations)
+                more = [randn(torch, c3, "bf16") for _ in range(7)]
+                t17 = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [src], dsts, c3, stream), 20, 3)
+                t87 = event_times_us(torch, lambda: hip.reduce_copy("bf16", "sum", [src] + more, dsts, c3, stream), 20, 3)
+                extras["accumulate_bf16_1in_7dst_128MiB"]["same_width_walks"] = {
+                    "copy_1in_7out": dict(stats(t17), GBps_median=gbps(8 * c3 * 2, t17[len(t17) // 2])),
+                    "fold_8in_7out": dict(stats(t87), GBps_median=gbps(15 * c3 * 2, t87[len(t87) // 2]))}
+                del src, dsts, more
 
         # ---- ring all-reduce, one rank's share at world 8: 7 reduce-copy + 7 copy steps ----
         if want("ring"):
@@ -566,6 +575,30 @@ def main():
                     "copy_step_1in_1out_32MiB": dict(stats(tc), GBps_median=gbps(2 * ce * 2, med(tc))),
                     "note": "single steps re-touch 128/64 MiB and are helped by the 256 MB Infinity Cache; "
                             "the 14-step figures walk 1.1 GiB of distinct data (1.3 GiB where the copy steps read buffers of their own)"}
+                # ... and the way the reference's host code would run the rank's share: the 14 steps as a schedule
+                # file through Engine::regOp / exeOp (regions of one input and one output tensor; the executor
+                # sends a graph of this shape to the queue: one launch)
+                import tempfile
+                from pccl_amd import engine as engine_mod
+                share = {}
+                for own_gather in (False, True):
+                    irs, per_region = lang.ring_rank_share(W, ce, dtype="bf16", gather_buffers_of_their_own=own_gather)
+                    with tempfile.TemporaryDirectory() as tmp:
+                        path = os.path.join(tmp, "share.sched")
+                        irs.save(path, per_region)
+                        eng = engine_mod.Engine(0, 1)
+                        eng.initEngine()
+                        eng.regOp("share", path)
+                        x = torch.cat([grad] + peers + [send] + ((late + [send]) if own_gather else []))
+                        y = torch.zeros_like(x)
+                        te = event_times_us(torch, lambda: eng.exeOp("share", x, y, stream), 20, 3)
+                        eng.waitOp("share", stream)
+                        assert torch.equal(y[:W * ce], ref_late if own_gather else ref_result), "engine result differs from the 14 launches"
+                        share["copy_steps_read_buffers_of_their_own" if own_gather else "as_configured"] = dict(
+                            stats(te), GBps_median=gbps(ring_bytes, med(te)))
+                        eng.close()
+                        del x, y
+                extras["ring_allreduce_rank_share"]["via_engine_exeOp"] = share
                 del late
                 del grad, peers, result, send
 
@@ -747,6 +780,29 @@ def main():
                 extras["unaligned_i32_4in_1out_1GiB"]["other_counts_and_folds"] = other
                 del fpool, ou
 
+        # ---- footprint: the same shapes at 256 MiB and at 1 GiB per operand, aligned ------------------
+        # (4 -> 1 is the shape of the unaligned leg above; a copy and 2 -> 1 stand beside it as the simplest
+        # walks over the same footprint; profiles/reduce_copy_4in_1GiB_counters.md holds the counters)
+        if want("footprint"):
+            with secondary_leg(extras, "footprint"):
+                cmax = 1 << 28
+                pool = [torch.randint(-(1 << 20), (1 << 20) + 1, (cmax,), dtype=torch.int32, device="cuda", generator=seeded(torch, 3)) for _ in range(4)]
+                dst = torch.empty(cmax, dtype=torch.int32, device="cuda")
+                foot = {}
+                for label, c in (("256MiB", 1 << 26), ("1GiB", 1 << 28)):
+                    for dtype, n_in in (("i32", 4), ("bf16", 4), ("i32", 2), ("i32", 1)):
+                        cnt = c * (2 if dtype == "bf16" else 1)      # same bytes per operand
+                        es = 2 if dtype == "bf16" else 4
+                        srcs = [x[:c] for x in pool[:n_in]]
+                        t = event_times_us(torch, lambda: hip.reduce_copy(dtype, "sum", srcs, [dst[:c]], cnt, stream), 12, 3)
+                        foot["%s_%din_1out_%s" % (dtype, n_in, label)] = dict(stats(t), GBps_median=gbps((n_in + 1) * cnt * es, t[len(t) // 2]))
+                chk = pool[0][:1 << 20] + pool[1][:1 << 20]
+                hip.reduce_copy("i32", "sum", [x[:1 << 20] for x in pool[:2]], [dst[:1 << 20]], 1 << 20, stream)
+                torch.cuda.synchronize()
+                assert torch.equal(dst[:1 << 20], chk)
+                extras["aligned_by_footprint"] = foot
+                del pool, dst
+
         # ---- small ops: 64 KiB direct launch and through the queue --------------------------
         if want("op64k"):
             with secondary_leg(extras, "op64k"):
@@ -783,9 +839,27 @@ def main():
                         hip.reduce_copy("bf16", "sum", o["ins"], o["outs"], o["count"], stream)
 
                 sched_moved = queue_bytes_moved(hip, bound, 2)
+                # the same graph with every op queueing its own entries (no chains: nothing stays in registers,
+                # every op reads and writes all its operands)
+                os.environ["PCCL_HIP_CHAINS"] = "0"
+                try:
+                    g0 = hip.Graph(bound)
+                finally:
+                    del os.environ["PCCL_HIP_CHAINS"]
+                for b in bufs["out"]:
+                    b.zero_()
+                t0 = event_times_us(torch, lambda: g0.run(stream), 30, 5)
+                done, total = g0.status(stream)
+                assert done == total == len(low)
+                for r in range(1, 8):
+                    assert torch.equal(bufs["out"][r][:per_rank // 2], bufs["out"][0][:per_rank // 2])
+                unchained = dict(stats(t0), us_per_op=round(t0[len(t0) // 2] / len(low), 4), GBps_median=gbps(sched_bytes, t0[len(t0) // 2]),
+                                 queue_entries=g0.info()["n_tiles"])
+                g0.destroy()
                 extras["schedule_4096_ops"] = {
                     "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med),
                                                   GBps_moved_median=gbps(sched_moved, med)),
+                    "one_persistent_launch_without_chains": unchained,
                     "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
                     "algorithmic_bytes": sched_bytes, "bytes_moved": sched_moved,
                     "note": "GBps_median counts the algorithmic bytes of the 4096 ops; chains of 14 ops keep the value in registers "

@@ -212,6 +212,41 @@ def ring_allreduce_signalled(world, chunk_elems, dtype="bf16", compute="sum", na
     return ir, W * chunk_elems
 
 
+def ring_rank_share(world, chunk_elems, dtype="bf16", compute="sum", name="ring_rank_share", gather_buffers_of_their_own=False):
+    """ONE rank's share of a ring all-reduce at world size `world`, its peers standing in as buffers: W - 1
+    reduce-copy steps (incoming chunk + local chunk -> output chunk + send buffer) and W - 1 copy steps
+    (incoming reduced chunk -> output chunk).  Step s of the first phase works on chunk (W - 1 - s) mod W, step s
+    of the second on chunk (W - s) mod W.
+
+    Regions ("devices" of the schedule file, each W * chunk_elems elements of the "in" and the "out" tensor):
+    0 = the rank itself ("in": its gradient, W chunks; "out": the result), 1 = what arrives from the neighbour
+    ("in": chunk s = the incoming buffer of step s; "out" chunk 0: the send buffer), and, with
+    gather_buffers_of_their_own, 2 = a second set of incoming buffers that the copy steps read (otherwise copy step
+    s reads the incoming buffer of reduce step s again).
+    Dependencies are the hazards of the buffers: every reduce step writes the one send buffer (step s behind step
+    s - 1), and copy step s overwrites the output chunk that reduce step s - 1 wrote.
+    Returns (ir, elements_per_region)."""
+    W, n = world, chunk_elems
+    ir = CollectiveIR(name, dtype=dtype, compute=compute)
+    for d in range(3 if gather_buffers_of_their_own else 2):
+        ir.add_device(Device(d, DeviceType.ROCM, memory_bandwidth=8.0e12, compute_capability=9.5))
+    reduce_ops = []
+    for s in range(W - 1):
+        c = (W - 1 - s) % W
+        reduce_ops.append(ir.create_operation(
+            PrimitiveOpType.REDUCE, src_chunk=Chunk({1}, 1, n, s * n), tgt_chunk=Chunk({0, 1}, 0, n, c * n), src_device=1, tgt_device=0,
+            dependencies=[reduce_ops[-1]] if reduce_ops else [],
+            metadata={"srcs": [("in", 1, s * n), ("in", 0, c * n)], "tgt_buffer": "out", "dsts": [("out", 1, 0)]}))
+    src_region = 2 if gather_buffers_of_their_own else 1
+    for s in range(W - 1):
+        c = (W - s) % W
+        ir.create_operation(
+            PrimitiveOpType.COPY, src_chunk=Chunk({0, 1}, src_region, n, s * n), tgt_chunk=Chunk({0, 1}, 0, n, c * n),
+            src_device=src_region, tgt_device=0, dependencies=[reduce_ops[s - 1]] if s else [],
+            metadata={"src_buffer": "in", "tgt_buffer": "out"})
+    return ir, W * n
+
+
 def log_uniform_sizes(n, seed, lo_bytes, hi_bytes, elem_bytes):
     """n sizes in elements, log-uniform in [lo_bytes, hi_bytes] (splitmix64 stream of `seed`)."""
     def mix(z):

@@ -110,6 +110,40 @@ def test_direct_allreduce_8_inputs(E, eng, oracle, tmp_path):
     H.assert_bits_equal(got[:per], oracle.reduce("f16", "sum", wide), "equals one 8-input fold in rank order")
 
 
+@pytest.mark.parametrize("own_gather,chunk", [(False, 40_003), (True, 1 << 20)])
+def test_rank_share_schedule_through_exeop(E, eng, oracle, tmp_path, own_gather, chunk):
+    """One rank's 14 ring steps at world size 8 (7 reduce-copy steps into an output chunk and the one send
+    buffer, 7 copy steps) as a schedule file through Engine::regOp / exeOp: 14 ops ordered by the hazards of their
+    buffers, which the executor sends to the queue as one launch.  Twice, on fresh inputs, against the CPU
+    checker replaying the file."""
+    import torch
+    from pccl_amd import lang
+    ir, per = lang.ring_rank_share(8, chunk, dtype="bf16", gather_buffers_of_their_own=own_gather)
+    p = str(tmp_path / "share.sched")
+    ir.save(p, per)
+    name = "share%d" % own_gather
+    eng.regOp(name, p)
+    info = eng.opInfo(name)
+    assert info["n_ops"] == 14 and info["devices"] == (3 if own_gather else 2) and info["elems_per_device"] == 8 * chunk
+    n = info["devices"] * per
+    stream = torch.cuda.current_stream().cuda_stream
+    for it in range(2):
+        host_in = H.gen("bf16", n, 79 + it, 0)
+        hdr, want = _oracle_replay(oracle, open(p).read(), host_in)
+        d_in, d_out = _to_dev(torch, host_in), torch.zeros(n * 2, dtype=torch.uint8, device="cuda")
+        eng.exeOp(name, d_in, d_out, stream)
+        eng.waitOp(name, stream)
+        got = d_out.cpu().numpy().view(np.uint16)
+        H.assert_bits_equal(got[:per], want[:per], "result, run %d" % it)
+        H.assert_bits_equal(got[per:per + chunk], want[per:per + chunk], "send buffer, run %d" % it)
+        assert not got[per + chunk:].any(), "nothing else of the output tensor is written"
+        # the result is the gradient with chunk c replaced: chunks 1..7 hold what the copy steps brought, chunk 0 the last fold
+        src = 2 if own_gather else 1
+        for s in range(7):
+            c = (8 - s) % 8
+            H.assert_bits_equal(got[c * chunk:(c + 1) * chunk], host_in[src * per + s * chunk:src * per + (s + 1) * chunk], "copy step %d" % s)
+
+
 @pytest.mark.parametrize("parts", [1, 4])
 def test_signalled_ring_schedule(E, eng, oracle, tmp_path, parts):
     """A schedule whose cross-rank hand-over goes through NOTIFY / GET_NOTIFIED on the workspace's
