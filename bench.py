@@ -153,6 +153,10 @@ def parse():
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="N",
                     help="also launch N plain copies (1 input -> 1 output) of the same 256 MiB buffers: the "
                          "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--timeline", action="store_true",
+                    help="instead of the benchmark: the queue executor's own per-entry timeline (pccl_hip_graph_trace) of one "
+                         "rank's 14 ring steps of 32 MiB (copy steps reading buffers of their own) and of the all-reduces over "
+                         "8 ranks x 32 MiB, as a JSON line: where the workgroups' time goes")
     ap.add_argument("--traffic-record", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="write %s from the output folders of the two rocprofv3 --pmc runs, then exit (no GPU needed)"
                          % os.path.relpath(TRAFFIC_RECORD, ROOT))
@@ -272,10 +276,85 @@ def cpu_baseline(count_sample):
             "other_shapes": other, "host_cpus_visible": os.cpu_count()}
 
 
+def queue_timeline(torch, hip, graph, stream, runs=3):
+    """Where the workgroups' time went in the last of `runs` traced runs of `graph`: shares of (workgroups x run
+    time) spent inside parts, waiting for dependencies, between a part's end and the next claim, before the
+    first claim and idle behind the last part; from the executor's per-entry records (claimed, ready, done)."""
+    import numpy as np
+    graph.trace(True)
+    for _ in range(runs):
+        graph.run(stream)
+        torch.cuda.synchronize()
+    tr = graph.read_trace(stream)
+    graph.trace(False)
+    tr = tr[tr[:, 1] > 0]
+    t0 = int(tr[:, 1].min())
+    wg = (tr[:, 0].astype(np.uint64) >> np.uint64(52)).astype(int)
+    cl, rd, dn = ((tr[:, k].astype(np.int64) - t0) / 100.0 for k in (1, 2, 3))    # microseconds on the 100 MHz clock
+    end, groups = float(dn.max()), sorted(set(wg.tolist()))
+    gaps, tail, first, per_gap = 0.0, 0.0, 0.0, []
+    for w in groups:
+        m = wg == w
+        order = np.argsort(cl[m])
+        c, d = cl[m][order], dn[m][order]
+        g = (c[1:] - d[:-1]).clip(min=0)
+        per_gap += g.tolist()
+        gaps += float(g.sum())
+        tail += end - float(d[-1])
+        first += float(c[0])
+    total = end * len(groups)
+    pct = lambda x: round(100.0 * x / total, 1)
+    q = lambda a, p: round(float(np.percentile(a, p)), 2) if len(a) else None
+    return {"traced_run_us": round(end, 1), "workgroups": len(groups), "entries": int(len(tr)),
+            "pct_in_parts": pct(float((dn - rd).sum())), "pct_waiting_for_dependencies": pct(float((rd - cl).sum())),
+            "pct_between_part_end_and_next_claim": pct(gaps), "pct_before_first_claim": pct(first), "pct_idle_at_the_end": pct(tail),
+            "part_us_median": q(dn - rd, 50), "part_us_p95": q(dn - rd, 95), "gap_us_median": q(per_gap, 50), "gap_us_p95": q(per_gap, 95),
+            "last_part_end_by_workgroup_us_p5_p50_p100": [q([float(dn[wg == w].max()) for w in groups], p) for p in (5, 50, 100)]}
+
+
+def timeline_main():
+    import torch
+    from pccl_amd import hip, lang
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    W, ce = 8, 1 << 24
+    grad = randn(torch, W * ce, "bf16", 1e-2, seed=1)
+    peers = [randn(torch, ce, "bf16", 1e-2, seed=1) for _ in range(W - 1)]
+    late = [randn(torch, ce, "bf16", 1e-2, seed=1) for _ in range(W - 1)]
+    result = torch.empty(W * ce, dtype=torch.bfloat16, device="cuda")
+    send = torch.empty(ce, dtype=torch.bfloat16, device="cuda")
+    ops = []
+    for s in range(W - 1):
+        c = (W - 1 - s) % W
+        ops.append(dict(dtype="bf16", compute="sum", ins=[peers[s], grad[c * ce:(c + 1) * ce]], outs=[result[c * ce:(c + 1) * ce], send],
+                        count=ce, deps=[len(ops) - 1] if ops else []))
+    for s in range(W - 1):
+        c = (W - s) % W
+        ops.append(dict(dtype="bf16", compute="sum", ins=[late[s]], outs=[result[c * ce:(c + 1) * ce]], count=ce, deps=[s - 1] if s else []))
+    g = hip.Graph(ops)
+    t = event_times_us(torch, lambda: g.run(stream), 20, 3)
+    out["ring_rank_share_14_steps_32MiB_copy_steps_read_buffers_of_their_own"] = dict(queue_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
+    g.destroy()
+    del grad, peers, late, result, send
+    for kind, emit in (("ring_allreduce_8_ranks_x_32_MiB", lang.ring_allreduce), ("direct_allreduce_8_ranks_x_32_MiB", lang.direct_allreduce)):
+        ir, per_rank = emit(8, (32 << 20) // 2 // 8, dtype="bf16")
+        rb = {"in": [randn(torch, per_rank, "bf16", 1e-2, seed=1) for _ in range(8)],
+              "out": [torch.zeros(per_rank, dtype=torch.bfloat16, device="cuda") for _ in range(8)]}
+        g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+        t = event_times_us(torch, lambda: g.run(stream), 20, 3)
+        out[kind] = dict(queue_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
+        g.destroy()
+    print(json.dumps({"queue_timeline": out}))
+
+
 def main():
     args = parse()
     if args.traffic_record:
         write_traffic_record(*args.traffic_record)
+        return
+    if args.timeline:
+        timeline_main()
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (peers are HBM buffers on the "
