@@ -829,7 +829,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     }
     occ = std::min(occ, o);
   }
-  const long long cap = (long long)pccl_host::compute_units() * occ;
+  // (fewer than kExitQuit: the exit word counts the workgroups that have left in 16 bits)
+  const long long cap = std::min<long long>((long long)pccl_host::compute_units() * occ, (long long)kExitQuit - 1);
   // ---- acyclicity (Kahn) -----------------------------------------------------
   std::vector<int> succ_start(n_ops + 1, 0);
   for (int i = 0; i < n_ops; ++i) succ_start[i + 1] = succ_start[i] + n_succ[i];

@@ -96,7 +96,8 @@ constexpr int kSuccNotify = -1;
 constexpr int kHotCompleted = 0;  // *layout.completed_operator
 constexpr int kHotTotal = 1;      // *layout.total_operator (never written during a run)
 constexpr int kHotAbort = 2;      // set when a bounded wait gave up
-constexpr int kHotExit = 3;       // 64 bits: workgroups that have left the current run | ops they completed << 32
+constexpr int kHotExit = 3;       // 64 bits: workgroups that have left the current run | those that left a run given up << 16 | ops they completed << 32
+constexpr unsigned int kExitQuit = 1u << 16;  // (a launch has fewer workgroups than that: graph_create checks)
 constexpr int kHotRun = 4;        // number of the current run (first run = 1), bumped by the last workgroup out
 constexpr int kHotWords = kHotRun + 1;
 
@@ -543,6 +544,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   __shared__ i32x4 s_facts;  // ... its part count, successor list and dependency counts (OpFacts)
   __shared__ long s_count;   // ... and its element count
   __shared__ int s_go;
+  __shared__ int s_quit;  // with s_go == 0: the workgroup leaves because the run was given up, not because the queues are empty
   __shared__ int s_last;
   __shared__ unsigned int s_done;  // ops this workgroup has completed (thread 0 only)
   if (threadIdx.x == 0) s_done = 0;
@@ -673,11 +675,15 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       i32x4 op_facts = {1, 0, 0, 0};
       long op_count = 0;
       size_t entry_index = 0;  // of e in the global order
+      int quit = 0;
       // claim entries until one needs the whole workgroup (COPY / REDUCE); signal ops
       // (NOTIFY / GET_NOTIFIED) are carried out right here by thread 0
       for (;;) {
         go = 0;
-        if (aborted) break;
+        if (aborted) {
+          quit = 1;
+          break;
+        }
         for (int i = 0; i < kQueues && !go; ++i) {
           const int q = (home + i) % kQueues;
           if (exhausted & (1u << q)) continue;
@@ -707,7 +713,14 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
             }
             if (t == 0 && q == 0) __hip_atomic_store(&hot[kHotCompleted].value, 0u, __ATOMIC_RELAXED, AGENT);
           } else {
-            exhausted |= 1u << q;
+            // A ticket came back without an entry.  The workgroup's own queue: go on to the next one, where
+            // the neighbouring XCD's workgroups may be behind (under load every other XCD of this part is a
+            // few per cent slower).  That one too: leave.  The queues run out at about the same time (entries
+            // are dealt round-robin), and asking all eight, a returning atomic each, one after the other, kept
+            // the last workgroups of every run for seven round trips with nothing to find.  Every queue keeps
+            // the workgroups it is home to until it is empty, so no entry is left behind; with fewer
+            // workgroups than queues some queue is nobody's home and every queue is asked.
+            exhausted |= (q != home && gridDim.x >= (unsigned int)kQueues) ? kAllQueues : (1u << q);
           }
         }
         if (!go) break;
@@ -738,6 +751,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
               return __hip_atomic_load(&g.ready[uid].value, __ATOMIC_RELAXED, AGENT) == n_pred;
             })) {
           go = 0;
+          quit = 1;
           break;
         }
         if (part_preds != 0) {
@@ -746,6 +760,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
                 return __hip_atomic_load(part_word, __ATOMIC_RELAXED, AGENT) == part_preds;
               })) {
             go = 0;
+            quit = 1;
             break;
           }
           __hip_atomic_store(part_word, 0u, __ATOMIC_RELAXED, AGENT);
@@ -762,6 +777,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
                 return (int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - want) >= 0;
               })) {
             go = 0;
+            quit = 1;
             break;
           }
         }
@@ -784,6 +800,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
         }
         if (gave_up) {
           go = 0;
+          quit = 1;
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
@@ -793,6 +810,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
       s_entry = e;
       cur_entry = e;
       s_go = go;
+      s_quit = quit;
       s_chain = chain_words;
       s_facts = op_facts;
       s_count = op_count;
@@ -859,22 +877,25 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
   }
 
   // leave: the last workgroup out re-arms the graph for the next run.  One returning atomic per
-  // workgroup carries both facts, "one more has left" (low word) and "it completed this many ops"
-  // (high word), so the last one out has the total without reading anything else.  No wait
+  // workgroup carries three facts: "one more has left" (bits 0-15), "it left because the run was given
+  // up" (counted in bits 16-31) and "it completed this many ops" (high word), so the last one out has
+  // the total and knows whether the run was given up without reading anything else.  No wait
   // stands before it: what the workgroup told others during the run (arrivals, counts put back for
   // the next run) has either been waited for where it mattered or only matters to the next launch.
   unsigned int total_done = 0;
+  bool aborted = false;
   if (threadIdx.x == 0) {
     unsigned long long *exits = (unsigned long long *)&hot[kHotExit].value;  // (the word has a 256-byte line to itself)
-    const unsigned long long before = __hip_atomic_fetch_add(exits, ((unsigned long long)s_done << 32) | 1ull, __ATOMIC_RELAXED, AGENT);
-    s_last = ((unsigned int)before == gridDim.x - 1);
+    const unsigned int quit = s_quit ? kExitQuit : 0u;
+    const unsigned long long before = __hip_atomic_fetch_add(exits, ((unsigned long long)s_done << 32) | (unsigned long long)(quit + 1u), __ATOMIC_RELAXED, AGENT);
+    s_last = (((unsigned int)before & (kExitQuit - 1u)) == gridDim.x - 1);
     total_done = (unsigned int)(before >> 32) + s_done;
+    aborted = (((unsigned int)before + quit) >> 16) != 0;
   }
   __syncthreads();
   if (!__builtin_amdgcn_readfirstlane(s_last)) return;
   if (threadIdx.x == 0) {
-    const bool aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT) != 0;
-    // after an abort the per-op state is inconsistent: leave it for the host to restore
+    // after a run that was given up the per-op state is inconsistent: leave it for the host to restore
     if (!aborted)
       for (int q = 0; q < kQueues; ++q) __hip_atomic_store(g.queue_head[q], 0, __ATOMIC_RELAXED, AGENT);
     __hip_atomic_store(&hot[kHotCompleted].value, total_done, __ATOMIC_RELAXED, AGENT);
