@@ -672,15 +672,17 @@ def test_rebind_refuses_a_move_that_breaks_element_alignment(hip, oracle):
     g.destroy()
 
 
-@pytest.mark.parametrize("block", ["1", "3", "32", "0"])
-def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, block):
+@pytest.mark.parametrize("block,last_level", [("1", "1"), ("3", "1"), ("32", "1"), ("0", "1"), ("3", "0")])
+def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, block, last_level):
     """Three chains of two many-part ops each (the second reads and overwrites what the first
     wrote, part by part) plus a single-part op: whatever the number of consecutive parts an op
     contributes to the queue order before the next op of its level takes its turn, the bits are
     those of the ops executed one after the other, and the order recorded by the timeline is
-    the blocked one."""
+    the blocked one; the last level goes op after op, longest parts first (PCCL_HIP_LAST_LEVEL=0:
+    in blocks like the others)."""
     import torch
     monkeypatch.setenv("PCCL_HIP_ORDER_BLOCK", block)
+    monkeypatch.setenv("PCCL_HIP_LAST_LEVEL", last_level)
     monkeypatch.setenv("PCCL_HIP_CHAINS", "0")  # every op queues its own entries: the order of those is the subject
     counts = [700 * 1000 + 3, 300 * 1000, 1000 * 1000 + 11]
     ops, want, outs = [], [], []
@@ -710,9 +712,10 @@ def test_ops_of_a_level_take_turns_in_blocks_of_parts(hip, oracle, monkeypatch, 
     # with `block` consecutive parts each
     n_parts = {u: int(part[uid == u].max()) + 1 for u in range(len(ops))}
     assert all(n_parts[c] == n_parts[3 + c] and n_parts[c] > 8 for c in range(3)) and n_parts[6] == 1
-    b = int(block) or 1 << 30
     expect = []
     for level_ops in ((0, 1, 2, 6), (3, 4, 5)):
+        # (ops 3, 4, 5 move the same bytes per part: "longest first" leaves them in their order)
+        b = 1 << 30 if level_ops[0] == 3 and last_level == "1" else (int(block) or 1 << 30)
         most = max(n_parts[u] for u in level_ops)
         for first in range(0, most, b):
             for u in level_ops:
