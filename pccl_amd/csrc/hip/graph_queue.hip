@@ -1241,6 +1241,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     }
   }
   C->spin_limit = G->spin_limit;
+  C->n_ops = (unsigned int)n_ops;
   C->queue_count = (const int *)(dev + off_qcount);
   C->chain = (const int *)(dev + off_chain);
   C->chain_table = (const ForwardStep *)(dev + off_chain_table);
@@ -1257,6 +1258,9 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   {
     long long t = 0;
     const int block = order_block();
+    // (PCCL_HIP_COUNT_ALL=1: also the parts of ops that nobody waits for are counted, see kEntryUncounted)
+    const char *count_env = getenv("PCCL_HIP_COUNT_ALL");
+    const int count_all_parts = count_env && count_env[0] == '1';
     for (int lo = 0; lo < n_ops;) {
       int hi = lo, most = 0;
       while (hi < n_ops && level[by_level[hi]] == level[by_level[lo]]) most = std::max(most, parts[by_level[hi++]]);
@@ -1280,7 +1284,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
           for (int p = first; p < (int)std::min<long long>((long long)first + step, parts[i]); ++p, ++t)
             qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32) |
                                       ((G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 || G->wait_of[i] >= 0 || G->notify_of[i] >= 0) ? kEntryChainHead : 0ull) |
-                                      (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull) | (notifies_by_part(i) ? kEntryNotifiesPart : 0ull));
+                                      (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull) | (notifies_by_part(i) ? kEntryNotifiesPart : 0ull) |
+                                      ((count_all_parts == 0 && n_succ[chain_tail[i]] == 0 && n_pred[i] == n_part_pred[i]) ? kEntryUncounted : 0ull));
         }
       lo = hi;
     }

@@ -56,6 +56,7 @@ struct GraphControl {
                                           // (chains do not) can change with the operands' addresses, and what is in
                                           // this block is frozen into any launch that a stream capture has recorded
   unsigned int spin_limit;
+  unsigned int n_ops;
 };
 
 // An op of many parts does not count them on one word: atomics on one address are carried out
@@ -88,7 +89,14 @@ constexpr unsigned long long kEntryChainHead = 1ull << 51;
 constexpr unsigned long long kEntryWaitsSignal = 1ull << 52;
 // ... | (whoever completes the part stores the part's signal word) << 53: the op carries a NOTIFY of one word per part.
 constexpr unsigned long long kEntryNotifiesPart = 1ull << 53;
-constexpr unsigned long long kEntryFlags = kEntryChainHead | kEntryWaitsSignal | kEntryNotifiesPart;
+// ... | (the part is not counted) << 54.  An op that nothing in the graph waits for, and that waits for no
+// whole op itself (its arrivals word is never written, so there is nothing to put back), is not counted
+// part by part: nobody would read the count.  Its completion is the run's: when every workgroup has left
+// and none gave up, every entry has been carried out, and the last workgroup out reports all ops
+// complete.  That takes one or two returning atomics out of the end of every workgroup whose last entry
+// is such an op: all of them in graphs of independent ops and chains.
+constexpr unsigned long long kEntryUncounted = 1ull << 54;
+constexpr unsigned long long kEntryFlags = kEntryChainHead | kEntryWaitsSignal | kEntryNotifiesPart | kEntryUncounted;
 // In a successor list: not an op, but "store the signal word of the NOTIFY this op carries".
 constexpr int kSuccNotify = -1;
 
@@ -665,7 +673,11 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           __hip_atomic_store((unsigned int *)f->notify_word + cur_part, base_of_run() + (f->notify_value & kSignalValue),
                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
-        finish_part(g, h, cur_op, cur_uid, cur_part, &s_done, cur_chain_ops, draw_ticket, notify);
+        // (a part that is not counted goes the way of a single-part op without successors: nothing but the next ticket)
+        OpFacts counted = cur_op;
+        const bool uncounted = (cur_entry & kEntryUncounted) != 0;
+        if (uncounted) counted.parts = 1;
+        finish_part(g, h, counted, cur_uid, cur_part, &s_done, uncounted ? 0 : cur_chain_ops, draw_ticket, notify);
       } else {
         draw_ticket();
       }
@@ -804,7 +816,7 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
           break;
         }
         if (cur_trace) cur_trace[kTraceDone] = wall_clock64();
-        finish_part(g, hc, OpFacts::of(sc), uid, 0, &s_done, 1, [] {}, notify);
+        if (!(e & kEntryUncounted)) finish_part(g, hc, OpFacts::of(sc), uid, 0, &s_done, 1, [] {}, notify);
         aborted = __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, AGENT);
       }
       s_entry = e;
@@ -878,8 +890,8 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
 
   // leave: the last workgroup out re-arms the graph for the next run.  One returning atomic per
   // workgroup carries three facts: "one more has left" (bits 0-15), "it left because the run was given
-  // up" (counted in bits 16-31) and "it completed this many ops" (high word), so the last one out has
-  // the total and knows whether the run was given up without reading anything else.  No wait
+  // up" (counted in bits 16-31) and "it completed this many of the ops that are counted" (high word), so
+  // the last one out knows whether the run was given up, and what to report, without reading anything else.  No wait
   // stands before it: what the workgroup told others during the run (arrivals, counts put back for
   // the next run) has either been waited for where it mattered or only matters to the next launch.
   unsigned int total_done = 0;
@@ -889,8 +901,9 @@ __device__ __forceinline__ void drain_body(const GraphControl &g) {
     const unsigned int quit = s_quit ? kExitQuit : 0u;
     const unsigned long long before = __hip_atomic_fetch_add(exits, ((unsigned long long)s_done << 32) | (unsigned long long)(quit + 1u), __ATOMIC_RELAXED, AGENT);
     s_last = (((unsigned int)before & (kExitQuit - 1u)) == gridDim.x - 1);
-    total_done = (unsigned int)(before >> 32) + s_done;
     aborted = (((unsigned int)before + quit) >> 16) != 0;
+    // (after a run that nobody gave up every op is complete, also those that are not counted: finish_part)
+    total_done = aborted ? (unsigned int)(before >> 32) + s_done : g.n_ops;
   }
   __syncthreads();
   if (!__builtin_amdgcn_readfirstlane(s_last)) return;
