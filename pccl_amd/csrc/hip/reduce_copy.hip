@@ -110,7 +110,13 @@ extern "C" int pccl_hip_reduce_copy(int dtype, int compute, const void *const *i
   const bool big = total_bytes > (192l << 20);
   int mem = kLaunchMemCached;
   if (total_bytes >= (48l << 20)) {
-    const bool non_temporal_stores = (n_in == 1 && n_out >= 3) || (n_in >= 3 && total_bytes > (4l << 30));
+    // (three and four inputs already from 1.4 GiB in all, i32, three allocations each, write-through vs
+    // non-temporal: 4 -> 1 at 256 MiB per operand 6.82 vs 6.56 but at 320 MiB 6.44 vs 6.58, 384 MiB 6.47 vs
+    // 6.66, 512 MiB 6.44 vs 6.63, 768 MiB 6.51 vs 6.57; 3 -> 1 at 256 MiB 7.27 vs 6.73 but at 384 MiB 6.59 vs
+    // 6.75, 512 MiB 6.56 vs 6.65, 1 GiB 6.46 vs 6.56; five to eight inputs keep write-through stores up
+    // to 4 GiB: 5 -> 1 at 320 MiB 6.68 vs 6.62, 7 -> 1 at 384 MiB 6.75 vs 6.75, 8 -> 1 at 256 MiB 6.86 vs 6.56)
+    const bool few_inputs_large = (n_in == 3 || n_in == 4) && n_out == 1 && total_bytes >= (1408l << 20);
+    const bool non_temporal_stores = (n_in == 1 && n_out >= 3) || few_inputs_large || (n_in >= 3 && total_bytes > (4l << 30));
     mem = non_temporal_stores ? kLaunchMemStream : kLaunchMemStreamWriteThrough;
   }
   if (t.cache_treatment >= 0) mem = std::min(t.cache_treatment, (int)kLaunchMemStreamWriteThrough);
