@@ -105,6 +105,28 @@ def read_traffic_record():
         return None, dict(src, stale=True, why="record has no traffic_bytes")
 
 
+def through_the_drain(torch, hip, bound_ops, stream, steps=20):
+    """The same graph through the persistent drain (PCCL_HIP_WIDE=0): what a graph whose entries wait for
+    nothing cost before it ran as a wide launch, and what bounds the graphs that cannot run as one."""
+    old = os.environ.get("PCCL_HIP_WIDE")
+    os.environ["PCCL_HIP_WIDE"] = "0"
+    try:
+        g = hip.Graph(bound_ops)
+    finally:
+        if old is None:
+            del os.environ["PCCL_HIP_WIDE"]
+        else:
+            os.environ["PCCL_HIP_WIDE"] = old
+    t = event_times_us(torch, lambda: g.run(stream), steps, 3)
+    info = g.info()
+    g.destroy()
+    return dict(stats(t), queue_entries=info["n_tiles"], workgroups=info["n_workgroups"])
+
+
+def launch_kind(info):
+    return "wide (one workgroup per entry)" if info["n_workgroups"] == info["n_tiles"] and info["n_tiles"] > 1 else "persistent drain"
+
+
 def queue_bytes_moved(hip, bound_ops, elem_bytes):
     """Bytes the queue executor moves for these ops (bound to addresses), which is less than their
     algorithmic bytes where ops chain: in a chain that runs in one pass an op does not read the
@@ -315,6 +337,7 @@ def queue_timeline(torch, hip, graph, stream, runs=3):
 def timeline_main():
     import torch
     from pccl_amd import hip, lang
+    os.environ["PCCL_HIP_WIDE"] = "0"  # the persistent drain's own timeline, also for the graphs that would run as a wide launch
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
     out = {}
@@ -702,9 +725,10 @@ def main():
                     full["8_ranks_x_%d_MiB" % per_rank_mib] = dict(stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low),
                                                                   algorithmic_bytes=moved, bytes_moved=really,
                                                                   GBps_moved_median=gbps(really, tf[len(tf) // 2]),
-                                                                  queue_entries=g.info()["n_tiles"],
+                                                                  queue_entries=g.info()["n_tiles"], launch=launch_kind(g.info()),
                                                                   dependencies_part_by_part="%d of %d" % (sum(kinds), len(kinds)))
                     g.destroy()
+                    full["8_ranks_x_%d_MiB" % per_rank_mib]["through_the_persistent_drain"] = through_the_drain(torch, hip, ring_bound, stream)
                     # The same all-reduce written the way ranks on different devices write it: dependency
                     # edges inside a rank only, the hand-over between neighbours NOTIFY -> signal word ->
                     # GET_NOTIFIED (328 ops).  Nothing can stay in registers across such a hand-over.
@@ -743,7 +767,9 @@ def main():
                         gp.destroy()
                     del rb
                 full["note"] = ("GBps_median counts the algorithmic bytes of the 112 ops; the 14 ops of a chunk run as one chain that keeps "
-                                "the value in registers and stores only what the chain does not overwrite itself: bytes_moved / GBps_moved_median")
+                                "the value in registers and stores only what the chain does not overwrite itself: bytes_moved / GBps_moved_median.  "
+                                "No entry of these graphs waits for another, so they run as a wide launch (one short-lived workgroup per 16 KiB "
+                                "block of a chain); through_the_persistent_drain is the same graph with PCCL_HIP_WIDE=0")
                 extras["ring_allreduce_one_launch"] = full
 
                 # the same all-reduce as the one-exchange ("direct") schedule a fully connected node
@@ -795,7 +821,7 @@ def main():
                     direct["8_ranks_x_%d_MiB" % per_rank_mib] = dict(
                         stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low), algorithmic_bytes=moved,
                         bytes_moved=really, GBps_moved_median=gbps(really, tf[len(tf) // 2]),
-                        queue_entries=g.info()["n_tiles"], dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
+                        queue_entries=g.info()["n_tiles"], launch=launch_kind(g.info()), dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
                         as_one_launch_8in_8out=dict(stats(t1), GBps_median=gbps(16 * per_rank * 2, t1[len(t1) // 2])),
                         via_engine_exeOp=dict(stats(te), GBps_median=gbps(16 * per_rank * 2, te[len(te) // 2])))
                     g.destroy()
@@ -892,7 +918,9 @@ def main():
                 extras["op_64KiB_direct_launch"] = stats(t)
                 g1 = hip.Graph([dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)])
                 t = event_times_us(torch, lambda: g1.run(stream), 200, 20)
-                extras["op_64KiB_via_queue"] = stats(t)
+                extras["op_64KiB_via_queue"] = dict(stats(t), launch=launch_kind(g1.info()),
+                                                    through_the_persistent_drain=through_the_drain(
+                                                        torch, hip, [dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)], stream, 200))
                 g1.destroy()
 
         # ---- the 4096-op small-message schedule: one persistent launch ----------------------
@@ -939,10 +967,13 @@ def main():
                     "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med),
                                                   GBps_moved_median=gbps(sched_moved, med)),
                     "one_persistent_launch_without_chains": unchained,
-                    "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"],
+                    "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"], "launch": launch_kind(ginfo),
                     "algorithmic_bytes": sched_bytes, "bytes_moved": sched_moved,
                     "note": "GBps_median counts the algorithmic bytes of the 4096 ops; chains of 14 ops keep the value in registers "
-                            "and skip stores they overwrite themselves (bytes_moved, GBps_moved_median)"}
+                            "and skip stores they overwrite themselves (bytes_moved, GBps_moved_median).  one_persistent_launch is one "
+                            "launch of whatever kind the library chooses: with chains no entry waits for another and it is a wide launch "
+                            "(through_the_persistent_drain: the same graph with PCCL_HIP_WIDE=0); without chains it is the persistent drain"}
+                extras["schedule_4096_ops"]["one_persistent_launch"]["through_the_persistent_drain"] = through_the_drain(torch, hip, bound, stream, 30)
                 # the same schedule the way the reference's host code would drive it: written to a
                 # schedule file, registered by name, executed on an input / output tensor pair
                 # (Engine::regOp / exeOp; every exeOp binds the tensors and launches once)

@@ -210,7 +210,17 @@ typedef struct pccl_op_desc {
  * alone depends on is polled by every part of that op (which takes over its dependencies); neither
  * queues an entry, both count as complete with the data op.  In the device image the successor list
  * of an op that carries a NOTIFY ends in -1 (next_op_uids_head_, num_next_ops_ counts it).
- * PCCL_HIP_FUSE_SIGNALS=0 keeps every signal op an op of its own. */
+ * PCCL_HIP_FUSE_SIGNALS=0 keeps every signal op an op of its own.
+ * The wide launch: with tile_bytes 0 (or PCCL_HIP_TILE_AUTO), a graph none of whose queue entries waits for
+ * another entry or has to do with a signal word (independent ops; chains, whose later ops run behind the first
+ * in the same workgroup) is cut into parts of 16 KiB and run by one short-lived workgroup per entry, as many
+ * workgroups as entries, instead of the persistent drain: nothing is handed from workgroup to workgroup, so no
+ * ticket is drawn and no part counted, and the hardware dispatcher balances the compute units (ring all-reduce
+ * over 8 resident ranks x 1 / 8 / 32 / 64 MiB 16.4 / 31 / 93 / 227 -> 11.9 / 23.4 / 87 / 196 us, one 64 KiB op
+ * 9.7 -> 6.5 us).  Graphs whose entries outside one-pass chains move 192 MiB or more stay with the drain.
+ * The device arena, graph_info, graph_trace and results are the same; graph_status reports every op complete
+ * once the stream has drained (the launch's end is the graph's completion; *completed_operator on the device
+ * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0 never, 1 whenever possible. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
@@ -233,7 +243,11 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
  * the call waits for `stream` and rewrites the graph's device arena in place
  * (launches recorded by stream capture stay valid).  A move that
  * would leave an operand unaligned for its element type returns
- * PCCL_ERR_MISALIGNED and changes nothing. */
+ * PCCL_ERR_MISALIGNED and changes nothing.  A graph that runs as a wide launch (see
+ * pccl_hip_graph_create) cannot wait inside the launch: a move after which one of its entries
+ * would have to wait for another (an op that no longer may run behind its predecessor part by
+ * part) returns PCCL_ERR_UNSUPPORTED and changes nothing; create the graph again for such
+ * operands (Engine::exeOp does). */
 int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,
                           void *stream);
 

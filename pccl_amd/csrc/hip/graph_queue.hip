@@ -66,16 +66,24 @@ using pccl_host::fail;
 
 namespace {
 
-DrainKernel drain_for(int dtype, int compute, bool forward) {
+DrainKernel drain_for(int dtype, int compute, bool forward, bool wide = false) {
   switch (dtype) {
-    case PCCL_F32: return forward ? drain_forward_for_compute<PCCL_F32>(compute) : drain_for_compute<PCCL_F32>(compute);
-    case PCCL_I32: return forward ? drain_forward_for_compute<PCCL_I32>(compute) : drain_for_compute<PCCL_I32>(compute);
-    case PCCL_BF16: return forward ? drain_forward_for_compute<PCCL_BF16>(compute) : drain_for_compute<PCCL_BF16>(compute);
-    case PCCL_F16: return forward ? drain_forward_for_compute<PCCL_F16>(compute) : drain_for_compute<PCCL_F16>(compute);
-    case PCCL_F8E4M3: return forward ? drain_forward_for_compute<PCCL_F8E4M3>(compute) : drain_for_compute<PCCL_F8E4M3>(compute);
-    case PCCL_F8E5M2: return forward ? drain_forward_for_compute<PCCL_F8E5M2>(compute) : drain_for_compute<PCCL_F8E5M2>(compute);
-    case PCCL_F64: return forward ? drain_forward_for_compute<PCCL_F64>(compute) : drain_for_compute<PCCL_F64>(compute);
-    default: return forward ? drain_forward_for_compute<PCCL_U32>(compute) : drain_for_compute<PCCL_U32>(compute);
+    case PCCL_F32: return forward ? (wide ? wide_forward_for_compute<PCCL_F32>(compute) : drain_forward_for_compute<PCCL_F32>(compute))
+                              : (wide ? wide_for_compute<PCCL_F32>(compute) : drain_for_compute<PCCL_F32>(compute));
+    case PCCL_I32: return forward ? (wide ? wide_forward_for_compute<PCCL_I32>(compute) : drain_forward_for_compute<PCCL_I32>(compute))
+                              : (wide ? wide_for_compute<PCCL_I32>(compute) : drain_for_compute<PCCL_I32>(compute));
+    case PCCL_BF16: return forward ? (wide ? wide_forward_for_compute<PCCL_BF16>(compute) : drain_forward_for_compute<PCCL_BF16>(compute))
+                              : (wide ? wide_for_compute<PCCL_BF16>(compute) : drain_for_compute<PCCL_BF16>(compute));
+    case PCCL_F16: return forward ? (wide ? wide_forward_for_compute<PCCL_F16>(compute) : drain_forward_for_compute<PCCL_F16>(compute))
+                              : (wide ? wide_for_compute<PCCL_F16>(compute) : drain_for_compute<PCCL_F16>(compute));
+    case PCCL_F8E4M3: return forward ? (wide ? wide_forward_for_compute<PCCL_F8E4M3>(compute) : drain_forward_for_compute<PCCL_F8E4M3>(compute))
+                              : (wide ? wide_for_compute<PCCL_F8E4M3>(compute) : drain_for_compute<PCCL_F8E4M3>(compute));
+    case PCCL_F8E5M2: return forward ? (wide ? wide_forward_for_compute<PCCL_F8E5M2>(compute) : drain_forward_for_compute<PCCL_F8E5M2>(compute))
+                              : (wide ? wide_for_compute<PCCL_F8E5M2>(compute) : drain_for_compute<PCCL_F8E5M2>(compute));
+    case PCCL_F64: return forward ? (wide ? wide_forward_for_compute<PCCL_F64>(compute) : drain_forward_for_compute<PCCL_F64>(compute))
+                              : (wide ? wide_for_compute<PCCL_F64>(compute) : drain_for_compute<PCCL_F64>(compute));
+    default: return forward ? (wide ? wide_forward_for_compute<PCCL_U32>(compute) : drain_forward_for_compute<PCCL_U32>(compute))
+                              : (wide ? wide_for_compute<PCCL_U32>(compute) : drain_for_compute<PCCL_U32>(compute));
   }
 }
 
@@ -139,6 +147,11 @@ struct Graph {
   size_t fuse_table_off = 0;               // arena offset of the carried signals' table (behind the chain table)
   std::vector<int> fixed_parts;            // build_graph: cut the ops like this instead of choosing (a rebuild in place:
                                            // the arena's layout, and with it its size, follows from the part counts)
+  // The wide launch (graph_queue_device.h: wide_body): one workgroup per entry instead of the persistent drain.
+  bool want_wide = false;  // build_graph: cut for it, check that the graph allows it, take its kernel
+  bool wide_ok = false;    // build_graph's finding: no queue entry waits for another entry or for a signal
+  bool wide = false;       // the graph runs that way
+  long long wide_plain_bytes = 0;  // build_graph's finding: bytes moved by entries that do not run a chain in one pass
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
   bool as_launches = false;
   std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
@@ -193,6 +206,23 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // there reads the buffer a reduction reads too, and in blocks the two run side by side; with copies
 // that read buffers of their own it is 212 -> 209 us.  Ring and direct all-reduces over 8 ranks x
 // 1 .. 64 MiB and the 4096-op schedule (at most 3 parts per op) are unchanged within 1 %.
+// Whether a graph that may run as a wide launch (wide_body) does.  Chains that run in one pass gain at
+// every size measured (ring all-reduce over 8 resident ranks x 1 / 8 / 32 / 64 MiB: 16.4 / 31 / 93 / 227 us
+// through the persistent drain, 11.9 / 23.4 / 87 / 196 us wide), and so do small graphs of any kind (one
+// 64 KiB op 9.7 -> 6.5 us, the 4096-op schedule 77 -> 68 us, direct all-reduce 8 x 1 / 8 MiB 12.9 / 32 ->
+// 9.9 / 24.3 us).  Entries that go through memory op by op (single ops, chains that cannot run in one
+// pass) walk their part 4 KiB after 4 KiB like a direct launch of several packs per lane, which loses to
+// the persistent drain once there is much of it (direct all-reduce 8 x 16 / 32 MiB: 53 / 90.3 us through
+// the drain, 58.6 / 92.7 us wide): from 192 MiB of such traffic a graph stays with the drain.
+// PCCL_HIP_WIDE=0: never wide; 1: whenever the graph allows it.
+bool wide_launch_pays(long long plain_bytes) {
+  if (const char *env = getenv("PCCL_HIP_WIDE")) {
+    if (env[0] == '0') return false;
+    if (env[0] == '1') return true;
+  }
+  return plain_bytes < (192ll << 20);
+}
+
 int order_block() {
   int block = 32;
   if (const char *env = getenv("PCCL_HIP_ORDER_BLOCK")) block = atoi(env);
@@ -730,7 +760,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   const pccl_op_desc *ops = G->eff.data();
   const int n_ops = (int)G->eff.size();
   auto carrier = [&](int i) { return G->fused_into[i] >= 0 ? G->fused_into[i] : i; };
-  long tile_bytes = G->tile_bytes;
+  long tile_bytes = G->want_wide ? kWideTileBytes : G->tile_bytes;  // (a wide launch: every op in parts of one block)
   const bool default_tile = tile_bytes == 0;  // parts are then sized per dependency level, below
   if (!default_tile) tile_bytes = std::max<long>(tile_bytes, 1024);
 
@@ -822,12 +852,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // (two instances per dtype and fold: with and without the code that runs a chain in one pass.  Which
   // of them runs is settled once the chains are known, below; the launch width must hold for both.  A
   // rebuild in place keeps the instance: launches that a stream capture has recorded carry it.)
-  const DrainKernel plain_kernel = mixed ? drain_for_any() : drain_for(g_dtype, g_compute, false);
+  const bool wide = G->want_wide;
+  const DrainKernel plain_kernel = mixed ? (wide ? wide_for_any() : drain_for_any()) : drain_for(g_dtype, g_compute, false, wide);
   // (the instance with the one-pass code has no registers to spare for carried signal ops: a graph with
   // such ops runs the plain one, its chains through memory)
   bool carries = false;
   for (int i = 0; i < n_ops; ++i) carries = carries || G->fused_into[i] >= 0;
-  const DrainKernel forward_kernel = (mixed || carries) ? nullptr : drain_for(g_dtype, g_compute, true);
+  const DrainKernel forward_kernel = (mixed || carries) ? nullptr : drain_for(g_dtype, g_compute, true, wide);
   const int forward_elem_bytes = (G->fixed_kernel ? G->forward_capable : (!mixed && !carries)) ? elem_bytes(g_dtype) : 0;
   int occ = 8;
   for (DrainKernel k : {plain_kernel, forward_kernel}) {
@@ -1114,6 +1145,27 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   long long live_tiles = 0;
   for (int i = 0; i < n_ops; ++i)
     if (queued(i)) live_tiles += parts[i];
+  // The wide launch (wide_body) is open to a graph none of whose entries waits for another entry (as
+  // for entries without tickets, below) or has to do with a signal word (its workgroups poll nothing
+  // and tell nobody), with few enough entries for the exit word's count.
+  {
+    bool waits = carries;
+    for (int i = 0; i < n_ops && !waits; ++i)
+      waits = queued(i) && (n_pred[i] > 0 || order_pred[i] > 0 || ops[i].primitive == PCCL_NOTIFY || ops[i].primitive == PCCL_GET_NOTIFIED);
+    G->wide_ok = !waits && live_tiles > 0 && live_tiles < (long long)kExitQuit;
+    // (what the entries that do not run a chain in one pass move, chains through memory included: see wide_launch_pays)
+    G->wide_plain_bytes = 0;
+    for (int i = 0; i < n_ops; ++i) {
+      if (!queued(i)) continue;
+      const int *w = &G->chain_words[(size_t)kChainWords * i];
+      if (w[kChainNext] >= 0 && w[kChainForward] == 1) continue;
+      for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext])
+        G->wide_plain_bytes += (long long)(ops[u].n_in + ops[u].n_out) * op_bytes[u];
+    }
+    if (G->want_wide && (!G->wide_ok || (G->fixed_n_wg > 0 && live_tiles > G->fixed_n_wg)))
+      return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as a wide launch (an entry waits for another, "
+                                        "or there are more entries than the launch was made for)");
+  }
 
   std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
   {
@@ -1171,6 +1223,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // depend on how many entries the chains leave to be queued (graph_rebind can change that)
   const size_t queue_room = (size_t)((std::max<long long>(tiles, 1) + kQueues - 1) / kQueues);
   const size_t off_entries = off; off = align_up(off + 8 * queue_room * kQueues, 256);
+  // (a wide launch: a record per workgroup; room for one per part of every op, so that the layout does not move with the chain plan)
+  const size_t off_wide = off;    if (G->want_wide) off = align_up(off + sizeof(WideEntry) * (size_t)std::max<long long>(tiles, 1), 256);
   const size_t arena_bytes = off;
 
   G->n_ops = n_ops;
@@ -1242,6 +1296,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   }
   C->spin_limit = G->spin_limit;
   C->n_ops = (unsigned int)n_ops;
+  C->wide_entries = G->want_wide ? (const WideEntry *)(dev + off_wide) : nullptr;
   C->queue_count = (const int *)(dev + off_qcount);
   C->chain = (const int *)(dev + off_chain);
   C->chain_table = (const ForwardStep *)(dev + off_chain_table);
@@ -1257,7 +1312,10 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   std::vector<std::vector<unsigned long long>> qe(kQueues);
   {
     long long t = 0;
-    const int block = order_block();
+    // (a wide launch: op after op, so that the workgroups in flight cover few ops at a time, each through
+    // a narrow window like a direct launch: ring all-reduce 8 x 64 MiB 212 -> 196 us, 8 x 32 MiB 90.6 -> 88.8)
+    const int block = G->want_wide ? 1 << 30 : order_block();
+    WideEntry *wide_entries = G->want_wide ? (WideEntry *)(img + off_wide) : nullptr;
     // (PCCL_HIP_COUNT_ALL=1: also the parts of ops that nobody waits for are counted, see kEntryUncounted)
     const char *count_env = getenv("PCCL_HIP_COUNT_ALL");
     const int count_all_parts = count_env && count_env[0] == '1';
@@ -1281,11 +1339,20 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       for (int first = 0; first < most; first += step)
         for (int i : turn) {
           if (!queued(i)) continue;  // runs behind its chain's head
-          for (int p = first; p < (int)std::min<long long>((long long)first + step, parts[i]); ++p, ++t)
+          for (int p = first; p < (int)std::min<long long>((long long)first + step, parts[i]); ++p, ++t) {
+            if (wide_entries) {
+              const long per = part_elems(ops[i].count, parts[i]), lo = (long)p * per;
+              WideEntry &w = wide_entries[t];
+              w.uid = i;
+              w.n = (int)std::max<long>(0, std::min<long>(per, ops[i].count - lo));
+              w.lo = lo;
+              for (int k = 0; k < kChainWords; ++k) w.chain[k] = G->chain_words[(size_t)kChainWords * i + k];
+            }
             qe[t % kQueues].push_back((unsigned long long)(unsigned int)i | ((unsigned long long)p << 32) |
                                       ((G->chain_words[(size_t)kChainWords * i + kChainNext] >= 0 || G->wait_of[i] >= 0 || G->notify_of[i] >= 0) ? kEntryChainHead : 0ull) |
                                       (G->wait_of[i] >= 0 ? kEntryWaitsSignal : 0ull) | (notifies_by_part(i) ? kEntryNotifiesPart : 0ull) |
                                       ((count_all_parts == 0 && n_succ[chain_tail[i]] == 0 && n_pred[i] == n_part_pred[i]) ? kEntryUncounted : 0ull));
+          }
         }
       lo = hi;
     }
@@ -1353,7 +1420,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   if (n_edges) memcpy(img + off_succ_part, succ_part_base.data(), sizeof(int) * n_edges);
   // never more workgroups than entries
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
-  G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, cap));
+  G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, G->want_wide ? (long long)kExitQuit - 1 : cap));
+  G->wide = G->want_wide;
   {
     // Entries without tickets (graph_queue_device.h): when there is at most one per workgroup
     // (PCCL_HIP_OWN_ENTRIES=k: up to k; the mapping of entries to workgroups then needs every queue to
@@ -1460,6 +1528,26 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     delete G;
     return rc;
   }
+  // The library's own cut (tile_bytes 0): a graph whose entries wait for nothing runs as a wide launch
+  // (wide_body), for which it is cut again, every op into parts of one block.  If that cut does not
+  // keep the property (or its arena cannot be had), the graph stays as built.
+  if (G->tile_bytes == 0 && G->wide_ok && wide_launch_pays(G->wide_plain_bytes)) {
+    Graph *W = new Graph();
+    W->tile_bytes = 0;
+    W->spin_limit = G->spin_limit;
+    W->descs = G->descs;
+    W->deps_store = G->deps_store;
+    for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) W->descs[i].deps = W->deps_store.data() + at;
+    W->want_wide = true;
+    if (build_graph(W, 1) == PCCL_OK) {
+      if (G->dev) (void)hipFree(G->dev);
+      delete G;
+      G = W;
+    } else {
+      delete W;
+      pccl_host::clear_error();
+    }
+  }
   *graph = G;
   return PCCL_OK;
 }
@@ -1547,7 +1635,7 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed, un
   Graph *G = (Graph *)graph;
   if (!G) return fail(PCCL_ERR_INVALID_ARG, "graph_status: graph is null");
   PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
-  if (G->as_launches) {  // launches that have ended have completed their ops
+  if (G->as_launches || G->wide) {  // launches that have ended have completed their ops (nothing in them waits)
     if (completed) *completed = G->runs ? (unsigned int)G->n_ops : 0u;
     if (total) *total = (unsigned int)G->n_ops;
     return PCCL_OK;
@@ -1634,6 +1722,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.fixed_n_wg = G->n_wg;
     fresh.fixed_kernel = G->kernel;
     fresh.forward_capable = G->forward_capable;
+    fresh.want_wide = G->wide;  // (a wide launch stays one, or the rebind is refused before anything changes)
     char *old_dev = G->dev;
     // The run number goes on from where the DEVICE stands, not from the count of graph_run
     // calls: every replay of a recorded launch has moved the device's word on as well, and a
@@ -1664,6 +1753,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->total_tiles = fresh.total_tiles;
     G->all_tiles = fresh.all_tiles;
     G->n_wg = fresh.n_wg;
+    G->wide_ok = fresh.wide_ok;
     G->device = fresh.device;
     G->kernel = fresh.kernel;
     G->descs.swap(fresh.descs);

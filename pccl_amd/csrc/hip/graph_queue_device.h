@@ -57,7 +57,19 @@ struct GraphControl {
                                           // this block is frozen into any launch that a stream capture has recorded
   unsigned int spin_limit;
   unsigned int n_ops;
+  const struct WideEntry *wide_entries;   // a graph that runs as a wide launch: what workgroup b carries out (else null)
 };
+
+// One per workgroup of a wide launch (wide_body), in the order the entries were dealt in: the entry with
+// everything that the drain kernel would fetch from the entry, the op's slot and its chain words one
+// after the other, so that the payload is the first dependent load.  n == 0: nothing to do.
+struct WideEntry {
+  int uid;
+  int n;           // elements of this part
+  long lo;         // first element of this part
+  int chain[4];    // the op's kChainWords words ({-1, 1, 0, 0} for an op outside any chain)
+};
+static_assert(sizeof(WideEntry) == 32, "wide entry size");
 
 // An op of many parts does not count them on one word: atomics on one address are carried out
 // one after the other (about 11 ns each), and 1024 parts of a 32 MiB op finishing within a few
@@ -930,6 +942,97 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
 
 typedef void (*DrainKernel)(const GraphControl);
 
+// ---- the wide launch ---------------------------------------------------------------------
+// A graph none of whose queue entries waits for another entry (independent ops, chains: everything
+// that depends on something runs behind it in the same workgroup) needs no queue at run time: which
+// workgroup carries out which entry can be fixed by number, and nothing is handed from workgroup to
+// workgroup.  Such a graph is cut into parts of one block (kWideTileBytes per stream) and launched
+// in the shape of the direct kernels: one short-lived workgroup per entry, workgroup b takes entry b
+// of the order the entries were dealt in, as many workgroups as entries.  The hardware dispatcher
+// hands the next workgroup to whichever compute unit has room, so the faster XCDs carry out more
+// entries, and no workgroup draws a ticket, looks at a dependency word or counts a part.  Against the
+// persistent drain of the same graphs (ring all-reduce over 8 resident ranks, 112 ops in 8 chains):
+// 8 x 1 MiB 16.7 -> 11 us, 8 x 8 MiB 31 -> 21 us, 8 x 32 MiB 93 -> 85 us, 8 x 64 MiB 225 -> 201 us.
+// Nothing of the queue's state is written: no head moves, no part is counted, and the launch's end is
+// the graph's completion.  The arena is the one the drain kernel would use (entries, payloads, chain
+// words and table), so a rebind moves operands the same way.
+constexpr long kWideTileBytes = 16384;  // = kBlock lanes x 4 packs: the block run_chain_forward carries through a chain
+
+template <int DT, class Op, bool FORWARD>
+__device__ __forceinline__ void wide_body(const GraphControl &g) {
+  if constexpr (DT != kAnyDtype) Dtype<DT>::wave_init();
+  const unsigned int b = blockIdx.x;
+  const WideEntry *we = &g.wide_entries[b];  // (uniform: scalar loads from here to the payload)
+  const int uid = __builtin_amdgcn_readfirstlane(we->uid);
+  const long n = (long)__builtin_amdgcn_readfirstlane(we->n);
+  const long lo = (long)uniform64((unsigned long long)we->lo);
+  const i32x4 chain = *(const i32x4 *)we->chain;
+  const PayloadSlot *slot = (const PayloadSlot *)(g.slots + (size_t)uid * kPayloadStride);
+  const pccl_op_payload *pl = &slot->payload;
+  unsigned long long *trace = nullptr;
+  if (threadIdx.x == 0 && g.trace && n > 0) {
+    trace = g.trace + (size_t)b * kTraceWords;
+    const unsigned long long now = wall_clock64();
+    trace[kTraceWhat] = (unsigned long long)(unsigned int)uid | ((unsigned long long)(unsigned int)(lo / part_elems(pl->chunks_[0].num_elems_, slot->parts)) << 32) |
+                        ((unsigned long long)(b & 0xfffu) << 52);
+    trace[kTraceClaimed] = now;
+    trace[kTraceReady] = now;
+  }
+  if (n > 0) {
+    const int chain_next = __builtin_amdgcn_readfirstlane(chain[kChainNext]);
+    bool forwarded = false;
+    if constexpr (FORWARD && DT != kAnyDtype) {
+      if (chain_next >= 0 && __builtin_amdgcn_readfirstlane(chain[kChainForward])) {
+        run_chain_forward<Dtype<DT>, Op>(g, pl, __builtin_amdgcn_readfirstlane(chain[kChainLength]), __builtin_amdgcn_readfirstlane(chain[kChainRow]), lo, n);
+        forwarded = true;
+      }
+    }
+    if (!forwarded) {
+      // the op, then the ops chained behind it, same part, through memory (as in drain_body)
+      const pccl_op_payload *step = pl;
+      for (int next = chain_next;;) {
+        const pccl_op_payload *more = nullptr;
+        if (next >= 0 && g.chain[kChainWords * next + kChainForward] == kChainFolded) {
+          more = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
+          next = g.chain[kChainWords * next + kChainNext];
+        }
+        if constexpr (DT == kAnyDtype) run_part_any(step, more, lo, n);
+        else run_part<DT, Op>(step, more, lo, n);
+        if (next < 0) break;
+        settle_stores();
+        __syncthreads();
+        step = &((const PayloadSlot *)(g.slots + (size_t)next * kPayloadStride))->payload;
+        next = g.chain[kChainWords * next + kChainNext];
+      }
+    }
+  }
+  // Nothing is counted on the way out: a workgroup that lives for a few microseconds would spend a
+  // tenth of them waiting for a returning atomic (ring all-reduce 8 x 32 MiB: 85 -> 94 us with a count
+  // per queue and an exit word).  The launch's end is the graph's completion; pccl_hip_graph_status
+  // reports it in stream order, and *completed_operator on the device is not written by such a launch.
+  if (trace) {
+    __syncthreads();
+    if (threadIdx.x == 0) trace[kTraceDone] = wall_clock64();
+  }
+}
+
+template <int DT, class Op>
+__global__ void __launch_bounds__(kBlock) wide_graph_kernel(const GraphControl g) {
+  wide_body<DT, Op, false>(g);
+}
+
+template <int DT, class Op>
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3))) wide_graph_forward_kernel(const GraphControl g) {
+  wide_body<DT, Op, true>(g);
+}
+
+// The instances, beside the drain kernel's in graph_queue_inst_<dtype>.hip / graph_queue_fwd_<dtype>.hip.
+template <int DT>
+DrainKernel wide_for_compute(int compute);
+template <int DT>
+DrainKernel wide_forward_for_compute(int compute);
+DrainKernel wide_for_any();
+
 // The instances of one dtype; defined in graph_queue_inst_<dtype>.hip.
 template <int DT>
 DrainKernel drain_for_compute(int compute);
@@ -950,6 +1053,15 @@ DrainKernel drain_for_any();
       case PCCL_MIN: return drain_graph_kernel<DT, OpMin>;       \
       default: return drain_graph_kernel<DT, OpMax>;             \
     }                                                            \
+  }                                                              \
+  template <>                                                    \
+  DrainKernel wide_for_compute<DT>(int compute) {                \
+    switch (compute) {                                           \
+      case PCCL_SUM: return wide_graph_kernel<DT, OpSum>;        \
+      case PCCL_PROD: return wide_graph_kernel<DT, OpProd>;      \
+      case PCCL_MIN: return wide_graph_kernel<DT, OpMin>;        \
+      default: return wide_graph_kernel<DT, OpMax>;              \
+    }                                                            \
   }
 
 #define PCCL_DEFINE_DRAIN_FORWARD_FOR_COMPUTE(DT)                        \
@@ -960,6 +1072,15 @@ DrainKernel drain_for_any();
       case PCCL_PROD: return drain_graph_forward_kernel<DT, OpProd>;     \
       case PCCL_MIN: return drain_graph_forward_kernel<DT, OpMin>;       \
       default: return drain_graph_forward_kernel<DT, OpMax>;             \
+    }                                                            \
+  }                                                              \
+  template <>                                                    \
+  DrainKernel wide_forward_for_compute<DT>(int compute) {        \
+    switch (compute) {                                           \
+      case PCCL_SUM: return wide_graph_forward_kernel<DT, OpSum>;  \
+      case PCCL_PROD: return wide_graph_forward_kernel<DT, OpProd>; \
+      case PCCL_MIN: return wide_graph_forward_kernel<DT, OpMin>;  \
+      default: return wide_graph_forward_kernel<DT, OpMax>;      \
     }                                                            \
   }
 

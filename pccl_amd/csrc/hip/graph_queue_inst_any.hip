@@ -4,4 +4,5 @@
 
 namespace pccl_queue {
 DrainKernel drain_for_any() { return drain_graph_kernel<kAnyDtype, void>; }
+DrainKernel wide_for_any() { return wide_graph_kernel<kAnyDtype, void>; }
 }  // namespace pccl_queue

@@ -91,11 +91,12 @@ def test_queue_run_with_signal_ops_replay(hip, oracle):
     g.destroy()
 
 
-def test_recorded_queue_run_survives_a_rebind_that_changes_aliasing(hip, oracle):
+def test_recorded_queue_run_survives_a_rebind_that_changes_aliasing(hip, oracle, monkeypatch):
     """A: t = a + b; B: u = t + c, recorded once.  Rebinding u onto a's buffer (shifted) turns
     the dependency from part-by-part to whole-op, which rebuilds the graph's contents; the
     recording made before must still be valid (same arena) and give sequential results."""
     import torch
+    monkeypatch.setenv("PCCL_HIP_WIDE", "0")  # (the persistent drain; a wide launch refuses such a rebind)
     count, shift = 1500 * 1000, 64
     a_full = H.gen("f32", count + shift, 401, 0)
     b, c = H.gen("f32", count, 401, 1), H.gen("f32", count, 401, 2)

@@ -592,11 +592,12 @@ def test_shifted_overlap_keeps_the_dependency_whole(hip, oracle):
     g.destroy()
 
 
-def test_rebind_that_changes_aliasing_rebuilds_the_graph(hip, oracle):
+def test_rebind_that_changes_aliasing_rebuilds_the_graph(hip, oracle, monkeypatch):
     """A: t = a + b; B: u = t + c.  Rebinding u onto a's buffer, shifted, makes B overwrite what
     A reads: the dependency turns whole-op (graph rebuilt inside rebind); rebinding it back
     restores the part-by-part form.  Results must match sequential execution each time."""
     import torch
+    monkeypatch.setenv("PCCL_HIP_WIDE", "0")  # (as a wide launch the graph would refuse that rebind: see the test below)
     count, shift = 1500 * 1000, 64
     a_full = H.gen("f32", count + shift, 99, 0)
     b, c = H.gen("f32", count, 99, 1), H.gen("f32", count, 99, 2)
@@ -632,6 +633,97 @@ def test_rebind_that_changes_aliasing_rebuilds_the_graph(hip, oracle):
     _run_and_check(torch, hip, g, 2)
     H.assert_bits_equal(du.download(), u, "after rebinding back")
     assert dA.guards_intact() and du.guards_intact() and dt.guards_intact()
+    g.destroy()
+
+
+def test_wide_launch_refuses_a_rebind_that_makes_an_entry_wait(hip, oracle):
+    """The same two ops with the library's own choices: B runs behind A in A's workgroups, no entry waits
+    for another, so the graph runs as a wide launch (one workgroup per entry, more than the device holds
+    at once).  The rebind that makes B wait for all of A cannot be carried out by such a launch: it is
+    refused before anything changes, the graph goes on with the operands it had, and other rebinds work."""
+    import torch
+    count, shift = 6 * 1000 * 1000, 64
+    a_full = H.gen("f32", count + shift, 199, 0)
+    b, c = H.gen("f32", count, 199, 1), H.gen("f32", count, 199, 2)
+    dA = H.DevBuf(torch, "f32", count + shift, 0, src=a_full)
+    db, dc = H.DevBuf(torch, "f32", count, 0, src=b), H.DevBuf(torch, "f32", count, 0, src=c)
+    dt, du, dv = H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0), H.DevBuf(torch, "f32", count, 0)
+    g = hip.Graph([dict(dtype="f32", compute="sum", ins=[dA.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
+                   dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0])])
+    info = g.info()
+    assert info["n_workgroups"] == info["n_tiles"] == (4 * count + 16383) // 16384, info  # one workgroup per 16 KiB part of A
+    t = oracle.reduce("f32", "sum", [a_full[:count], b])
+    u = oracle.reduce("f32", "sum", [t, c])
+    for _ in range(2):
+        _run_and_check(torch, hip, g, 2)
+        H.assert_bits_equal(du.download(), u, "wide launch")
+        H.assert_bits_equal(dt.download(), t, "t")
+    with pytest.raises(hip.PcclError) as e:
+        g.rebind(du.ptr, dA.ptr + 4 * shift, 4 * count, _stream(torch))
+    assert e.value.code == hip.ERR_UNSUPPORTED and "wide launch" in str(e.value)
+    du.upload(np.zeros(count, dtype=np.float32).view(u.dtype))
+    _run_and_check(torch, hip, g, 2)
+    H.assert_bits_equal(du.download(), u, "after the refused rebind")
+    g.rebind(du.ptr, dv.ptr, 4 * count, _stream(torch))  # (a move that keeps the plan)
+    _run_and_check(torch, hip, g, 2)
+    H.assert_bits_equal(dv.download(), u, "after a rebind that keeps the plan")
+    assert all(d.guards_intact() for d in (dA, dt, du, dv))
+    g.destroy()
+
+
+def test_wide_launch_and_persistent_drain_leave_the_same_bytes(hip, oracle, monkeypatch):
+    """Independent ops of ragged sizes and odd alignments, a chain that runs in one pass, and a fold of
+    three inputs with a copy of its output that the fold stores itself: as a wide launch, with a
+    timeline, and through the persistent drain (PCCL_HIP_WIDE=0)."""
+    import torch
+    rng = np.random.default_rng(5)
+    def build():
+        ops, checks = [], []
+        for k in range(12):  # independent ops
+            n_in, count = int(rng.integers(1, 6)), int(rng.integers(1, 70000))
+            srcs = [H.gen("bf16", count, 300 + k, j) for j in range(n_in)]
+            ds = [H.DevBuf(torch, "bf16", count, int(rng.integers(0, 8)) * 2, src=x) for x in srcs]
+            do = H.DevBuf(torch, "bf16", count, int(rng.integers(0, 8)) * 2)
+            ops.append(dict(dtype="bf16", compute="sum", ins=[d.ptr for d in ds], outs=[do.ptr], count=count, deps=[]))
+            checks.append((do, oracle.reduce("bf16", "sum", srcs), ds))
+        count = 150001
+        x = [H.gen("bf16", count, 340, j) for j in range(5)]
+        dx = [H.DevBuf(torch, "bf16", count, 0, src=v) for v in x]
+        d1, d2, d3, d4 = (H.DevBuf(torch, "bf16", count, 0) for _ in range(4))
+        base = len(ops)
+        # a chain that runs in one pass
+        ops.append(dict(dtype="bf16", compute="sum", ins=[dx[0].ptr, dx[1].ptr], outs=[d1.ptr], count=count, deps=[]))
+        ops.append(dict(dtype="bf16", compute="sum", ins=[d1.ptr, dx[2].ptr], outs=[d2.ptr], count=count, deps=[base]))
+        r1 = oracle.reduce("bf16", "sum", [x[0], x[1]])
+        r2 = oracle.reduce("bf16", "sum", [r1, x[2]])
+        # three inputs (through memory), then a copy of the result, which the fold stores itself
+        ops.append(dict(dtype="bf16", compute="sum", ins=[dx[2].ptr, dx[3].ptr, dx[4].ptr], outs=[d3.ptr], count=count, deps=[]))
+        ops.append(dict(dtype="bf16", compute="sum", ins=[d3.ptr], outs=[d4.ptr], count=count, deps=[base + 2]))
+        r3 = oracle.reduce("bf16", "sum", [x[2], x[3], x[4]])
+        checks += [(d1, r1, dx), (d2, r2, []), (d3, r3, []), (d4, r3, [])]
+        return ops, checks
+    ops, checks = build()
+    g = hip.Graph(ops)
+    info = g.info()
+    assert info["n_workgroups"] == info["n_tiles"], info  # a wide launch
+    g.trace(True)
+    for _ in range(2):
+        for do, _, _ in checks: do.upload(np.zeros(do.count, dtype=np.uint16))
+        _run_and_check(torch, hip, g, len(ops))
+        for k, (do, want, _) in enumerate(checks):
+            H.assert_bits_equal(do.download(), want, "wide launch, output %d" % k)
+            assert do.guards_intact()
+    uid, part, ready, done = _timeline(torch, g)
+    assert len(uid) == info["n_tiles"] and (done >= ready).all()
+    g.destroy()
+    monkeypatch.setenv("PCCL_HIP_WIDE", "0")
+    g = hip.Graph(ops)
+    info = g.info()
+    assert info["n_workgroups"] <= 4096 and info["n_workgroups"] <= info["n_tiles"]
+    for do, _, _ in checks: do.upload(np.zeros(do.count, dtype=np.uint16))
+    _run_and_check(torch, hip, g, len(ops))
+    for k, (do, want, _) in enumerate(checks):
+        H.assert_bits_equal(do.download(), want, "persistent drain, output %d" % k)
     g.destroy()
 
 
@@ -730,6 +822,7 @@ def test_independent_ops_taken_without_tickets(hip, oracle, monkeypatch, own_rou
     """Entries that wait for no other entry of the graph are taken by workgroup number where they are few per
     workgroup: one each (built-in), several rounds (PCCL_HIP_OWN_ENTRIES=16), or by ticket (=0).  Same bytes."""
     import torch
+    monkeypatch.setenv("PCCL_HIP_WIDE", "0")  # (the persistent drain is the subject; such a graph would run as a wide launch)
     if own_rounds is not None:
         monkeypatch.setenv("PCCL_HIP_OWN_ENTRIES", own_rounds)
     rng = np.random.default_rng(77)
