@@ -217,10 +217,10 @@ typedef struct pccl_op_desc {
  * workgroups as entries, instead of the persistent drain: nothing is handed from workgroup to workgroup, so no
  * ticket is drawn and no part counted, and the hardware dispatcher balances the compute units (ring all-reduce
  * over 8 resident ranks x 1 / 8 / 32 / 64 MiB 16.4 / 31 / 93 / 227 -> 11.9 / 23.4 / 87 / 196 us, one 64 KiB op
- * 9.7 -> 6.5 us).  Graphs whose entries outside one-pass chains move 192 MiB or more stay with the drain.
+ * 9.7 -> 6.5 us; entries outside one-pass chains are cut into 32 KiB parts once they move 192 MiB or more).
  * The device arena, graph_info, graph_trace and results are the same; graph_status reports every op complete
  * once the stream has drained (the launch's end is the graph's completion; *completed_operator on the device
- * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0 never, 1 whenever possible. */
+ * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0: never. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 

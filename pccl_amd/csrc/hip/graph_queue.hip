@@ -152,10 +152,39 @@ struct Graph {
   bool wide_ok = false;    // build_graph's finding: no queue entry waits for another entry or for a signal
   bool wide = false;       // the graph runs that way
   long long wide_plain_bytes = 0;  // build_graph's finding: bytes moved by entries that do not run a chain in one pass
+  int wide_plain_streams = 0;      // ... and the most operands such an entry walks at once (a copy stored by its producer counted in)
+  std::vector<long> wide_tile_of;  // build_graph with want_wide: bytes per part, op by op (empty: kWideTileBytes for all)
+  unsigned wide_lds = 0;           // dynamic LDS of the wide launch (never touched: an occupancy cap like the direct kernels')
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
   bool as_launches = false;
   std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
 };
+
+// How a graph that runs as a wide launch is cut and capped, from the plan of its first build (G).
+// Chains that run in one pass: parts of one block (kWideTileBytes).  Everything else walks its part
+// 4 KiB after 4 KiB like a direct launch of several packs per lane, for which the direct kernels' rules
+// hold: much traffic wants longer parts and few workgroups per compute unit (about 20 workgroups x
+// streams).  Direct all-reduce over 8 resident ranks (eight folds 8 -> 8), 16 KiB parts uncapped
+// against 32 KiB parts at two workgroups per compute unit: 8 x 8 MiB 24.3 / 29.4 us, 8 x 16 MiB 58.6 /
+// 47.5, 8 x 32 MiB 92.7 / 87.8, 8 x 64 MiB 221 / 215 (through the persistent drain 31.8 / 53 / 90.3 / 222).
+void wide_cut_of(const Graph *G, Graph *W) {
+  const bool much = G->wide_plain_bytes >= (192ll << 20);
+  const int n = (int)G->eff.size();
+  W->wide_tile_of.assign(n, kWideTileBytes);
+  W->wide_lds = 0;
+  if (!much) return;
+  std::vector<char> one_pass(n, 0);  // op belongs to a chain that runs in one pass (its head says so)
+  for (int h = 0; h < n; ++h) {
+    const int *w = &G->chain_words[(size_t)kChainWords * h];
+    if (w[kChainNext] < 0 || w[kChainForward] != 1 || w[kChainLength] <= 1) continue;
+    for (int u = h, k = 0; u >= 0 && k < w[kChainLength]; u = G->chain_words[(size_t)kChainWords * u + kChainNext], ++k) one_pass[u] = 1;
+  }
+  for (int i = 0; i < n; ++i)
+    if (!one_pass[i]) W->wide_tile_of[i] = 2 * kWideTileBytes;
+  const int streams = std::max(1, G->wide_plain_streams);
+  const int wgs = std::max(2, std::min(8, (20 + streams / 2) / streams));
+  if (wgs < 3) W->wide_lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);  // (the kernel's registers allow three)
+}
 
 // ---- which dependencies can be met part by part -------------------------------
 // B depends on A.  Part p of B needs only part p of A when both ops are cut alike (same
@@ -206,21 +235,17 @@ Conflict conflict_of(const pccl_op_desc &a, const pccl_op_desc &b, uintptr_t byt
 // there reads the buffer a reduction reads too, and in blocks the two run side by side; with copies
 // that read buffers of their own it is 212 -> 209 us.  Ring and direct all-reduces over 8 ranks x
 // 1 .. 64 MiB and the 4096-op schedule (at most 3 parts per op) are unchanged within 1 %.
-// Whether a graph that may run as a wide launch (wide_body) does.  Chains that run in one pass gain at
-// every size measured (ring all-reduce over 8 resident ranks x 1 / 8 / 32 / 64 MiB: 16.4 / 31 / 93 / 227 us
-// through the persistent drain, 11.9 / 23.4 / 87 / 196 us wide), and so do small graphs of any kind (one
-// 64 KiB op 9.7 -> 6.5 us, the 4096-op schedule 77 -> 68 us, direct all-reduce 8 x 1 / 8 MiB 12.9 / 32 ->
-// 9.9 / 24.3 us).  Entries that go through memory op by op (single ops, chains that cannot run in one
-// pass) walk their part 4 KiB after 4 KiB like a direct launch of several packs per lane, which loses to
-// the persistent drain once there is much of it (direct all-reduce 8 x 16 / 32 MiB: 53 / 90.3 us through
-// the drain, 58.6 / 92.7 us wide): from 192 MiB of such traffic a graph stays with the drain.
-// PCCL_HIP_WIDE=0: never wide; 1: whenever the graph allows it.
-bool wide_launch_pays(long long plain_bytes) {
-  if (const char *env = getenv("PCCL_HIP_WIDE")) {
-    if (env[0] == '0') return false;
-    if (env[0] == '1') return true;
-  }
-  return plain_bytes < (192ll << 20);
+// Whether a graph that may run as a wide launch (wide_body) does: whenever it may.  Chains that run in
+// one pass gain at every size measured (ring all-reduce over 8 resident ranks x 1 / 8 / 32 / 64 MiB:
+// 16.4 / 31 / 93 / 227 us through the persistent drain, 11.9 / 23.4 / 87 / 196 us wide), and so do graphs
+// of single ops and of chains through memory, cut as wide_cut_of says (one 64 KiB op 9.7 -> 6.5 us, the
+// 4096-op schedule 77 -> 68 us, direct all-reduce 8 x 1 / 8 / 16 / 32 / 64 MiB 12.9 / 32 / 53 / 90.5 / 223 ->
+// 9.9 / 24 / 46 / 89 / 218 us, 14 independent copies of 32 MiB 188 -> 156 us, 4096 independent 2 -> 1 ops
+// of 64 KiB 73 -> 56 us, of 256 KiB 401 -> 403 us).
+// PCCL_HIP_WIDE=0: never.
+bool wide_launch_pays() {
+  const char *env = getenv("PCCL_HIP_WIDE");
+  return !(env && env[0] == '0');
 }
 
 int order_block() {
@@ -979,6 +1004,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
         continue;
       }
       long part_bytes = tile_bytes, even_bytes = tile_bytes;
+      if (G->want_wide && !G->wide_tile_of.empty()) part_bytes = even_bytes = G->wide_tile_of[i];  // (see wide_cut_of)
       if (default_tile) {
         auto rule = [&](long long bytes) {
           const double want = 16384.0 * std::pow((double)bytes / (double)(8 << 20), 2.0 / 3.0) * (768.0 / (double)cap);
@@ -1147,20 +1173,25 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     if (queued(i)) live_tiles += parts[i];
   // The wide launch (wide_body) is open to a graph none of whose entries waits for another entry (as
   // for entries without tickets, below) or has to do with a signal word (its workgroups poll nothing
-  // and tell nobody), with few enough entries for the exit word's count.
+  // and tell nobody), with no more entries than kMaxWideEntries (40 bytes of arena each).
   {
     bool waits = carries;
     for (int i = 0; i < n_ops && !waits; ++i)
       waits = queued(i) && (n_pred[i] > 0 || order_pred[i] > 0 || ops[i].primitive == PCCL_NOTIFY || ops[i].primitive == PCCL_GET_NOTIFIED);
-    G->wide_ok = !waits && live_tiles > 0 && live_tiles < (long long)kExitQuit;
+    G->wide_ok = !waits && live_tiles > 0 && live_tiles <= kMaxWideEntries;
     // (what the entries that do not run a chain in one pass move, chains through memory included: see wide_launch_pays)
     G->wide_plain_bytes = 0;
+    G->wide_plain_streams = 0;
     for (int i = 0; i < n_ops; ++i) {
       if (!queued(i)) continue;
       const int *w = &G->chain_words[(size_t)kChainWords * i];
       if (w[kChainNext] >= 0 && w[kChainForward] == 1) continue;
-      for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext])
+      for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext]) {
         G->wide_plain_bytes += (long long)(ops[u].n_in + ops[u].n_out) * op_bytes[u];
+        const int after = G->chain_words[(size_t)kChainWords * u + kChainNext];
+        const bool stores_next = after >= 0 && G->chain_words[(size_t)kChainWords * after + kChainForward] == kChainFolded;
+        G->wide_plain_streams = std::max(G->wide_plain_streams, ops[u].n_in + ops[u].n_out + (stores_next ? ops[after].n_out : 0));
+      }
     }
     if (G->want_wide && (!G->wide_ok || (G->fixed_n_wg > 0 && live_tiles > G->fixed_n_wg)))
       return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as a wide launch (an entry waits for another, "
@@ -1420,7 +1451,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   if (n_edges) memcpy(img + off_succ_part, succ_part_base.data(), sizeof(int) * n_edges);
   // never more workgroups than entries
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
-  G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, G->want_wide ? (long long)kExitQuit - 1 : cap));
+  G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, G->want_wide ? kMaxWideEntries : cap));
   G->wide = G->want_wide;
   {
     // Entries without tickets (graph_queue_device.h): when there is at most one per workgroup
@@ -1531,7 +1562,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   // The library's own cut (tile_bytes 0): a graph whose entries wait for nothing runs as a wide launch
   // (wide_body), for which it is cut again, every op into parts of one block.  If that cut does not
   // keep the property (or its arena cannot be had), the graph stays as built.
-  if (G->tile_bytes == 0 && G->wide_ok && wide_launch_pays(G->wide_plain_bytes)) {
+  if (G->tile_bytes == 0 && G->wide_ok && wide_launch_pays()) {
     Graph *W = new Graph();
     W->tile_bytes = 0;
     W->spin_limit = G->spin_limit;
@@ -1539,6 +1570,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
     W->deps_store = G->deps_store;
     for (int i = 0, at = 0; i < n_ops; at += ops[i].n_deps, ++i) W->descs[i].deps = W->deps_store.data() + at;
     W->want_wide = true;
+    wide_cut_of(G, W);
     if (build_graph(W, 1) == PCCL_OK) {
       if (G->dev) (void)hipFree(G->dev);
       delete G;
@@ -1580,7 +1612,7 @@ int pccl_hip_graph_run(void *graph, void *stream) {
     std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
     memcpy(&control, G->image.data(), sizeof(control));
   }
-  hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), 0, (hipStream_t)stream, control);
+  hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), G->wide ? G->wide_lds : 0u, (hipStream_t)stream, control);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run launch failed: %s", hipGetErrorString(e));
   {
@@ -1723,6 +1755,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.fixed_kernel = G->kernel;
     fresh.forward_capable = G->forward_capable;
     fresh.want_wide = G->wide;  // (a wide launch stays one, or the rebind is refused before anything changes)
+    fresh.wide_lds = G->wide_lds;
     char *old_dev = G->dev;
     // The run number goes on from where the DEVICE stands, not from the count of graph_run
     // calls: every replay of a recorded launch has moved the device's word on as well, and a

@@ -956,6 +956,7 @@ typedef void (*DrainKernel)(const GraphControl);
 // Nothing of the queue's state is written: no head moves, no part is counted, and the launch's end is
 // the graph's completion.  The arena is the one the drain kernel would use (entries, payloads, chain
 // words and table), so a rebind moves operands the same way.
+constexpr long long kMaxWideEntries = 1ll << 20;  // workgroups of one wide launch (16 GiB of output in 16 KiB parts)
 constexpr long kWideTileBytes = 16384;  // = kBlock lanes x 4 packs: the block run_chain_forward carries through a chain
 
 template <int DT, class Op, bool FORWARD>
