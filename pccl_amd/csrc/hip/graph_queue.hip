@@ -150,6 +150,7 @@ struct Graph {
   // The wide launch (graph_queue_device.h: wide_body): one workgroup per entry instead of the persistent drain.
   bool want_wide = false;  // build_graph: cut for it, check that the graph allows it, take its kernel
   bool wide_ok = false;    // build_graph's finding: no queue entry waits for another entry or for a signal
+  bool wide_slow = false;  // ... but a long chain goes through memory op by op, which the drain does better
   bool wide = false;       // the graph runs that way
   long long wide_plain_bytes = 0;  // build_graph's finding: bytes moved by entries that do not run a chain in one pass
   int wide_plain_streams = 0;      // ... and the most operands such an entry walks at once (a copy stored by its producer counted in)
@@ -1182,16 +1183,23 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     // (what the entries that do not run a chain in one pass move, chains through memory included: see wide_launch_pays)
     G->wide_plain_bytes = 0;
     G->wide_plain_streams = 0;
+    G->wide_slow = false;
     for (int i = 0; i < n_ops; ++i) {
       if (!queued(i)) continue;
       const int *w = &G->chain_words[(size_t)kChainWords * i];
       if (w[kChainNext] >= 0 && w[kChainForward] == 1) continue;
+      int steps = 0;  // ops of the chain that run (a copy that its producer stores does not)
       for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext]) {
         G->wide_plain_bytes += (long long)(ops[u].n_in + ops[u].n_out) * op_bytes[u];
         const int after = G->chain_words[(size_t)kChainWords * u + kChainNext];
         const bool stores_next = after >= 0 && G->chain_words[(size_t)kChainWords * after + kChainForward] == kChainFolded;
         G->wide_plain_streams = std::max(G->wide_plain_streams, ops[u].n_in + ops[u].n_out + (stores_next ? ops[after].n_out : 0));
+        if (G->chain_words[(size_t)kChainWords * u + kChainForward] != kChainFolded || u == i) ++steps;
       }
+      // A long chain through memory is a row of dependent round trips per workgroup (stores acknowledged,
+      // barrier, next op's loads), which the drain's longer parts carry better than short-lived workgroups:
+      // one rank's 14 ring steps as one such chain 209 us through the drain, 247 us wide.
+      if (steps > 2) G->wide_slow = true;
     }
     if (G->want_wide && (!G->wide_ok || (G->fixed_n_wg > 0 && live_tiles > G->fixed_n_wg)))
       return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as a wide launch (an entry waits for another, "
@@ -1562,7 +1570,7 @@ int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, v
   // The library's own cut (tile_bytes 0): a graph whose entries wait for nothing runs as a wide launch
   // (wide_body), for which it is cut again, every op into parts of one block.  If that cut does not
   // keep the property (or its arena cannot be had), the graph stays as built.
-  if (G->tile_bytes == 0 && G->wide_ok && wide_launch_pays()) {
+  if (G->tile_bytes == 0 && G->wide_ok && !G->wide_slow && wide_launch_pays()) {
     Graph *W = new Graph();
     W->tile_bytes = 0;
     W->spin_limit = G->spin_limit;

@@ -350,12 +350,16 @@ __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const p
   constexpr int kBatch = 4;  // packs a lane carries through the chain at a time (16 KiB per workgroup and stream)
   constexpr int kAhead = 4;  // ops whose other input is requested ahead of the value reaching them
   __shared__ __attribute__((aligned(16))) ForwardStep s_step[kMaxForwardSteps];
+  // (the first three operands' addresses together with the input count: which of them is output 0 depends
+  // on the count, and a load that waits for the count would be one more round trip in front of the data:
+  // ring all-reduce 8 x 8 / 16 / 32 MiB as a wide launch 23.4 / 49 / 86.7 -> 22.5 / 46 / 84.8 us)
   const int head_n_in = hp->n_in_;
+  const char *head_in0 = (const char *)hp->chunks_[0].addr_, *head_a1 = (const char *)hp->chunks_[1].addr_, *head_a2 = (const char *)hp->chunks_[2].addr_;
   if (threadIdx.x < 2u * (unsigned)n_steps)  // two lanes per row
     ((u32x4 *)s_step)[threadIdx.x] = ((const u32x4 *)(g.chain_table + first_row))[threadIdx.x];
   __syncthreads();
   // the elements before output 0's first 16-byte boundary are left to the edge code below
-  const unsigned long long out0 = (unsigned long long)hp->chunks_[head_n_in].addr_ + (unsigned long long)lo * D::kElemBytes;
+  const unsigned long long out0 = (unsigned long long)(head_n_in == 2 ? head_a2 : head_a1) + (unsigned long long)lo * D::kElemBytes;
   long peel = (long)((16 - (out0 & 15)) & 15) / D::kElemBytes;
   if (peel > count) peel = count;
   const long n_packs = (count - peel) / kEpp;
@@ -381,8 +385,8 @@ __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const p
     u32x4 cur[kBatch], in1[kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
-      cur[u] = load_pack<D, true, kMemCoherent>((const char *)hp->chunks_[0].addr_ + chunk, off[u]);
-      if (head_n_in == 2) in1[u] = load_pack<D, true, kMemCoherent>((const char *)hp->chunks_[1].addr_ + chunk, off[u]);
+      cur[u] = load_pack<D, true, kMemCoherent>(head_in0 + chunk, off[u]);
+      if (head_n_in == 2) in1[u] = load_pack<D, true, kMemCoherent>(head_a1 + chunk, off[u]);
     }
     for (int s0 = 0; s0 < n_steps; s0 += kAhead) {
       u32x4 other[kAhead][kBatch];
@@ -425,8 +429,8 @@ __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const p
     const long e = (long)threadIdx.x - (kBlock - kWave);
     if (e < n_edge) {
       const long i = lo + (e < peel ? e : tail_begin + (e - peel));
-      E cur = load_elem<E, kMemCoherent>((const E *)hp->chunks_[0].addr_ + i), second = cur;
-      if (head_n_in == 2) second = load_elem<E, kMemCoherent>((const E *)hp->chunks_[1].addr_ + i);
+      E cur = load_elem<E, kMemCoherent>((const E *)head_in0 + i), second = cur;
+      if (head_n_in == 2) second = load_elem<E, kMemCoherent>((const E *)head_a1 + i);
       E other[kMaxForwardSteps];
 #pragma unroll
       for (int s = 1; s < kMaxForwardSteps; ++s) {
