@@ -338,7 +338,7 @@ int pccl_hip_graph_set_spin_limit(void *graph, unsigned int microseconds);
  * call then uploads the state afresh).  Calls issued at the same time from several threads are
  * serialised by the library; work of the caller's own on other streams that touches the operands is the
  * caller's to order.  Not meant to be recorded by stream capture (the upload reads host memory and the
- * call waits for a stream). */
+ * call waits for a stream).  Every graph goes through the persistent drain here (no wide launch). */
 #define PCCL_HIP_STATIC_ARENA_BYTES (8u << 20)
 int pccl_hip_graph_run_static(const pccl_op_desc *ops, int n_ops, long tile_bytes, void *stream,
                               unsigned int *completed, unsigned int *total);
