@@ -75,6 +75,33 @@ def test_ring_allreduce_from_native_file(E, eng, oracle, tmp_path):
     H.assert_bits_equal(d_out2.cpu().numpy().view(np.uint16), want, "input re-bound alone")
 
 
+def test_ring_allreduce_in_place_and_back(E, eng, oracle, tmp_path):
+    """exeOp with one tensor as input and output (every chunk is read by the op that first writes it, so the
+    result is the out-of-place one), then on separate tensors again, then in place again: the executor moves
+    the operands where it can and builds the graph again where it cannot."""
+    import torch
+    p = str(tmp_path / "ring.sched")
+    E.write_ring_allreduce(p, "bf16", "sum", 8, 70_001)
+    eng.regOp("ring", p)
+    info = eng.opInfo("ring")
+    n = info["devices"] * info["elems_per_device"]
+    stream = torch.cuda.current_stream().cuda_stream
+    for round_, seed in enumerate((81, 82, 83, 84)):
+        host_in = H.gen("bf16", n, seed, 0)
+        _, want = _oracle_replay(oracle, open(p).read(), host_in)
+        d_in = _to_dev(torch, host_in)
+        if round_ % 2 == 0:
+            eng.exeOp("ring", d_in, d_in, stream)
+            eng.waitOp("ring", stream)
+            H.assert_bits_equal(d_in.cpu().numpy().view(np.uint16), want, "in place, call %d" % round_)
+        else:
+            d_out = torch.zeros(n * 2, dtype=torch.uint8, device="cuda")
+            eng.exeOp("ring", d_in, d_out, stream)
+            eng.waitOp("ring", stream)
+            H.assert_bits_equal(d_out.cpu().numpy().view(np.uint16), want, "out of place, call %d" % round_)
+            H.assert_bits_equal(d_in.cpu().numpy().view(np.uint16), host_in, "input untouched, call %d" % round_)
+
+
 def test_python_emitted_schedule(E, eng, oracle, tmp_path):
     import torch
     from pccl_amd import lang
