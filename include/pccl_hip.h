@@ -213,10 +213,10 @@ typedef struct pccl_op_desc {
  * PCCL_HIP_FUSE_SIGNALS=0 keeps every signal op an op of its own.
  * The wide launch: with tile_bytes 0 (or PCCL_HIP_TILE_AUTO), a graph none of whose queue entries waits for
  * another entry or has to do with a signal word (independent ops; chains, whose later ops run behind the first
- * in the same workgroup) is cut into parts of 16 KiB and run by one short-lived workgroup per entry, as many
+ * in the same workgroup) is cut into parts of 8 to 32 KiB and run by one short-lived workgroup per entry, as many
  * workgroups as entries, instead of the persistent drain: nothing is handed from workgroup to workgroup, so no
  * ticket is drawn and no part counted, and the hardware dispatcher balances the compute units (ring all-reduce
- * over 8 resident ranks x 1 / 8 / 32 / 64 MiB 16.4 / 31 / 93 / 227 -> 11.9 / 23.4 / 87 / 196 us, one 64 KiB op
+ * over 8 resident ranks x 1 / 8 / 32 / 64 MiB 16.4 / 30 / 92.5 / 227 -> 9.6 / 21.8 / 84.5 / 200 us, one 64 KiB op
  * 9.7 -> 6.5 us; entries outside one-pass chains are cut into 32 KiB parts once they move 192 MiB or more).
  * The device arena, graph_info, graph_trace and results are the same; graph_status reports every op complete
  * once the stream has drained (the launch's end is the graph's completion; *completed_operator on the device

@@ -66,23 +66,23 @@ using pccl_host::fail;
 
 namespace {
 
-DrainKernel drain_for(int dtype, int compute, bool forward, bool wide = false) {
+DrainKernel drain_for(int dtype, int compute, bool forward, bool wide = false, bool wide_small = false) {
   switch (dtype) {
-    case PCCL_F32: return forward ? (wide ? wide_forward_for_compute<PCCL_F32>(compute) : drain_forward_for_compute<PCCL_F32>(compute))
+    case PCCL_F32: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_F32>(compute) : wide_forward_for_compute<PCCL_F32>(compute)) : drain_forward_for_compute<PCCL_F32>(compute))
                               : (wide ? wide_for_compute<PCCL_F32>(compute) : drain_for_compute<PCCL_F32>(compute));
-    case PCCL_I32: return forward ? (wide ? wide_forward_for_compute<PCCL_I32>(compute) : drain_forward_for_compute<PCCL_I32>(compute))
+    case PCCL_I32: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_I32>(compute) : wide_forward_for_compute<PCCL_I32>(compute)) : drain_forward_for_compute<PCCL_I32>(compute))
                               : (wide ? wide_for_compute<PCCL_I32>(compute) : drain_for_compute<PCCL_I32>(compute));
-    case PCCL_BF16: return forward ? (wide ? wide_forward_for_compute<PCCL_BF16>(compute) : drain_forward_for_compute<PCCL_BF16>(compute))
+    case PCCL_BF16: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_BF16>(compute) : wide_forward_for_compute<PCCL_BF16>(compute)) : drain_forward_for_compute<PCCL_BF16>(compute))
                               : (wide ? wide_for_compute<PCCL_BF16>(compute) : drain_for_compute<PCCL_BF16>(compute));
-    case PCCL_F16: return forward ? (wide ? wide_forward_for_compute<PCCL_F16>(compute) : drain_forward_for_compute<PCCL_F16>(compute))
+    case PCCL_F16: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_F16>(compute) : wide_forward_for_compute<PCCL_F16>(compute)) : drain_forward_for_compute<PCCL_F16>(compute))
                               : (wide ? wide_for_compute<PCCL_F16>(compute) : drain_for_compute<PCCL_F16>(compute));
-    case PCCL_F8E4M3: return forward ? (wide ? wide_forward_for_compute<PCCL_F8E4M3>(compute) : drain_forward_for_compute<PCCL_F8E4M3>(compute))
+    case PCCL_F8E4M3: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_F8E4M3>(compute) : wide_forward_for_compute<PCCL_F8E4M3>(compute)) : drain_forward_for_compute<PCCL_F8E4M3>(compute))
                               : (wide ? wide_for_compute<PCCL_F8E4M3>(compute) : drain_for_compute<PCCL_F8E4M3>(compute));
-    case PCCL_F8E5M2: return forward ? (wide ? wide_forward_for_compute<PCCL_F8E5M2>(compute) : drain_forward_for_compute<PCCL_F8E5M2>(compute))
+    case PCCL_F8E5M2: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_F8E5M2>(compute) : wide_forward_for_compute<PCCL_F8E5M2>(compute)) : drain_forward_for_compute<PCCL_F8E5M2>(compute))
                               : (wide ? wide_for_compute<PCCL_F8E5M2>(compute) : drain_for_compute<PCCL_F8E5M2>(compute));
-    case PCCL_F64: return forward ? (wide ? wide_forward_for_compute<PCCL_F64>(compute) : drain_forward_for_compute<PCCL_F64>(compute))
+    case PCCL_F64: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_F64>(compute) : wide_forward_for_compute<PCCL_F64>(compute)) : drain_forward_for_compute<PCCL_F64>(compute))
                               : (wide ? wide_for_compute<PCCL_F64>(compute) : drain_for_compute<PCCL_F64>(compute));
-    default: return forward ? (wide ? wide_forward_for_compute<PCCL_U32>(compute) : drain_forward_for_compute<PCCL_U32>(compute))
+    default: return forward ? (wide ? (wide_small ? wide_forward_small_for_compute<PCCL_U32>(compute) : wide_forward_for_compute<PCCL_U32>(compute)) : drain_forward_for_compute<PCCL_U32>(compute))
                               : (wide ? wide_for_compute<PCCL_U32>(compute) : drain_for_compute<PCCL_U32>(compute));
   }
 }
@@ -156,6 +156,8 @@ struct Graph {
   int wide_plain_streams = 0;      // ... and the most operands such an entry walks at once (a copy stored by its producer counted in)
   std::vector<long> wide_tile_of;  // build_graph with want_wide: bytes per part, op by op (empty: kWideTileBytes for all)
   unsigned wide_lds = 0;           // dynamic LDS of the wide launch (never touched: an occupancy cap like the direct kernels')
+  bool wide_small = false;         // one-pass chains in 8 KiB blocks (the SMALL instances of wide_body)
+  long long wide_chain_bytes = 0;  // build_graph's finding: bytes the ops of one-pass chains name
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
   bool as_launches = false;
   std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
@@ -173,13 +175,21 @@ void wide_cut_of(const Graph *G, Graph *W) {
   const int n = (int)G->eff.size();
   W->wide_tile_of.assign(n, kWideTileBytes);
   W->wide_lds = 0;
-  if (!much) return;
   std::vector<char> one_pass(n, 0);  // op belongs to a chain that runs in one pass (its head says so)
   for (int h = 0; h < n; ++h) {
     const int *w = &G->chain_words[(size_t)kChainWords * h];
     if (w[kChainNext] < 0 || w[kChainForward] != 1 || w[kChainLength] <= 1) continue;
     for (int u = h, k = 0; u >= 0 && k < w[kChainLength]; u = G->chain_words[(size_t)kChainWords * u + kChainNext], ++k) one_pass[u] = 1;
   }
+  // One-pass chains whose ops name less than 512 MiB in all: blocks of 8 KiB and the SMALL kernel instance
+  // (wide_body).  Ring all-reduce over 8 ranks x 1 / 8 MiB (37 / 294 MB named) 11.4 / 22.9 -> 9.6 / 21.8 us;
+  // x 16 MiB (587 MB) would gain too (46 -> 44.7 us), but the 4096-op schedule (764 MB in 288 short chains)
+  // loses (64 -> 67.8 us) and 8 x 32 MiB as well (84.8 -> 89 us).
+  W->wide_small = G->wide_chain_bytes > 0 && G->wide_chain_bytes < (512ll << 20);
+  if (W->wide_small)
+    for (int i = 0; i < n; ++i)
+      if (one_pass[i]) W->wide_tile_of[i] = kWideSmallTileBytes;
+  if (!much) return;
   for (int i = 0; i < n; ++i)
     if (!one_pass[i]) W->wide_tile_of[i] = 2 * kWideTileBytes;
   const int streams = std::max(1, G->wide_plain_streams);
@@ -884,7 +894,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // such ops runs the plain one, its chains through memory)
   bool carries = false;
   for (int i = 0; i < n_ops; ++i) carries = carries || G->fused_into[i] >= 0;
-  const DrainKernel forward_kernel = (mixed || carries) ? nullptr : drain_for(g_dtype, g_compute, true, wide);
+  const DrainKernel forward_kernel = (mixed || carries) ? nullptr : drain_for(g_dtype, g_compute, true, wide, G->wide_small);
   const int forward_elem_bytes = (G->fixed_kernel ? G->forward_capable : (!mixed && !carries)) ? elem_bytes(g_dtype) : 0;
   int occ = 8;
   for (DrainKernel k : {plain_kernel, forward_kernel}) {
@@ -1183,11 +1193,16 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     // (what the entries that do not run a chain in one pass move, chains through memory included: see wide_launch_pays)
     G->wide_plain_bytes = 0;
     G->wide_plain_streams = 0;
+    G->wide_chain_bytes = 0;
     G->wide_slow = false;
     for (int i = 0; i < n_ops; ++i) {
       if (!queued(i)) continue;
       const int *w = &G->chain_words[(size_t)kChainWords * i];
-      if (w[kChainNext] >= 0 && w[kChainForward] == 1) continue;
+      if (w[kChainNext] >= 0 && w[kChainForward] == 1) {
+        for (int u = i, k = 0; u >= 0 && k < w[kChainLength]; u = G->chain_words[(size_t)kChainWords * u + kChainNext], ++k)
+          G->wide_chain_bytes += (long long)(ops[u].n_in + ops[u].n_out) * op_bytes[u];
+        continue;
+      }
       int steps = 0;  // ops of the chain that run (a copy that its producer stores does not)
       for (int u = i; u >= 0; u = G->chain_words[(size_t)kChainWords * u + kChainNext]) {
         G->wide_plain_bytes += (long long)(ops[u].n_in + ops[u].n_out) * op_bytes[u];
@@ -1764,6 +1779,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.forward_capable = G->forward_capable;
     fresh.want_wide = G->wide;  // (a wide launch stays one, or the rebind is refused before anything changes)
     fresh.wide_lds = G->wide_lds;
+    fresh.wide_small = G->wide_small;
     char *old_dev = G->dev;
     // The run number goes on from where the DEVICE stands, not from the count of graph_run
     // calls: every replay of a recorded launch has moved the device's word on as well, and a

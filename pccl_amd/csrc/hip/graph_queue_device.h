@@ -343,12 +343,12 @@ __device__ __forceinline__ unsigned long long uniform64(unsigned long long v) { 
   return ((unsigned long long)hi << 32) | lo;
 }
 
-template <class D, class Op>
+// kBatch: packs a lane carries through the chain at a time (4: 16 KiB per workgroup and stream);
+// kAhead: ops whose other input is requested ahead of the value reaching them.
+template <class D, class Op, int kBatch = 4, int kAhead = 4>
 __device__ __forceinline__ void run_chain_forward(const GraphControl &g, const pccl_op_payload *hp, int n_steps, int first_row, long lo, long count) {
   typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
-  constexpr int kBatch = 4;  // packs a lane carries through the chain at a time (16 KiB per workgroup and stream)
-  constexpr int kAhead = 4;  // ops whose other input is requested ahead of the value reaching them
   __shared__ __attribute__((aligned(16))) ForwardStep s_step[kMaxForwardSteps];
   // (the first three operands' addresses together with the input count: which of them is output 0 depends
   // on the count, and a load that waits for the count would be one more round trip in front of the data:
@@ -961,9 +961,13 @@ typedef void (*DrainKernel)(const GraphControl);
 // the graph's completion.  The arena is the one the drain kernel would use (entries, payloads, chain
 // words and table), so a rebind moves operands the same way.
 constexpr long long kMaxWideEntries = 1ll << 20;  // workgroups of one wide launch (16 GiB of output in 16 KiB parts)
-constexpr long kWideTileBytes = 16384;  // = kBlock lanes x 4 packs: the block run_chain_forward carries through a chain
+constexpr long kWideTileBytes = 16384;
+constexpr long kWideSmallTileBytes = 8192;  // = kBlock lanes x 2 packs: the block of the SMALL instances  // = kBlock lanes x 4 packs: the block run_chain_forward carries through a chain
 
-template <int DT, class Op, bool FORWARD>
+// SMALL: one-pass chains in blocks of kWideSmallTileBytes, two packs per lane with eight ops' inputs ahead,
+// four wavefronts per SIMD: the better shape while the chains move little (ring all-reduce over 8 resident
+// ranks x 1 / 8 / 16 MiB 11.4 / 22.9 / 46 -> 9.8 / 21.6 / 44.8 us), the worse one from 8 x 32 MiB (84.8 -> 89 us).
+template <int DT, class Op, bool FORWARD, bool SMALL = false>
 __device__ __forceinline__ void wide_body(const GraphControl &g) {
   if constexpr (DT != kAnyDtype) Dtype<DT>::wave_init();
   const unsigned int b = blockIdx.x;
@@ -988,7 +992,7 @@ __device__ __forceinline__ void wide_body(const GraphControl &g) {
     bool forwarded = false;
     if constexpr (FORWARD && DT != kAnyDtype) {
       if (chain_next >= 0 && __builtin_amdgcn_readfirstlane(chain[kChainForward])) {
-        run_chain_forward<Dtype<DT>, Op>(g, pl, __builtin_amdgcn_readfirstlane(chain[kChainLength]), __builtin_amdgcn_readfirstlane(chain[kChainRow]), lo, n);
+        run_chain_forward<Dtype<DT>, Op, SMALL ? 2 : 4, SMALL ? 8 : 4>(g, pl, __builtin_amdgcn_readfirstlane(chain[kChainLength]), __builtin_amdgcn_readfirstlane(chain[kChainRow]), lo, n);
         forwarded = true;
       }
     }
@@ -1031,11 +1035,18 @@ __global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 
   wide_body<DT, Op, true>(g);
 }
 
+template <int DT, class Op>
+__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) wide_graph_forward_small_kernel(const GraphControl g) {
+  wide_body<DT, Op, true, true>(g);
+}
+
 // The instances, beside the drain kernel's in graph_queue_inst_<dtype>.hip / graph_queue_fwd_<dtype>.hip.
 template <int DT>
 DrainKernel wide_for_compute(int compute);
 template <int DT>
 DrainKernel wide_forward_for_compute(int compute);
+template <int DT>
+DrainKernel wide_forward_small_for_compute(int compute);
 DrainKernel wide_for_any();
 
 // The instances of one dtype; defined in graph_queue_inst_<dtype>.hip.
@@ -1086,6 +1097,15 @@ DrainKernel drain_for_any();
       case PCCL_PROD: return wide_graph_forward_kernel<DT, OpProd>; \
       case PCCL_MIN: return wide_graph_forward_kernel<DT, OpMin>;  \
       default: return wide_graph_forward_kernel<DT, OpMax>;      \
+    }                                                            \
+  }                                                              \
+  template <>                                                    \
+  DrainKernel wide_forward_small_for_compute<DT>(int compute) {  \
+    switch (compute) {                                           \
+      case PCCL_SUM: return wide_graph_forward_small_kernel<DT, OpSum>;  \
+      case PCCL_PROD: return wide_graph_forward_small_kernel<DT, OpProd>; \
+      case PCCL_MIN: return wide_graph_forward_small_kernel<DT, OpMin>;  \
+      default: return wide_graph_forward_small_kernel<DT, OpMax>;  \
     }                                                            \
   }
 

@@ -651,7 +651,7 @@ def test_wide_launch_refuses_a_rebind_that_makes_an_entry_wait(hip, oracle):
     g = hip.Graph([dict(dtype="f32", compute="sum", ins=[dA.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
                    dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0])])
     info = g.info()
-    assert info["n_workgroups"] == info["n_tiles"] == (4 * count + 16383) // 16384, info  # one workgroup per 16 KiB part of A
+    assert info["n_workgroups"] == info["n_tiles"] == (4 * count + 8191) // 8192, info  # one workgroup per 8 KiB block of the chain
     t = oracle.reduce("f32", "sum", [a_full[:count], b])
     u = oracle.reduce("f32", "sum", [t, c])
     for _ in range(2):
