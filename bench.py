@@ -123,8 +123,8 @@ def through_the_drain(torch, hip, bound_ops, stream, steps=20):
     return dict(stats(t), queue_entries=info["n_tiles"], workgroups=info["n_workgroups"])
 
 
-def launch_kind(info):
-    return "wide (one workgroup per entry)" if info["n_workgroups"] == info["n_tiles"] and info["n_tiles"] > 1 else "persistent drain"
+def launch_kind(graph):
+    return {"wide": "wide (one workgroup per entry)", "drain": "persistent drain", "launches": "plain launches"}[graph.launch_kind()]
 
 
 def queue_bytes_moved(hip, bound_ops, elem_bytes):
@@ -725,7 +725,7 @@ def main():
                     full["8_ranks_x_%d_MiB" % per_rank_mib] = dict(stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low),
                                                                   algorithmic_bytes=moved, bytes_moved=really,
                                                                   GBps_moved_median=gbps(really, tf[len(tf) // 2]),
-                                                                  queue_entries=g.info()["n_tiles"], launch=launch_kind(g.info()),
+                                                                  queue_entries=g.info()["n_tiles"], launch=launch_kind(g),
                                                                   dependencies_part_by_part="%d of %d" % (sum(kinds), len(kinds)))
                     g.destroy()
                     full["8_ranks_x_%d_MiB" % per_rank_mib]["through_the_persistent_drain"] = through_the_drain(torch, hip, ring_bound, stream)
@@ -821,7 +821,7 @@ def main():
                     direct["8_ranks_x_%d_MiB" % per_rank_mib] = dict(
                         stats(tf), GBps_median=gbps(moved, tf[len(tf) // 2]), ops=len(low), algorithmic_bytes=moved,
                         bytes_moved=really, GBps_moved_median=gbps(really, tf[len(tf) // 2]),
-                        queue_entries=g.info()["n_tiles"], launch=launch_kind(g.info()), dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
+                        queue_entries=g.info()["n_tiles"], launch=launch_kind(g), dependencies_part_by_part="%d of %d" % (sum(dkinds), len(dkinds)),
                         as_one_launch_8in_8out=dict(stats(t1), GBps_median=gbps(16 * per_rank * 2, t1[len(t1) // 2])),
                         via_engine_exeOp=dict(stats(te), GBps_median=gbps(16 * per_rank * 2, te[len(te) // 2])))
                     g.destroy()
@@ -918,7 +918,7 @@ def main():
                 extras["op_64KiB_direct_launch"] = stats(t)
                 g1 = hip.Graph([dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)])
                 t = event_times_us(torch, lambda: g1.run(stream), 200, 20)
-                extras["op_64KiB_via_queue"] = dict(stats(t), launch=launch_kind(g1.info()),
+                extras["op_64KiB_via_queue"] = dict(stats(t), launch=launch_kind(g1),
                                                     through_the_persistent_drain=through_the_drain(
                                                         torch, hip, [dict(dtype="bf16", compute="sum", ins=[x, y], outs=[z], count=n64)], stream, 200))
                 g1.destroy()
@@ -967,7 +967,7 @@ def main():
                     "one_persistent_launch": dict(stats(t), us_per_op=round(med / len(low), 4), GBps_median=gbps(sched_bytes, med),
                                                   GBps_moved_median=gbps(sched_moved, med)),
                     "one_persistent_launch_without_chains": unchained,
-                    "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"], "launch": launch_kind(ginfo),
+                    "ops": len(low), "queue_entries": ginfo["n_tiles"], "workgroups": ginfo["n_workgroups"], "launch": launch_kind(g),
                     "algorithmic_bytes": sched_bytes, "bytes_moved": sched_moved,
                     "note": "GBps_median counts the algorithmic bytes of the 4096 ops; chains of 14 ops keep the value in registers "
                             "and skip stores they overwrite themselves (bytes_moved, GBps_moved_median).  one_persistent_launch is one "

@@ -302,6 +302,10 @@ int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier, int 
  * number of launches for a graph that runs as plain launches; n_workgroups = width of the launch. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 
+/* How the graph runs, for inspection: *kind = 0 the persistent drain, 1 a wide launch, 2 plain launches
+ * (see pccl_hip_graph_create).  No counterpart in the reference. */
+int pccl_hip_graph_launch_kind(void *graph, int *kind);
+
 /* signal_base the NEXT pccl_hip_graph_run of this graph will use: a party outside the
  * graph that wants to satisfy a GET_NOTIFIED(value) stores *base + value to the word.
  * The run number itself lives on the device and moves on with every execution of the

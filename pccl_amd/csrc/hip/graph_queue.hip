@@ -1863,6 +1863,14 @@ int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_
   return PCCL_OK;
 }
 
+int pccl_hip_graph_launch_kind(void *graph, int *kind) {
+  pccl_host::clear_error();
+  Graph *G = (Graph *)graph;
+  if (!G || !kind) return fail(PCCL_ERR_INVALID_ARG, "graph_launch_kind: null argument");
+  *kind = G->as_launches ? 2 : G->wide ? 1 : 0;
+  return PCCL_OK;
+}
+
 int pccl_hip_classify_dependencies(const pccl_op_desc *ops, int n_ops, const int *parts, unsigned char *kinds) {
   pccl_host::clear_error();
   if (n_ops < 0 || (n_ops > 0 && (!ops || !parts))) return fail(PCCL_ERR_INVALID_ARG, "classify_dependencies: bad arguments");

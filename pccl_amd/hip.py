@@ -83,6 +83,7 @@ def lib():
         L.pccl_hip_graph_status.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint)]
         L.pccl_hip_graph_rebind.argtypes = [vp, vp, vp, cl, vp]
         L.pccl_hip_graph_info.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.pccl_hip_graph_launch_kind.argtypes = [vp, ctypes.POINTER(ci)]
         L.pccl_hip_classify_dependencies.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), vp]
         L.pccl_hip_plan_chains.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ci, ctypes.POINTER(ci)]
         L.pccl_hip_plan_signals.argtypes = [ctypes.POINTER(OpDesc), ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
@@ -312,6 +313,12 @@ class Graph:
         lay, nt, nw = ctypes.c_void_p(None), ctypes.c_int(0), ctypes.c_int(0)
         _check(lib().pccl_hip_graph_info(self._h, ctypes.byref(lay), ctypes.byref(nt), ctypes.byref(nw)))
         return {"device_layout": lay.value, "n_tiles": nt.value, "n_workgroups": nw.value}
+
+    def launch_kind(self):
+        """'drain' (the persistent kernel), 'wide' (one workgroup per entry) or 'launches' (plain launches)."""
+        kind = ctypes.c_int(0)
+        _check(lib().pccl_hip_graph_launch_kind(self._h, ctypes.byref(kind)))
+        return ("drain", "wide", "launches")[kind.value]
 
     def dependency_kinds(self):
         """One flag per dependency (ops in uid order, dependencies in list order): 1 = met part

@@ -651,6 +651,7 @@ def test_wide_launch_refuses_a_rebind_that_makes_an_entry_wait(hip, oracle):
     g = hip.Graph([dict(dtype="f32", compute="sum", ins=[dA.ptr, db.ptr], outs=[dt.ptr], count=count, deps=[]),
                    dict(dtype="f32", compute="sum", ins=[dt.ptr, dc.ptr], outs=[du.ptr], count=count, deps=[0])])
     info = g.info()
+    assert g.launch_kind() == "wide"
     assert info["n_workgroups"] == info["n_tiles"] == (4 * count + 8191) // 8192, info  # one workgroup per 8 KiB block of the chain
     t = oracle.reduce("f32", "sum", [a_full[:count], b])
     u = oracle.reduce("f32", "sum", [t, c])
@@ -705,7 +706,7 @@ def test_wide_launch_and_persistent_drain_leave_the_same_bytes(hip, oracle, monk
     ops, checks = build()
     g = hip.Graph(ops)
     info = g.info()
-    assert info["n_workgroups"] == info["n_tiles"], info  # a wide launch
+    assert g.launch_kind() == "wide" and info["n_workgroups"] == info["n_tiles"], info
     g.trace(True)
     for _ in range(2):
         for do, _, _ in checks: do.upload(np.zeros(do.count, dtype=np.uint16))
@@ -719,7 +720,7 @@ def test_wide_launch_and_persistent_drain_leave_the_same_bytes(hip, oracle, monk
     monkeypatch.setenv("PCCL_HIP_WIDE", "0")
     g = hip.Graph(ops)
     info = g.info()
-    assert info["n_workgroups"] <= 4096 and info["n_workgroups"] <= info["n_tiles"]
+    assert g.launch_kind() == "drain" and info["n_workgroups"] <= 4096 and info["n_workgroups"] <= info["n_tiles"]
     for do, _, _ in checks: do.upload(np.zeros(do.count, dtype=np.uint16))
     _run_and_check(torch, hip, g, len(ops))
     for k, (do, want, _) in enumerate(checks):
