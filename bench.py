@@ -334,6 +334,28 @@ def queue_timeline(torch, hip, graph, stream, runs=3):
             "last_part_end_by_workgroup_us_p5_p50_p100": [q([float(dn[wg == w].max()) for w in groups], p) for p in (5, 50, 100)]}
 
 
+def wide_timeline(torch, hip, graph, stream, runs=3):
+    """A wide launch's entries in time (one short-lived workgroup per entry; first timestamp when the workgroup
+    has its record, last when its stores are out): how long an entry lives, when the last one starts, and how
+    many are running at tenths of the run."""
+    import numpy as np
+    graph.trace(True)
+    for _ in range(runs):
+        graph.run(stream)
+        torch.cuda.synchronize()
+    tr = graph.read_trace(stream)
+    graph.trace(False)
+    tr = tr[tr[:, 1] > 0]
+    t0 = int(tr[:, 1].min())
+    start, done = ((tr[:, k].astype(np.int64) - t0) / 100.0 for k in (1, 3))
+    end = float(done.max())
+    life = done - start
+    return {"traced_run_us": round(end, 1), "entries": int(len(tr)),
+            "entry_us_p5_p50_p95_max": [round(float(np.percentile(life, p)), 1) for p in (5, 50, 95, 100)],
+            "last_entry_starts_at_us": round(float(start.max()), 1),
+            "running_at_tenths_of_the_run": [int(((start <= x) & (done > x)).sum()) for x in np.linspace(0.0, end, 11)[1:-1]]}
+
+
 def timeline_main():
     import torch
     from pccl_amd import hip, lang
@@ -367,6 +389,15 @@ def timeline_main():
         g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
         t = event_times_us(torch, lambda: g.run(stream), 20, 3)
         out[kind] = dict(queue_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
+        g.destroy()
+        del os.environ["PCCL_HIP_WIDE"]  # ... and the same graph as the wide launch it runs as by default
+        try:
+            g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+        finally:
+            os.environ["PCCL_HIP_WIDE"] = "0"
+        if g.launch_kind() == "wide":
+            t = event_times_us(torch, lambda: g.run(stream), 20, 3)
+            out[kind]["as_the_wide_launch"] = dict(wide_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
         g.destroy()
     print(json.dumps({"queue_timeline": out}))
 
