@@ -124,7 +124,8 @@ def through_the_drain(torch, hip, bound_ops, stream, steps=20):
 
 
 def launch_kind(graph):
-    return {"wide": "wide (one workgroup per entry)", "drain": "persistent drain", "launches": "plain launches"}[graph.launch_kind()]
+    return {"wide": "wide (one workgroup per entry)", "drain": "persistent drain", "launches": "plain launches",
+            "chains": "wide (a few chains, one workgroup per 4 KiB of each)"}[graph.launch_kind()]
 
 
 def queue_bytes_moved(hip, bound_ops, elem_bytes):
@@ -395,7 +396,7 @@ def timeline_main():
             g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
         finally:
             os.environ["PCCL_HIP_WIDE"] = "0"
-        if g.launch_kind() == "wide":
+        if g.launch_kind() in ("wide", "chains"):
             t = event_times_us(torch, lambda: g.run(stream), 20, 3)
             out[kind]["as_the_wide_launch"] = dict(wide_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
         g.destroy()

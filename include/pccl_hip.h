@@ -220,7 +220,16 @@ typedef struct pccl_op_desc {
  * 9.7 -> 6.5 us; entries outside one-pass chains are cut into 32 KiB parts once they move 192 MiB or more).
  * The device arena, graph_info, graph_trace and results are the same; graph_status reports every op complete
  * once the stream has drained (the launch's end is the graph's completion; *completed_operator on the device
- * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0: never. */
+ * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0: never.
+ * Such a graph of at most 16 entries, each of which is one fold (one op of 1..8 inputs, with a COPY of its
+ * result that it stores itself; or a chain that runs in one pass, takes at most 8 inputs in all and leaves
+ * its final value in at most 8 outputs, every earlier output being overwritten by a later op of the chain:
+ * the 14 ops of a ring all-reduce's chunk), all ops of one element size, runs in the shape of a direct
+ * launch instead: a workgroup per 4 KiB of every stream of a chain, the chains' operands in a small table of
+ * the arena that all workgroups of a chain share (ring all-reduce over 8 resident ranks x 1 / 32 / 64 MiB
+ * 9.6 / 84.5 / 200 -> 6.9 / 80-82 / 172 us, direct all-reduce 8 x 32 MiB 88 -> 78 us = one 8 -> 8 launch).
+ * graph_info then reports workgroups for n_tiles, graph_trace records one entry per workgroup.
+ * PCCL_HIP_CHAIN_LAUNCH=0: the table-driven wide launch for these too. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);
 
@@ -246,8 +255,8 @@ int pccl_hip_graph_status(void *graph, void *stream, unsigned int *completed,
  * PCCL_ERR_MISALIGNED and changes nothing.  A graph that runs as a wide launch (see
  * pccl_hip_graph_create) cannot wait inside the launch: a move after which one of its entries
  * would have to wait for another (an op that no longer may run behind its predecessor part by
- * part) returns PCCL_ERR_UNSUPPORTED and changes nothing; create the graph again for such
- * operands (Engine::exeOp does). */
+ * part, or chains that come out differently) returns PCCL_ERR_UNSUPPORTED and changes nothing;
+ * create the graph again for such operands (Engine::exeOp does). */
 int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_base, long nbytes,
                           void *stream);
 
@@ -302,8 +311,9 @@ int pccl_hip_plan_signals(const pccl_op_desc *ops, int n_ops, int *carrier, int 
  * number of launches for a graph that runs as plain launches; n_workgroups = width of the launch. */
 int pccl_hip_graph_info(void *graph, void **device_layout, int *n_tiles, int *n_workgroups);
 
-/* How the graph runs, for inspection: *kind = 0 the persistent drain, 1 a wide launch, 2 plain launches
- * (see pccl_hip_graph_create).  No counterpart in the reference. */
+/* How the graph runs, for inspection: *kind = 0 the persistent drain, 1 a wide launch, 2 plain launches,
+ * 3 a wide launch in the shape of a direct one (a few chains that are each one fold); see
+ * pccl_hip_graph_create.  No counterpart in the reference. */
 int pccl_hip_graph_launch_kind(void *graph, int *kind);
 
 /* signal_base the NEXT pccl_hip_graph_run of this graph will use: a party outside the

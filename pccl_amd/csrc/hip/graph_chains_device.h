@@ -1,0 +1,192 @@
+// graph_chains_device.h -- a graph of a few independent chains as ONE launch in the shape of the direct
+// kernels: the chains' operands come through a table that all workgroups share.
+//
+// Open to graphs whose queue entries wait for nothing (as for any wide launch, graph_queue_device.h)
+// when every entry is either one op or a chain that comes down to "fold these inputs, store the
+// result to these outputs": the head's inputs folded like one reduction, then one more input per
+// later op, each fold rounded to the element type where the op's store would round it, and every
+// output that survives (an output that a later op of the chain writes again is never stored) holding
+// the chain's final value.  A ring all-reduce over ranks that live on one device is eight such
+// chains (eight inputs, eight outputs each), a direct all-reduce eight folds 8 -> 8.
+// A workgroup takes 4 KiB of every stream of its chain, one pack per lane: all loads at once, the
+// folds, all stores, like reduce_copy_lean_kernel (packs cut on output 0's 16-byte boundaries, the other
+// operands at whatever element-aligned address that gives them, the few elements in front of the
+// first and behind the last pack by the chain's last workgroup).  Which chain a workgroup belongs to follows from the
+// launch's arguments alone (first workgroup of every chain); the chain's row of the table is the same
+// for all its workgroups, so it is fetched once per compute unit and then comes from the scalar cache:
+// no per-entry record, no table staged through LDS, no barrier in front of the first load, and
+// workgroups that live a fifth as long as a wide launch's 16 KiB entries, which is what that launch
+// loses against a direct one at both ends of an entry's life.  Ring all-reduce over 8 resident ranks,
+// 112 ops, wide launch -> this: see graph_queue.hip (chains_launch_of).
+// The table lives in the graph's arena: a rebind rewrites it like the payloads, and launches that a
+// stream capture has recorded follow.
+#pragma once
+#include "graph_queue_device.h"
+#include "reduce_copy_kernel.h"
+
+namespace pccl_queue {
+
+constexpr int kMaxLaunchChains = 16;
+constexpr int kChainStreams = 8;  // inputs, and outputs, of one chain
+
+struct LaunchChain {
+  unsigned long long in[kChainStreams];   // the head's inputs, then the other input of every later op that has one
+  unsigned long long out[kChainStreams];  // the surviving outputs
+  long long count;                        // elements of every stream
+  int n_head;                             // inputs folded as one reduction (the head op's)
+  int n_in, n_out;
+  unsigned int fed;                       // bit k (k >= n_head): the handed-on value is the second operand of the fold with input k
+  int uid;                                // the head op (trace records)
+  unsigned int n_wg;                      // workgroups of this chain: one per 4 KiB of floor(bytes / 16) packs, at least one
+};
+static_assert(sizeof(LaunchChain) == 160, "launch chain row");
+
+// The launch's arguments.  Nothing here depends on an address (a recorded launch keeps its copy).
+struct ChainsLaunch {
+  const LaunchChain *chains;
+  unsigned long long *trace;                 // per workgroup: kTraceWords words, or null
+  unsigned int first_wg[kMaxLaunchChains];   // first workgroup of chain k; beyond the last chain: 0xffffffff
+  int rotate;                                // workgroup -> chunk rotation inside a chain (rotated_chunk)
+};
+
+template <class D, class Op, int N>
+__device__ __forceinline__ u32x4 fold_head(const u32x4 *v) {
+  u32x4 w[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) w[k] = v[k];
+  return fold_pack<D, Op, N>(w);
+}
+
+template <class D, class Op, int N>
+__device__ __forceinline__ typename D::elem_t fold_head_elem(const typename D::elem_t *v) {
+  typename D::elem_t w[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) w[k] = v[k];
+  return D::template elem<Op, N>(w);
+}
+
+// MEM: kLaunchMemCached or kLaunchMemStreamWriteThrough (reduce_copy_kernel.h)
+template <int DT, class Op, int MEM>
+__global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch a) {
+  typedef Dtype<DT> D;
+  typedef typename D::elem_t E;
+  constexpr int kEpp = 16 / D::kElemBytes;
+  D::wave_init();
+  // (through the buffer instructions: the operands' addresses come out of memory, not out of the
+  // kernel's pointer arguments, and a plain access through such an address would be a flat one; they
+  // also take the operands that are only element-aligned)
+  constexpr int kLdPolicy = MEM == pccl_dev::kLaunchMemCached ? 0 : 2;             // nt
+  constexpr int kStPolicy = MEM == pccl_dev::kLaunchMemCached ? 0 : kCachePolicySc1;
+  const unsigned int b = blockIdx.x;
+  int ci = 0;
+#pragma unroll
+  for (int k = 1; k < kMaxLaunchChains; ++k) ci += b >= a.first_wg[k] ? 1 : 0;  // (first_wg ascends)
+  const LaunchChain *c = a.chains + ci;  // uniform: scalar loads
+  const unsigned int k = b - a.first_wg[ci];
+  const unsigned int n_chunks = c->n_wg;
+  const long long count = c->count;
+  const int n_head = c->n_head, n_in = c->n_in, n_out = c->n_out;
+  const unsigned int fed = c->fed;
+  // (the whole row before anything is stored: the loads stay scalar)
+  unsigned long long in[kChainStreams], out[kChainStreams];
+#pragma unroll
+  for (int i = 0; i < kChainStreams; ++i) {
+    in[i] = c->in[i];
+    out[i] = c->out[i];
+  }
+  const int uid = c->uid;
+  const unsigned int chunk = a.rotate ? pccl_dev::rotated_chunk(k, n_chunks) : k;
+  unsigned long long *trace = nullptr;
+  if (a.trace && threadIdx.x == 0) {
+    trace = a.trace + (size_t)b * kTraceWords;
+    const unsigned long long now = wall_clock64();
+    trace[kTraceWhat] = (unsigned long long)(unsigned int)uid | ((unsigned long long)chunk << 32) | ((unsigned long long)(b & 0xfffu) << 52);
+    trace[kTraceClaimed] = now;
+    trace[kTraceReady] = now;
+  }
+  // packs are cut so that output 0 is 16-byte aligned; the elements in front of the first pack and
+  // behind the last one are left to the chain's last workgroup
+  long long peel = (long long)((16 - (out[0] & 15)) & 15) / D::kElemBytes;
+  if (peel > count) peel = count;
+  const long long n_packs = (count - peel) / kEpp;
+  const size_t wg_off = (size_t)peel * D::kElemBytes + (size_t)chunk * (kBlock * 16);
+  const unsigned int lane_off = threadIdx.x * 16u;
+  if ((long long)chunk * kBlock + threadIdx.x < n_packs) {
+    u32x4 v[kChainStreams];
+#pragma unroll
+    for (int i = 0; i < kChainStreams; ++i)
+      if (i < n_in) v[i] = __builtin_amdgcn_raw_buffer_load_b128(whole_buffer((const char *)in[i] + wg_off), (int)lane_off, 0, kLdPolicy);
+    u32x4 cur;
+    switch (n_head) {
+      case 1: cur = v[0]; break;
+      case 2: cur = fold_head<D, Op, 2>(v); break;
+      case 3: cur = fold_head<D, Op, 3>(v); break;
+      case 4: cur = fold_head<D, Op, 4>(v); break;
+      case 5: cur = fold_head<D, Op, 5>(v); break;
+      case 6: cur = fold_head<D, Op, 6>(v); break;
+      case 7: cur = fold_head<D, Op, 7>(v); break;
+      default: cur = fold_head<D, Op, 8>(v); break;
+    }
+#pragma unroll
+    for (int i = 1; i < kChainStreams; ++i)
+      if (i >= n_head && i < n_in) cur = ((fed >> i) & 1u) ? fold_two<D, Op>(v[i], cur) : fold_two<D, Op>(cur, v[i]);
+#pragma unroll
+    for (int j = 0; j < kChainStreams; ++j)
+      if (j < n_out) __builtin_amdgcn_raw_buffer_store_b128(cur, whole_buffer((char *)out[j] + wg_off), (int)lane_off, 0, kStPolicy);
+  }
+  if (k == n_chunks - 1 && threadIdx.x >= kBlock - kWave) {  // fewer than two packs' worth of elements: one per lane
+    const long long tail_begin = peel + n_packs * kEpp, n_edge = peel + (count - tail_begin);
+    const long long e = (long long)threadIdx.x - (kBlock - kWave);
+    if (e < n_edge) {
+      const long long i = e < peel ? e : tail_begin + (e - peel);
+      E x[kChainStreams];
+#pragma unroll
+      for (int s = 0; s < kChainStreams; ++s)
+        if (s < n_in) x[s] = ((const E *)in[s])[i];
+      E cur;
+      switch (n_head) {
+        case 1: cur = x[0]; break;
+        case 2: cur = fold_head_elem<D, Op, 2>(x); break;
+        case 3: cur = fold_head_elem<D, Op, 3>(x); break;
+        case 4: cur = fold_head_elem<D, Op, 4>(x); break;
+        case 5: cur = fold_head_elem<D, Op, 5>(x); break;
+        case 6: cur = fold_head_elem<D, Op, 6>(x); break;
+        case 7: cur = fold_head_elem<D, Op, 7>(x); break;
+        default: cur = fold_head_elem<D, Op, 8>(x); break;
+      }
+#pragma unroll
+      for (int s = 1; s < kChainStreams; ++s)
+        if (s >= n_head && s < n_in) {
+          const E two[2] = {((fed >> s) & 1u) ? x[s] : cur, ((fed >> s) & 1u) ? cur : x[s]};
+          cur = D::template elem<Op, 2>(two);
+        }
+#pragma unroll
+      for (int j = 0; j < kChainStreams; ++j)
+        if (j < n_out) ((E *)out[j])[i] = cur;
+    }
+  }
+  if (trace) {
+    settle_stores();
+    trace[kTraceDone] = wall_clock64();
+  }
+}
+
+typedef void (*ChainsKernel)(const ChainsLaunch);
+// The instances of one dtype; defined in graph_chains_inst_<dtype>.hip.  mem: 0 cached, otherwise
+// non-temporal loads and write-through stores.
+template <int DT>
+ChainsKernel chains_for_compute(int compute, int mem);
+
+#define PCCL_DEFINE_CHAINS_FOR_COMPUTE(DT)                                                                                  \
+  template <>                                                                                                               \
+  ChainsKernel chains_for_compute<DT>(int compute, int mem) {                                                               \
+    constexpr int kC = pccl_dev::kLaunchMemCached, kW = pccl_dev::kLaunchMemStreamWriteThrough;                             \
+    switch (compute) {                                                                                                      \
+      case PCCL_SUM: return mem ? graph_chains_kernel<DT, OpSum, kW> : graph_chains_kernel<DT, OpSum, kC>;                  \
+      case PCCL_PROD: return mem ? graph_chains_kernel<DT, OpProd, kW> : graph_chains_kernel<DT, OpProd, kC>;               \
+      case PCCL_MIN: return mem ? graph_chains_kernel<DT, OpMin, kW> : graph_chains_kernel<DT, OpMin, kC>;                  \
+      default: return mem ? graph_chains_kernel<DT, OpMax, kW> : graph_chains_kernel<DT, OpMax, kC>;                        \
+    }                                                                                                                       \
+  }
+
+}  // namespace pccl_queue

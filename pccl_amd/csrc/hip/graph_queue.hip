@@ -58,6 +58,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "graph_chains_device.h"
 #include "graph_queue_device.h"
 
 using namespace pccl_dev;
@@ -158,6 +159,15 @@ struct Graph {
   unsigned wide_lds = 0;           // dynamic LDS of the wide launch (never touched: an occupancy cap like the direct kernels')
   bool wide_small = false;         // one-pass chains in 8 KiB blocks (the SMALL instances of wide_body)
   long long wide_chain_bytes = 0;  // build_graph's finding: bytes the ops of one-pass chains name
+  // A wide launch of a few chains that are each one fold (graph_chains_device.h): the kernel, its
+  // arguments (the table of the chains' operands is in the arena at chains_off), its grid and LDS cap.
+  bool chains_launch = false;
+  ChainsKernel chains_kernel = nullptr;
+  ChainsLaunch chains_args = {};
+  size_t chains_off = 0;
+  unsigned chains_grid = 0, chains_lds = 0;
+  int chains_mem = 0, chains_dtype = 0, chains_compute = 0;
+  const Graph *fixed_chains = nullptr;  // build_graph: the launch must come out like this graph's (a rebuild in place)
   // A graph that runs as plain launches instead (see plan_launches): no arena, no drain kernel.
   bool as_launches = false;
   std::vector<pccl_op_desc> launches;  // in an order that respects the dependencies (deps unused)
@@ -741,6 +751,111 @@ void fill_chain_table(const std::vector<int> &words, int n_ops, const char *payl
   }
 }
 
+ChainsKernel chains_kernel_for(int dtype, int compute, int mem) {
+  switch (dtype) {
+    case PCCL_F32: return chains_for_compute<PCCL_F32>(compute, mem);
+    case PCCL_I32: return chains_for_compute<PCCL_I32>(compute, mem);
+    case PCCL_U32: return chains_for_compute<PCCL_U32>(compute, mem);
+    case PCCL_F64: return chains_for_compute<PCCL_F64>(compute, mem);
+    case PCCL_BF16: return chains_for_compute<PCCL_BF16>(compute, mem);
+    case PCCL_F16: return chains_for_compute<PCCL_F16>(compute, mem);
+    case PCCL_F8E4M3: return chains_for_compute<PCCL_F8E4M3>(compute, mem);
+    default: return chains_for_compute<PCCL_F8E5M2>(compute, mem);
+  }
+}
+
+// PCCL_HIP_CHAIN_LAUNCH=0: graphs that could run as graph_chains_kernel run as the table-driven wide launch.
+bool chain_launch_on() {
+  const char *env = getenv("PCCL_HIP_CHAIN_LAUNCH");
+  return !(env && env[0] == '0');
+}
+
+// The rows of a graph that runs as graph_chains_kernel (graph_chains_device.h), one per queued op in op
+// order, from the ops as they stand and their chain words; false when the graph does not fit: more than
+// kMaxLaunchChains queued ops, an op or chain that is not one fold with all surviving outputs holding its
+// final value (a chain through memory other than a copy stored by its producer; an output of a one-pass
+// chain that no later op overwrites although a later op still folds), more than kChainStreams inputs or
+// outputs, a fold in another dtype or compute op than the graph's kernel, an op of another element size.
+// Which outputs survive depends on the operands' addresses, whether the graph fits does not, short of a
+// rebind that changes the chains themselves.  The caller has made sure that no queued op waits for anything.
+bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<int> &words, int dtype, int compute,
+                      std::vector<LaunchChain> *rows) {
+  const int n = (int)ops.size();
+  std::vector<char> member(n, 0);
+  for (int i = 0; i < n; ++i) {
+    const int next = words[(size_t)kChainWords * i + kChainNext];
+    if (next >= 0) member[next] = 1;
+  }
+  rows->clear();
+  for (int h = 0; h < n; ++h) {
+    if (member[h]) continue;
+    if ((int)rows->size() == kMaxLaunchChains) return false;
+    std::vector<int> steps;
+    for (int u = h; u >= 0; u = words[(size_t)kChainWords * u + kChainNext]) steps.push_back(u);
+    const pccl_op_desc &head = ops[h];
+    const long long bytes = (long long)head.count * elem_bytes(head.dtype);
+    if (head.count <= 0 || bytes / 16 / kBlock >= (1ll << 31)) return false;
+    LaunchChain c;
+    memset(&c, 0, sizeof(c));
+    c.uid = h;
+    c.count = head.count;
+    c.n_wg = (unsigned int)std::max<long long>(1, (bytes / 16 + kBlock - 1) / kBlock);
+    bool ok = true;
+    auto folds_like_the_kernel = [&](const pccl_op_desc &o) { return o.n_in == 1 || (o.dtype == dtype && o.compute == compute); };
+    auto add_in = [&](const void *p) {
+      if (c.n_in == kChainStreams) { ok = false; return; }
+      c.in[c.n_in++] = (unsigned long long)(uintptr_t)p;
+    };
+    auto add_out = [&](const void *p) {
+      if (c.n_out == kChainStreams) { ok = false; return; }
+      c.out[c.n_out++] = (unsigned long long)(uintptr_t)p;
+    };
+    for (int u : steps) {
+      const pccl_op_desc &o = ops[u];
+      ok = ok && (o.primitive == PCCL_COPY || o.primitive == PCCL_REDUCE) && o.n_in >= 1 && o.n_in <= PCCL_MAX_INPUTS &&
+           folds_like_the_kernel(o) && o.count == head.count && elem_bytes(o.dtype) == elem_bytes(dtype);
+    }
+    if (!ok) return false;
+    c.n_head = head.n_in;
+    for (int k = 0; k < head.n_in; ++k) add_in(head.ins[k]);
+    const int forward = words[(size_t)kChainWords * h + kChainForward];
+    if (steps.size() == 1) {
+      for (int j = 0; j < head.n_out; ++j) add_out(head.outs[j]);
+    } else if (forward == 1) {
+      size_t last_fold = 0;  // the last op that changes the value
+      for (size_t t = 1; t < steps.size(); ++t) {
+        const pccl_op_desc &o = ops[steps[t]];
+        if (o.n_in == 2) {
+          const int fed = words[(size_t)kChainWords * steps[t] + kChainForward];
+          if (fed == 1) c.fed |= 1u << c.n_in;
+          add_in(o.ins[1 - fed]);
+          last_fold = t;
+        } else if (o.n_in != 1) {
+          ok = false;
+        }
+      }
+      for (size_t t = 0; t < steps.size() && ok; ++t)
+        for (int j = 0; j < ops[steps[t]].n_out && ok; ++j) {
+          const void *addr = ops[steps[t]].outs[j];
+          bool written_again = false;  // (as in fill_chain_table)
+          for (size_t later = t + 1; later < steps.size() && !written_again; ++later)
+            for (int k = 0; k < ops[steps[later]].n_out; ++k) written_again = written_again || ops[steps[later]].outs[k] == addr;
+          if (written_again) continue;
+          if (t < last_fold) ok = false;  // an earlier value that stays in memory
+          else add_out(addr);
+        }
+    } else if (steps.size() == 2 && words[(size_t)kChainWords * steps[1] + kChainForward] == kChainFolded) {
+      for (int j = 0; j < head.n_out; ++j) add_out(head.outs[j]);
+      for (int j = 0; j < ops[steps[1]].n_out; ++j) add_out(ops[steps[1]].outs[j]);
+    } else {
+      ok = false;
+    }
+    if (!ok || c.n_out < 1) return false;
+    rows->push_back(c);
+  }
+  return !rows->empty();
+}
+
 // plan_chains for a graph's ops, and in the length word of every op the signal ops it carries: a
 // workgroup that completes the op counts those complete with it (such an op is in no chain, so the
 // word would otherwise say 1).
@@ -1220,6 +1335,53 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as a wide launch (an entry waits for another, "
                                         "or there are more entries than the launch was made for)");
   }
+  // A wide launch of at most kMaxLaunchChains entries that are each one fold runs in the shape of the
+  // direct kernels instead (graph_chains_device.h), with the direct launch's rules for one launch of all
+  // this traffic (reduce_copy.hip): streaming treatment and chunk rotation from 48 MiB in all, an
+  // occupancy cap beyond the Infinity Cache.
+  std::vector<LaunchChain> launch_rows;
+  G->chains_launch = false;
+  if (G->want_wide && !mixed && (G->fixed_chains ? G->fixed_chains->chains_launch : chain_launch_on()) &&
+      launch_chains_of(G->eff, G->chain_words, g_dtype, g_compute, &launch_rows)) {
+    ChainsLaunch &a = G->chains_args;
+    memset(&a, 0, sizeof(a));
+    long long blocks = 0, total_bytes = 0;
+    int streams = 1;
+    bool folds = false;
+    for (size_t k = 0; k < (size_t)kMaxLaunchChains; ++k) {
+      a.first_wg[k] = k < launch_rows.size() ? (unsigned int)blocks : 0xffffffffu;
+      if (k >= launch_rows.size()) continue;
+      const LaunchChain &c = launch_rows[k];
+      blocks += c.n_wg;
+      total_bytes += (long long)(c.n_in + c.n_out) * c.count * elem_bytes(g_dtype);
+      streams = std::max(streams, c.n_in + c.n_out);
+      folds = folds || c.n_in > 1;
+    }
+    if (blocks < (1ll << 31)) {
+      G->chains_launch = true;
+      G->chains_grid = (unsigned)blocks;
+      G->chains_mem = total_bytes >= (48ll << 20) ? 1 : 0;
+      a.rotate = G->chains_mem;
+      G->chains_lds = 0;
+      if (total_bytes > (192ll << 20)) {
+        int wgs = std::max(2, std::min(8, (20 + streams / 2) / streams));
+        if (elem_bytes(g_dtype) == 1 && folds) wgs = std::max(wgs, 4);
+        if (wgs < 8) G->chains_lds = std::min(65536u, (unsigned)(160 * 1024 / wgs) - 256u);
+      }
+      G->chains_dtype = g_dtype;
+      G->chains_compute = g_compute;
+      G->chains_kernel = chains_kernel_for(g_dtype, g_compute, G->chains_mem);
+    }
+  }
+  if (const Graph *F = G->fixed_chains) {
+    // (launches that a stream capture has recorded carry the kernel, the grid and the arguments)
+    const bool same = F->chains_launch == G->chains_launch &&
+                      (!F->chains_launch || (F->chains_grid == G->chains_grid && F->chains_lds == G->chains_lds && F->chains_kernel == G->chains_kernel &&
+                                             F->chains_args.rotate == G->chains_args.rotate &&
+                                             !memcmp(F->chains_args.first_wg, G->chains_args.first_wg, sizeof(F->chains_args.first_wg))));
+    if (!same)
+      return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as the launch it was made for (its chains come out differently)");
+  }
 
   std::vector<int> succ_part_base(n_edges ? n_edges : 1, -1), n_part_next(n_ops, 0), n_part_pred(n_ops, 0);
   {
@@ -1279,11 +1441,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   const size_t off_entries = off; off = align_up(off + 8 * queue_room * kQueues, 256);
   // (a wide launch: a record per workgroup; room for one per part of every op, so that the layout does not move with the chain plan)
   const size_t off_wide = off;    if (G->want_wide) off = align_up(off + sizeof(WideEntry) * (size_t)std::max<long long>(tiles, 1), 256);
+  const size_t off_lchains = off; if (G->want_wide) off = align_up(off + sizeof(LaunchChain) * (size_t)kMaxLaunchChains, 256);
   const size_t arena_bytes = off;
 
   G->n_ops = n_ops;
-  G->total_tiles = (int)live_tiles;  // entries that are queued; the arena has room for an entry per part of every op
-  G->all_tiles = (int)tiles;
+  // entries that are queued (the arena has room for an entry per part of every op); a launch of chains: its workgroups, which is what a trace records
+  G->total_tiles = (int)(G->chains_launch ? (long long)G->chains_grid : live_tiles);
+  G->all_tiles = (int)std::max<long long>(tiles, G->total_tiles);
   G->payload_off = off_payload;
   G->kernel_elem_bytes = elem_bytes(g_dtype);
   if (G->fixed_kernel) {
@@ -1351,6 +1515,11 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   C->spin_limit = G->spin_limit;
   C->n_ops = (unsigned int)n_ops;
   C->wide_entries = G->want_wide ? (const WideEntry *)(dev + off_wide) : nullptr;
+  G->chains_off = off_lchains;
+  if (G->chains_launch) {
+    memcpy(img + off_lchains, launch_rows.data(), sizeof(LaunchChain) * launch_rows.size());
+    G->chains_args.chains = (const LaunchChain *)(dev + off_lchains);
+  }
   C->queue_count = (const int *)(dev + off_qcount);
   C->chain = (const int *)(dev + off_chain);
   C->chain_table = (const ForwardStep *)(dev + off_chain_table);
@@ -1475,6 +1644,7 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // never more workgroups than entries
   // (a rebuild in place keeps the count: launches that a stream capture has recorded carry it)
   G->n_wg = G->fixed_n_wg > 0 ? G->fixed_n_wg : (int)std::max<long long>(1, std::min<long long>(live_tiles, G->want_wide ? kMaxWideEntries : cap));
+  if (G->chains_launch) G->n_wg = (int)G->chains_grid;
   G->wide = G->want_wide;
   {
     // Entries without tickets (graph_queue_device.h): when there is at most one per workgroup
@@ -1631,11 +1801,18 @@ int pccl_hip_graph_run(void *graph, void *stream) {
   }
   if (G->total_tiles == 0) return PCCL_OK;
   GraphControl control;
+  ChainsLaunch args;
   {
     std::lock_guard<std::mutex> lock(G->mu);  // spin_limit may be changed by another thread
     memcpy(&control, G->image.data(), sizeof(control));
+    args = G->chains_args;
   }
-  hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), G->wide ? G->wide_lds : 0u, (hipStream_t)stream, control);
+  if (G->chains_launch) {
+    args.trace = control.trace;
+    hipLaunchKernelGGL(G->chains_kernel, dim3(G->chains_grid), dim3(kBlock), G->chains_lds, (hipStream_t)stream, args);
+  } else {
+    hipLaunchKernelGGL(G->kernel, dim3((unsigned)G->n_wg), dim3(kBlock), G->wide ? G->wide_lds : 0u, (hipStream_t)stream, control);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(PCCL_ERR_HIP, "graph_run launch failed: %s", hipGetErrorString(e));
   {
@@ -1764,6 +1941,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // finish first.  Only a failed upload can leave the graph unusable.
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
   const std::vector<pccl_op_desc> eff_next = effective_of(G, next);
+  std::vector<LaunchChain> rows_next;
   const std::vector<unsigned char> edges_after = classify_dependencies(eff_next, G->parts, G->topo, &G->part_eligible);
   if (edges_after != G->part_edge || plan_chains_of(G, eff_next, G->parts, edges_after, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
@@ -1778,6 +1956,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     fresh.fixed_kernel = G->kernel;
     fresh.forward_capable = G->forward_capable;
     fresh.want_wide = G->wide;  // (a wide launch stays one, or the rebind is refused before anything changes)
+    if (G->wide) fresh.fixed_chains = G;  // (... and runs as the same launch)
     fresh.wide_lds = G->wide_lds;
     fresh.wide_small = G->wide_small;
     char *old_dev = G->dev;
@@ -1811,6 +1990,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     G->all_tiles = fresh.all_tiles;
     G->n_wg = fresh.n_wg;
     G->wide_ok = fresh.wide_ok;
+    G->chains_args = fresh.chains_args;  // (the same launch as before; the table's address is the arena's)
+    G->chains_off = fresh.chains_off;
     G->device = fresh.device;
     G->kernel = fresh.kernel;
     G->descs.swap(fresh.descs);
@@ -1832,6 +2013,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
+  if (G->chains_launch && !launch_chains_of(eff_next, G->chain_words, G->chains_dtype, G->chains_compute, &rows_next))
+    return fail(PCCL_ERR_UNSUPPORTED, "graph_rebind: with these operands the graph no longer runs as the launch it was made for; create it again");
   G->descs.swap(next);
   for (size_t i = 0; i < G->eff.size(); ++i) {  // (the same ops: the dependency lists stay, the operands move)
     memcpy(G->eff[i].ins, eff_next[i].ins, sizeof(G->eff[i].ins));
@@ -1850,6 +2033,11 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->payload_off, payloads,
                                 G->fuse_table_off + sizeof(SignalFuse) * (size_t)G->n_ops - G->payload_off,
                                 hipMemcpyHostToDevice, (hipStream_t)stream));
+  if (G->chains_launch) {
+    memcpy(G->image.data() + G->chains_off, rows_next.data(), sizeof(LaunchChain) * rows_next.size());
+    PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->chains_off, G->image.data() + G->chains_off, sizeof(LaunchChain) * rows_next.size(),
+                                  hipMemcpyHostToDevice, (hipStream_t)stream));
+  }
   return PCCL_OK;
 }
 
@@ -1867,7 +2055,7 @@ int pccl_hip_graph_launch_kind(void *graph, int *kind) {
   pccl_host::clear_error();
   Graph *G = (Graph *)graph;
   if (!G || !kind) return fail(PCCL_ERR_INVALID_ARG, "graph_launch_kind: null argument");
-  *kind = G->as_launches ? 2 : G->wide ? 1 : 0;
+  *kind = G->as_launches ? 2 : G->chains_launch ? 3 : G->wide ? 1 : 0;
   return PCCL_OK;
 }
 

@@ -315,10 +315,11 @@ class Graph:
         return {"device_layout": lay.value, "n_tiles": nt.value, "n_workgroups": nw.value}
 
     def launch_kind(self):
-        """'drain' (the persistent kernel), 'wide' (one workgroup per entry) or 'launches' (plain launches)."""
+        """'drain' (the persistent kernel), 'wide' (one workgroup per entry), 'launches' (plain launches) or 'chains'
+        (a wide launch in the shape of a direct one: a few chains that are each one fold, a workgroup per 4 KiB)."""
         kind = ctypes.c_int(0)
         _check(lib().pccl_hip_graph_launch_kind(self._h, ctypes.byref(kind)))
-        return ("drain", "wide", "launches")[kind.value]
+        return ("drain", "wide", "launches", "chains")[kind.value]
 
     def dependency_kinds(self):
         """One flag per dependency (ops in uid order, dependencies in list order): 1 = met part

@@ -72,22 +72,30 @@ def test_ring_chains_in_one_pass(hip, oracle, monkeypatch, dtype, compute):
         monkeypatch.setenv("PCCL_HIP_CHAINS", "0")
         plain = hip.Graph(bound, tile_bytes=tile)
         monkeypatch.setenv("PCCL_HIP_CHAINS", "1")
-        g = hip.Graph(bound, tile_bytes=tile)
-        # 14 ops share the entries of one (the built-in choice may also cut a chain into fewer parts)
-        if tile:
-            assert g.info()["n_tiles"] * 14 == plain.info()["n_tiles"], (sizes, offsets)
-        else:
-            assert g.info()["n_tiles"] * 14 <= plain.info()["n_tiles"], (sizes, offsets)
+        # (at most 16 chains and the built-in cut: the graph runs as one launch of chains, a workgroup per 4 KiB;
+        # PCCL_HIP_CHAIN_LAUNCH=0: as entries that 14 ops share)
+        for chain_launch in ("1", "0"):
+            monkeypatch.setenv("PCCL_HIP_CHAIN_LAUNCH", chain_launch)
+            g = hip.Graph(bound, tile_bytes=tile)
+            if chain_launch == "1" and tile == 0 and len(sizes) <= 2:
+                assert g.launch_kind() == "chains", (sizes, offsets)
+            if g.launch_kind() != "chains":
+                # 14 ops share the entries of one (the built-in choice may also cut a chain into fewer parts)
+                if tile:
+                    assert g.info()["n_tiles"] * 14 == plain.info()["n_tiles"], (sizes, offsets)
+                else:
+                    assert g.info()["n_tiles"] * 14 <= plain.info()["n_tiles"], (sizes, offsets)
+            for it in range(2):
+                for b in dev["out"]:
+                    b.view().fill_(0xFF)
+                _run(torch, hip, g, len(ops))
+                for r in range(8):
+                    H.assert_bits_equal(dev["out"][r].download(), host["out"][r], "%s %s sizes %s offsets %s run %d rank %d (%s)"
+                                        % (dtype, compute, sizes, offsets, it, r, g.launch_kind()))
+                    assert dev["out"][r].guards_intact()
+            g.destroy()
         plain.destroy()
-        for it in range(2):
-            for b in dev["out"]:
-                b.view().fill_(0xFF)
-            _run(torch, hip, g, len(ops))
-            for r in range(8):
-                H.assert_bits_equal(dev["out"][r].download(), host["out"][r], "%s %s sizes %s offsets %s run %d rank %d"
-                                    % (dtype, compute, sizes, offsets, it, r))
-                assert dev["out"][r].guards_intact()
-        g.destroy()
+        monkeypatch.delenv("PCCL_HIP_CHAIN_LAUNCH")
 
 
 def test_two_outputs_and_value_handed_on_as_second_input(hip, oracle):
@@ -448,3 +456,114 @@ def test_later_op_writes_over_an_earlier_output_at_a_shift(hip, oracle):
         _run(torch, hip, g, 3)
         H.assert_bits_equal(dt.download(), ht, "t, count %d, several parts" % count)
         g.destroy()
+
+
+@pytest.mark.parametrize("dtype,compute", [("bf16", "sum"), ("f32", "prod"), ("f64", "min"), ("f8e4m3", "max"), ("i32", "sum")])
+def test_folds_and_their_broadcast_copies_as_one_launch_of_chains(hip, oracle, monkeypatch, dtype, compute):
+    """A direct all-reduce over 8 ranks (rank r folds slice r of all inputs, a copy broadcasts the result:
+    16 ops, 8 queue entries) plus independent ops of 1..8 inputs and several outputs, at most 16 entries in
+    all, none of which waits for anything: the graph runs as one launch of chains, a workgroup per 4 KiB,
+    whatever the operands' alignment.  Bits as through the persistent drain and as the CPU checker's."""
+    import torch
+    es = H.ELEM_BYTES[dtype]
+    kw = dict(mean=1.0, sigma=0.05) if compute == "prod" else dict(sigma=1.0)
+    for slice_elems, offsets in ((4096 // es * 3, (0, 0)), (1237, (es, 3 * es)), (7, (es, 0)), (40001, (0, max(4, es)))):
+        per_rank = 8 * slice_elems
+        host_in = [H.gen(dtype, per_rank, 1200, r, **kw) for r in range(8)]
+        dev_in = [H.DevBuf(torch, dtype, per_rank, offsets[0], src=host_in[r]) for r in range(8)]
+        dev_out = [H.DevBuf(torch, dtype, per_rank, offsets[1]) for _ in range(8)]
+        ops, want = [], [np.zeros(per_rank, dtype=H.STORAGE[dtype]) for _ in range(8)]
+        for r in range(8):
+            lo = r * slice_elems
+            ops.append(dict(dtype=dtype, compute=compute, ins=[d.ptr + lo * es for d in dev_in], outs=[dev_out[r].ptr + lo * es],
+                            count=slice_elems, deps=[]))
+            ops.append(dict(dtype=dtype, compute=compute, ins=[dev_out[r].ptr + lo * es],
+                            outs=[dev_out[d].ptr + lo * es for d in range(8) if d != r], count=slice_elems, deps=[len(ops) - 1]))
+            folded = oracle.reduce(dtype, compute, [x[lo:lo + slice_elems] for x in host_in])
+            for d in range(8):
+                want[d][lo:lo + slice_elems] = folded
+        extra = []
+        for k, (n_in, n_out, count) in enumerate(((1, 3, 5000), (3, 2, 999), (8, 1, 12345), (2, 8, 1), (5, 1, 4096 // es), (1, 1, 70001))):
+            srcs = [H.gen(dtype, count, 1300 + k, j, **kw) for j in range(n_in)]
+            ds = [H.DevBuf(torch, dtype, count, ((k + j) % 5) * es, src=x) for j, x in enumerate(srcs)]
+            do = [H.DevBuf(torch, dtype, count, ((k + 2 * j) % 7) * es) for j in range(n_out)]
+            ops.append(dict(dtype=dtype, compute=compute, ins=[d.ptr for d in ds], outs=[d.ptr for d in do], count=count, deps=[]))
+            extra.append((do, oracle.reduce(dtype, compute, srcs) if n_in > 1 else srcs[0], ds))
+        for form, env in (("chains", {}), ("wide", {"PCCL_HIP_CHAIN_LAUNCH": "0"}), ("drain", {"PCCL_HIP_WIDE": "0"})):
+            for k, v in env.items():
+                monkeypatch.setenv(k, v)
+            g = hip.Graph(ops)
+            for k in env:
+                monkeypatch.delenv(k)
+            assert g.launch_kind() == form, (form, g.launch_kind(), slice_elems)
+            if form == "chains":
+                g.trace(True)
+            for it in range(2):
+                for b in dev_out + [b for do, _, _ in extra for b in do]:
+                    b.view().fill_(0xFF)
+                _run(torch, hip, g, len(ops))
+                for r in range(8):
+                    H.assert_bits_equal(dev_out[r].download(), want[r], "%s %s %s slice %d run %d rank %d" % (form, dtype, compute, slice_elems, it, r))
+                    assert dev_out[r].guards_intact()
+                for k, (do, w, _) in enumerate(extra):
+                    for b in do:
+                        H.assert_bits_equal(b.download(), w, "%s %s %s extra op %d" % (form, dtype, compute, k))
+                        assert b.guards_intact()
+            if form == "chains":
+                tr = g.read_trace(_stream(torch))
+                info = g.info()
+                assert len(tr) == info["n_workgroups"] == info["n_tiles"] and (tr[:, 3] >= tr[:, 1]).all() and (tr[:, 1] > 0).all()
+            g.destroy()
+
+
+def test_launch_of_chains_follows_rebinds_also_when_recorded(hip, oracle):
+    """A ring all-reduce over 8 ranks that runs as one launch of chains: its operands move to other tensors
+    (other alignment included) by rebinds, eagerly and between replays of a HIP graph that recorded the
+    launch: the table of the chains' operands lives in the graph's arena, so the recorded launch follows.
+    A rebind that changes the chains themselves (the output tensor becomes the input tensor) is refused
+    and leaves the graph as it was."""
+    import torch
+    dtype, es = "bf16", 2
+    ops, per_rank = S.ring_allreduce_ops(8, [3001], dtype=dtype, compute="sum")
+    host = {"in": [H.gen(dtype, per_rank, 1400, r) for r in range(8)], "out": [np.zeros(per_rank, dtype=H.STORAGE[dtype]) for _ in range(8)]}
+    oracle.run_ops(S.materialise(ops, lambda b, r, e, n: host[b][r][e:e + n]), oracle.topo_sort(len(ops), S.edges_of(ops)))
+    # all ranks' tensors in one allocation each, so that one rebind moves all eight
+    ins = H.DevBuf(torch, dtype, 8 * per_rank, 0, src=np.concatenate(host["in"]))
+    outs = [H.DevBuf(torch, dtype, 8 * per_rank, off) for off in (0, 4, 40)]
+    ins2 = H.DevBuf(torch, dtype, 8 * per_rank, 12, src=np.concatenate(host["in"]))
+    where = {"in": ins, "out": outs[0]}
+    g = hip.Graph(S.materialise(ops, lambda b, r, e, n: where[b].ptr + (r * per_rank + e) * es))
+    assert g.launch_kind() == "chains"
+    stream = torch.cuda.Stream()
+    want = np.concatenate(host["out"])
+
+    def check(buf, what):
+        H.assert_bits_equal(buf.download(), want, what)
+        assert buf.guards_intact()
+
+    with torch.cuda.stream(stream):
+        g.run(stream.cuda_stream)
+        stream.synchronize()
+        check(outs[0], "eager")
+        g.rebind(outs[0].ptr, outs[1].ptr, 8 * per_rank * es, stream.cuda_stream)
+        g.rebind(ins.ptr, ins2.ptr, 8 * per_rank * es, stream.cuda_stream)
+        g.run(stream.cuda_stream)
+        stream.synchronize()
+        check(outs[1], "after rebinds to tensors of another alignment")
+        with pytest.raises(hip.PcclError) as e:
+            g.rebind(outs[1].ptr, ins2.ptr, 8 * per_rank * es, stream.cuda_stream)
+        assert e.value.code == hip.ERR_UNSUPPORTED
+        cg = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cg, stream=stream):
+            g.run(stream.cuda_stream)
+        current = outs[1]
+        for target in (outs[2], outs[0], outs[1]):
+            g.rebind(current.ptr, target.ptr, 8 * per_rank * es, stream.cuda_stream)
+            current = target
+            target.view().fill_(0xFF)
+            stream.synchronize()
+            cg.replay()
+            stream.synchronize()
+            check(target, "replay after a rebind")
+    assert g.status(stream.cuda_stream) == (len(ops), len(ops))
+    g.destroy()
