@@ -221,14 +221,16 @@ typedef struct pccl_op_desc {
  * The device arena, graph_info, graph_trace and results are the same; graph_status reports every op complete
  * once the stream has drained (the launch's end is the graph's completion; *completed_operator on the device
  * is not written by such a launch); graph_rebind see there.  PCCL_HIP_WIDE=0: never.
- * Such a graph of at most 16 entries, each of which is one fold (one op of 1..8 inputs, with a COPY of its
+ * Such a graph of at most 64 entries, each of which is one fold (one op of 2..8 inputs, with a COPY of its
  * result that it stores itself; or a chain that runs in one pass, takes at most 8 inputs in all and leaves
  * its final value in at most 8 outputs, every earlier output being overwritten by a later op of the chain:
- * the 14 ops of a ring all-reduce's chunk), all ops of one element size, runs in the shape of a direct
- * launch instead: a workgroup per 4 KiB of every stream of a chain, the chains' operands in a small table of
- * the arena that all workgroups of a chain share (ring all-reduce over 8 resident ranks x 1 / 32 / 64 MiB
- * 9.6 / 84.5 / 200 -> 6.9 / 80-82 / 172 us, direct all-reduce 8 x 32 MiB 88 -> 78 us = one 8 -> 8 launch).
- * graph_info then reports workgroups for n_tiles, graph_trace records one entry per workgroup.
+ * the 14 ops of a ring all-reduce's chunk) over at least four streams, all ops of one element size, runs in
+ * the shape of a direct launch instead: a workgroup per 4 KiB of every stream of a chain, the chains'
+ * operands in a small table of the arena that all workgroups of a chain share (ring all-reduce over 8
+ * resident ranks x 1 / 32 / 64 MiB 9.6 / 84.5 / 200 -> 7 / 80-83 / 172 us, direct all-reduce 8 x 32 MiB
+ * 88 -> 78-80 us = one 8 -> 8 launch).  graph_info then reports workgroups for n_tiles, graph_trace records
+ * one entry per workgroup.  Copies and folds over fewer streams fit that launch too but are better off with
+ * the table (PCCL_HIP_CHAIN_LAUNCH=2 takes it for them all the same).
  * PCCL_HIP_CHAIN_LAUNCH=0: the table-driven wide launch for these too. */
 #define PCCL_HIP_TILE_AUTO (-1l)
 int pccl_hip_graph_create(const pccl_op_desc *ops, int n_ops, long tile_bytes, void **graph);

@@ -1,4 +1,4 @@
-// graph_chains_device.h -- a graph of a few independent chains as ONE launch in the shape of the direct
+// graph_chains_device.h -- a graph of independent chains as ONE launch in the shape of the direct
 // kernels: the chains' operands come through a table that all workgroups share.
 //
 // Open to graphs whose queue entries wait for nothing (as for any wide launch, graph_queue_device.h)
@@ -11,13 +11,14 @@
 // A workgroup takes 4 KiB of every stream of its chain, one pack per lane: all loads at once, the
 // folds, all stores, like reduce_copy_lean_kernel (packs cut on output 0's 16-byte boundaries, the other
 // operands at whatever element-aligned address that gives them, the few elements in front of the
-// first and behind the last pack by the chain's last workgroup).  Which chain a workgroup belongs to follows from the
-// launch's arguments alone (first workgroup of every chain); the chain's row of the table is the same
+// first and behind the last pack by the chain's last workgroup).  Which chain a workgroup belongs to
+// follows from the launch's arguments alone (first workgroup of every chain; with more than
+// kLaunchChainGroups chains, of every group of chains, and the rows of the group say the rest); the chain's row of the table is the same
 // for all its workgroups, so it is fetched once per compute unit and then comes from the scalar cache:
 // no per-entry record, no table staged through LDS, no barrier in front of the first load, and
 // workgroups that live a fifth as long as a wide launch's 16 KiB entries, which is what that launch
 // loses against a direct one at both ends of an entry's life.  Ring all-reduce over 8 resident ranks,
-// 112 ops, wide launch -> this: see graph_queue.hip (chains_launch_of).
+// 112 ops, wide launch -> this: see graph_queue.hip (launch_chains_of).
 // The table lives in the graph's arena: a rebind rewrites it like the payloads, and launches that a
 // stream capture has recorded follow.
 #pragma once
@@ -26,7 +27,9 @@
 
 namespace pccl_queue {
 
-constexpr int kMaxLaunchChains = 16;
+constexpr int kLaunchChainGroups = 16;  // chains, or groups of up to kLaunchChainsPerGroup chains, that the launch's arguments name
+constexpr int kLaunchChainsPerGroup = 4;
+constexpr int kMaxLaunchChains = kLaunchChainGroups * kLaunchChainsPerGroup;
 constexpr int kChainStreams = 8;  // inputs, and outputs, of one chain
 
 struct LaunchChain {
@@ -38,15 +41,21 @@ struct LaunchChain {
   unsigned int fed;                       // bit k (k >= n_head): the handed-on value is the second operand of the fold with input k
   int uid;                                // the head op (trace records)
   unsigned int n_wg;                      // workgroups of this chain: one per 4 KiB of floor(bytes / 16) packs, at least one
+  unsigned int first_wg;                  // the chain's first workgroup
+  int reserved[7];
 };
-static_assert(sizeof(LaunchChain) == 160, "launch chain row");
+static_assert(sizeof(LaunchChain) == 192, "launch chain row");
 
 // The launch's arguments.  Nothing here depends on an address (a recorded launch keeps its copy).
 struct ChainsLaunch {
   const LaunchChain *chains;
   unsigned long long *trace;                 // per workgroup: kTraceWords words, or null
-  unsigned int first_wg[kMaxLaunchChains];   // first workgroup of chain k; beyond the last chain: 0xffffffff
-  int rotate;                                // workgroup -> chunk rotation inside a chain (rotated_chunk)
+  unsigned int first_wg[kLaunchChainGroups];  // first workgroup of chain k * group; beyond the last chain: 0xffffffff
+  int rotate;                                 // workgroup -> chunk rotation inside a chain (rotated_chunk)
+  int group;                                  // 1 for up to kLaunchChainGroups chains (the arguments alone say which chain a
+                                              // workgroup belongs to: a launch of many short-lived workgroups loses 5-8 % to
+                                              // a longer argument block), else up to kLaunchChainsPerGroup: the rows' first_wg decide
+  int n_chains;
 };
 
 template <class D, class Op, int N>
@@ -80,9 +89,17 @@ __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch
   const unsigned int b = blockIdx.x;
   int ci = 0;
 #pragma unroll
-  for (int k = 1; k < kMaxLaunchChains; ++k) ci += b >= a.first_wg[k] ? 1 : 0;  // (first_wg ascends)
+  for (int k = 1; k < kLaunchChainGroups; ++k) ci += b >= a.first_wg[k] ? 1 : 0;  // (first_wg ascends)
+  if (a.group > 1) {
+    ci *= a.group;
+    int more = 0;
+#pragma unroll
+    for (int k = 1; k < kLaunchChainsPerGroup; ++k)
+      more += (k < a.group && ci + k < a.n_chains && b >= a.chains[ci + k].first_wg) ? 1 : 0;
+    ci += more;
+  }
   const LaunchChain *c = a.chains + ci;  // uniform: scalar loads
-  const unsigned int k = b - a.first_wg[ci];
+  const unsigned int k = b - c->first_wg;
   const unsigned int n_chunks = c->n_wg;
   const long long count = c->count;
   const int n_head = c->n_head, n_in = c->n_in, n_out = c->n_out;

@@ -764,10 +764,11 @@ ChainsKernel chains_kernel_for(int dtype, int compute, int mem) {
   }
 }
 
-// PCCL_HIP_CHAIN_LAUNCH=0: graphs that could run as graph_chains_kernel run as the table-driven wide launch.
-bool chain_launch_on() {
+// PCCL_HIP_CHAIN_LAUNCH=0: graphs that could run as graph_chains_kernel run as the table-driven wide launch;
+// 2: every graph that fits that kernel runs as it, also where it is not the better choice (launch_chains_of).
+int chain_launch_mode() {
   const char *env = getenv("PCCL_HIP_CHAIN_LAUNCH");
-  return !(env && env[0] == '0');
+  return env && env[0] == '0' ? 0 : env && env[0] == '2' ? 2 : 1;
 }
 
 // The rows of a graph that runs as graph_chains_kernel (graph_chains_device.h), one per queued op in op
@@ -776,10 +777,18 @@ bool chain_launch_on() {
 // final value (a chain through memory other than a copy stored by its producer; an output of a one-pass
 // chain that no later op overwrites although a later op still folds), more than kChainStreams inputs or
 // outputs, a fold in another dtype or compute op than the graph's kernel, an op of another element size.
+// *pays: every chain folds at least two inputs and walks at least four streams.  Eight independent ops of
+// 1 / 4 / 16 / 32 MiB per stream, table-driven wide launch against this one, us: copies 1 -> 1 7.2 / 15 /
+// 44 / 81 against 7.8 / 17 / 53 / 103 and folds 2 -> 1 7.5 / 19 / 62 / 118 against 7.9 / 19 / 66 / 124, but
+// 2 -> 2 8 / 23 / 80 / 183 against 8.5 / 23 / 83 / 167, 4 -> 1 9 / 30 / 106 / 209 against 9.8 / 26 / 101 / 192,
+// 8 -> 1 15 / 56 / 222 / 440 against 14 / 53 / 189 / 368, 4 -> 4 15 / 47 / 205 / 401 against 14 / 45 / 178 / 340;
+// fan-out copies 1 -> 8 lose a fifth around 256 MiB in all (all-gather and broadcast over 8 ranks x 32 MiB:
+// 44 -> 54, 45 -> 53 us) although they gain beyond 1 GiB, so copies stay with the table.
 // Which outputs survive depends on the operands' addresses, whether the graph fits does not, short of a
 // rebind that changes the chains themselves.  The caller has made sure that no queued op waits for anything.
 bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<int> &words, int dtype, int compute,
-                      std::vector<LaunchChain> *rows) {
+                      std::vector<LaunchChain> *rows, bool *pays) {
+  *pays = true;
   const int n = (int)ops.size();
   std::vector<char> member(n, 0);
   for (int i = 0; i < n; ++i) {
@@ -823,7 +832,7 @@ bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<in
       for (int j = 0; j < head.n_out; ++j) add_out(head.outs[j]);
     } else if (forward == 1) {
       size_t last_fold = 0;  // the last op that changes the value
-      for (size_t t = 1; t < steps.size(); ++t) {
+      for (size_t t = 1; t < steps.size() && ok; ++t) {
         const pccl_op_desc &o = ops[steps[t]];
         if (o.n_in == 2) {
           const int fed = words[(size_t)kChainWords * steps[t] + kChainForward];
@@ -851,6 +860,7 @@ bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<in
       ok = false;
     }
     if (!ok || c.n_out < 1) return false;
+    *pays = *pays && c.n_in >= 2 && c.n_in + c.n_out >= 4;
     rows->push_back(c);
   }
   return !rows->empty();
@@ -1340,18 +1350,23 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // this traffic (reduce_copy.hip): streaming treatment and chunk rotation from 48 MiB in all, an
   // occupancy cap beyond the Infinity Cache.
   std::vector<LaunchChain> launch_rows;
+  bool launch_pays = false;
   G->chains_launch = false;
-  if (G->want_wide && !mixed && (G->fixed_chains ? G->fixed_chains->chains_launch : chain_launch_on()) &&
-      launch_chains_of(G->eff, G->chain_words, g_dtype, g_compute, &launch_rows)) {
+  if (G->want_wide && !mixed && (G->fixed_chains ? G->fixed_chains->chains_launch : chain_launch_mode() != 0) &&
+      launch_chains_of(G->eff, G->chain_words, g_dtype, g_compute, &launch_rows, &launch_pays) &&
+      (launch_pays || G->fixed_chains || chain_launch_mode() == 2)) {
     ChainsLaunch &a = G->chains_args;
     memset(&a, 0, sizeof(a));
     long long blocks = 0, total_bytes = 0;
     int streams = 1;
     bool folds = false;
-    for (size_t k = 0; k < (size_t)kMaxLaunchChains; ++k) {
-      a.first_wg[k] = k < launch_rows.size() ? (unsigned int)blocks : 0xffffffffu;
-      if (k >= launch_rows.size()) continue;
-      const LaunchChain &c = launch_rows[k];
+    a.n_chains = (int)launch_rows.size();
+    a.group = (a.n_chains + kLaunchChainGroups - 1) / kLaunchChainGroups;
+    for (int k = 0; k < kLaunchChainGroups; ++k) a.first_wg[k] = 0xffffffffu;
+    for (size_t k = 0; k < launch_rows.size(); ++k) {
+      LaunchChain &c = launch_rows[k];
+      c.first_wg = (unsigned int)blocks;
+      if (k % (size_t)a.group == 0) a.first_wg[k / (size_t)a.group] = c.first_wg;
       blocks += c.n_wg;
       total_bytes += (long long)(c.n_in + c.n_out) * c.count * elem_bytes(g_dtype);
       streams = std::max(streams, c.n_in + c.n_out);
@@ -1377,7 +1392,8 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
     // (launches that a stream capture has recorded carry the kernel, the grid and the arguments)
     const bool same = F->chains_launch == G->chains_launch &&
                       (!F->chains_launch || (F->chains_grid == G->chains_grid && F->chains_lds == G->chains_lds && F->chains_kernel == G->chains_kernel &&
-                                             F->chains_args.rotate == G->chains_args.rotate &&
+                                             F->chains_args.rotate == G->chains_args.rotate && F->chains_args.group == G->chains_args.group &&
+                                             F->chains_args.n_chains == G->chains_args.n_chains &&
                                              !memcmp(F->chains_args.first_wg, G->chains_args.first_wg, sizeof(F->chains_args.first_wg))));
     if (!same)
       return fail(PCCL_ERR_UNSUPPORTED, "with these operands the graph does not run as the launch it was made for (its chains come out differently)");
@@ -1942,6 +1958,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
   const std::vector<pccl_op_desc> eff_next = effective_of(G, next);
   std::vector<LaunchChain> rows_next;
+  bool pays_next = false;
   const std::vector<unsigned char> edges_after = classify_dependencies(eff_next, G->parts, G->topo, &G->part_eligible);
   if (edges_after != G->part_edge || plan_chains_of(G, eff_next, G->parts, edges_after, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
@@ -2013,7 +2030,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
-  if (G->chains_launch && !launch_chains_of(eff_next, G->chain_words, G->chains_dtype, G->chains_compute, &rows_next))
+  if (G->chains_launch && (!launch_chains_of(eff_next, G->chain_words, G->chains_dtype, G->chains_compute, &rows_next, &pays_next) ||
+                           (int)rows_next.size() != G->chains_args.n_chains))
     return fail(PCCL_ERR_UNSUPPORTED, "graph_rebind: with these operands the graph no longer runs as the launch it was made for; create it again");
   G->descs.swap(next);
   for (size_t i = 0; i < G->eff.size(); ++i) {  // (the same ops: the dependency lists stay, the operands move)
@@ -2034,6 +2052,8 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
                                 G->fuse_table_off + sizeof(SignalFuse) * (size_t)G->n_ops - G->payload_off,
                                 hipMemcpyHostToDevice, (hipStream_t)stream));
   if (G->chains_launch) {
+    const LaunchChain *before = (const LaunchChain *)(G->image.data() + G->chains_off);
+    for (size_t k = 0; k < rows_next.size(); ++k) rows_next[k].first_wg = before[k].first_wg;  // (the same ops of the same lengths)
     memcpy(G->image.data() + G->chains_off, rows_next.data(), sizeof(LaunchChain) * rows_next.size());
     PCCL_HIP_CHECK(hipMemcpyAsync(G->dev + G->chains_off, G->image.data() + G->chains_off, sizeof(LaunchChain) * rows_next.size(),
                                   hipMemcpyHostToDevice, (hipStream_t)stream));

@@ -77,7 +77,7 @@ def test_ring_chains_in_one_pass(hip, oracle, monkeypatch, dtype, compute):
         for chain_launch in ("1", "0"):
             monkeypatch.setenv("PCCL_HIP_CHAIN_LAUNCH", chain_launch)
             g = hip.Graph(bound, tile_bytes=tile)
-            if chain_launch == "1" and tile == 0 and len(sizes) <= 2:
+            if chain_launch == "1" and tile == 0:
                 assert g.launch_kind() == "chains", (sizes, offsets)
             if g.launch_kind() != "chains":
                 # 14 ops share the entries of one (the built-in choice may also cut a chain into fewer parts)
@@ -461,9 +461,11 @@ def test_later_op_writes_over_an_earlier_output_at_a_shift(hip, oracle):
 @pytest.mark.parametrize("dtype,compute", [("bf16", "sum"), ("f32", "prod"), ("f64", "min"), ("f8e4m3", "max"), ("i32", "sum")])
 def test_folds_and_their_broadcast_copies_as_one_launch_of_chains(hip, oracle, monkeypatch, dtype, compute):
     """A direct all-reduce over 8 ranks (rank r folds slice r of all inputs, a copy broadcasts the result:
-    16 ops, 8 queue entries) plus independent ops of 1..8 inputs and several outputs, at most 16 entries in
-    all, none of which waits for anything: the graph runs as one launch of chains, a workgroup per 4 KiB,
-    whatever the operands' alignment.  Bits as through the persistent drain and as the CPU checker's."""
+    16 ops, 8 queue entries), none of whose entries waits for anything: the graph runs as one launch of
+    chains, a workgroup per 4 KiB, whatever the operands' alignment.  With independent ops of 1..8 inputs and
+    several outputs beside it (copies and thin folds, for which that launch is not the library's choice:
+    PCCL_HIP_CHAIN_LAUNCH=2 takes it wherever the graph fits): bits as from the table-driven wide launch,
+    through the persistent drain, and as the CPU checker's."""
     import torch
     es = H.ELEM_BYTES[dtype]
     kw = dict(mean=1.0, sigma=0.05) if compute == "prod" else dict(sigma=1.0)
@@ -482,6 +484,9 @@ def test_folds_and_their_broadcast_copies_as_one_launch_of_chains(hip, oracle, m
             folded = oracle.reduce(dtype, compute, [x[lo:lo + slice_elems] for x in host_in])
             for d in range(8):
                 want[d][lo:lo + slice_elems] = folded
+        g = hip.Graph(ops)
+        assert g.launch_kind() == "chains", (g.launch_kind(), slice_elems)  # (the library's own choice for these folds)
+        g.destroy()
         extra = []
         for k, (n_in, n_out, count) in enumerate(((1, 3, 5000), (3, 2, 999), (8, 1, 12345), (2, 8, 1), (5, 1, 4096 // es), (1, 1, 70001))):
             srcs = [H.gen(dtype, count, 1300 + k, j, **kw) for j in range(n_in)]
@@ -489,7 +494,7 @@ def test_folds_and_their_broadcast_copies_as_one_launch_of_chains(hip, oracle, m
             do = [H.DevBuf(torch, dtype, count, ((k + 2 * j) % 7) * es) for j in range(n_out)]
             ops.append(dict(dtype=dtype, compute=compute, ins=[d.ptr for d in ds], outs=[d.ptr for d in do], count=count, deps=[]))
             extra.append((do, oracle.reduce(dtype, compute, srcs) if n_in > 1 else srcs[0], ds))
-        for form, env in (("chains", {}), ("wide", {"PCCL_HIP_CHAIN_LAUNCH": "0"}), ("drain", {"PCCL_HIP_WIDE": "0"})):
+        for form, env in (("chains", {"PCCL_HIP_CHAIN_LAUNCH": "2"}), ("wide", {}), ("wide", {"PCCL_HIP_CHAIN_LAUNCH": "0"}), ("drain", {"PCCL_HIP_WIDE": "0"})):
             for k, v in env.items():
                 monkeypatch.setenv(k, v)
             g = hip.Graph(ops)
@@ -567,3 +572,41 @@ def test_launch_of_chains_follows_rebinds_also_when_recorded(hip, oracle):
             check(target, "replay after a rebind")
     assert g.status(stream.cuda_stream) == (len(ops), len(ops))
     g.destroy()
+
+
+@pytest.mark.parametrize("collective", ["ring_reduce_scatter", "ring_all_gather", "all_to_all", "broadcast"])
+def test_other_collectives_over_resident_ranks_in_every_form(hip, oracle, monkeypatch, collective):
+    """The other collectives of the schedule language over 8 ranks that live on this device.  All-gather (chains
+    of copies), all-to-all (64 independent copies) and broadcast (one copy to seven outputs) fit the launch of
+    chains but are better off as the table-driven wide launch, which is the library's choice;
+    PCCL_HIP_CHAIN_LAUNCH=2 takes the launch of chains for them.  A ring reduce-scatter's chains leave their
+    partial sums in memory, which that launch cannot do: wide either way.  Same bits in every form."""
+    import torch
+    from pccl_amd import lang
+    dtype, es, chunk = "bf16", 2, 2501
+    emit = getattr(lang, collective)
+    ir, per_rank = emit(8, chunk, dtype=dtype) if collective != "broadcast" else emit(8, 8 * chunk, dtype=dtype)
+    low = ir.lower()
+    host = {"in": [H.gen(dtype, per_rank, 1500, r) for r in range(8)], "out": [np.zeros(per_rank, dtype=H.STORAGE[dtype]) for _ in range(8)]}
+    dev = {"in": [H.DevBuf(torch, dtype, per_rank, 2 * (r % 3), src=host["in"][r]) for r in range(8)],
+           "out": [H.DevBuf(torch, dtype, per_rank, 2 * (r % 5)) for r in range(8)]}
+    h_ops = lang.bind(low, lambda b, r, e: host[b][r][e:])
+    for o in h_ops:  # (the CPU checker takes arrays of the op's length)
+        o["ins"], o["outs"] = [x[:o["count"]] for x in o["ins"]], [x[:o["count"]] for x in o["outs"]]
+    oracle.run_ops(h_ops, oracle.topo_sort(len(h_ops), [(d, i) for i, o in enumerate(h_ops) for d in o.get("deps", [])]))
+    forced = "wide" if collective == "ring_reduce_scatter" else "chains"
+    for want, env in ((forced, {"PCCL_HIP_CHAIN_LAUNCH": "2"}), ("wide", {}), ("drain", {"PCCL_HIP_WIDE": "0"})):
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        g = hip.Graph(lang.bind(low, lambda b, r, e: dev[b][r].ptr + e * es))
+        for k in env:
+            monkeypatch.delenv(k)
+        assert g.launch_kind() == want, (want, g.launch_kind())
+        for it in range(2):
+            for b in dev["out"]:
+                b.upload(np.zeros(per_rank, dtype=H.STORAGE[dtype]))
+            _run(torch, hip, g, len(low))
+            for r in range(8):
+                H.assert_bits_equal(dev["out"][r].download(), host["out"][r], "%s as %s run %d rank %d" % (collective, want, it, r))
+                assert dev["out"][r].guards_intact()
+        g.destroy()
