@@ -391,15 +391,21 @@ def timeline_main():
         t = event_times_us(torch, lambda: g.run(stream), 20, 3)
         out[kind] = dict(queue_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
         g.destroy()
-        del os.environ["PCCL_HIP_WIDE"]  # ... and the same graph as the wide launch it runs as by default
-        try:
-            g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
-        finally:
-            os.environ["PCCL_HIP_WIDE"] = "0"
-        if g.launch_kind() in ("wide", "chains"):
-            t = event_times_us(torch, lambda: g.run(stream), 20, 3)
-            out[kind]["as_the_wide_launch"] = dict(wide_timeline(torch, hip, g, stream), untraced_events_median_us=round(t[len(t) // 2], 1))
-        g.destroy()
+        # ... and the same graph as the wide launch it runs as by default (a launch of chains), and as the
+        # table-driven wide launch that it would be without that
+        for key, env in (("as_the_launch_it_runs_as", {}), ("as_the_table_driven_wide_launch", {"PCCL_HIP_CHAIN_LAUNCH": "0"})):
+            del os.environ["PCCL_HIP_WIDE"]
+            os.environ.update(env)
+            try:
+                g = hip.Graph(lang.bind(ir.lower(), lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+            finally:
+                os.environ["PCCL_HIP_WIDE"] = "0"
+                for k in env:
+                    del os.environ[k]
+            if g.launch_kind() in ("wide", "chains"):
+                t = event_times_us(torch, lambda: g.run(stream), 20, 3)
+                out[kind][key] = dict(wide_timeline(torch, hip, g, stream), launch=launch_kind(g), untraced_events_median_us=round(t[len(t) // 2], 1))
+            g.destroy()
     print(json.dumps({"queue_timeline": out}))
 
 
