@@ -803,11 +803,37 @@ def main():
                         full["8_ranks_x_%d_MiB" % per_rank_mib]["linked_by_signal_words_only"]["a_word_per_part"] = dict(
                             stats(tp), words_per_signal=K, ops=len(lowp), queue_entries=gp.info()["n_tiles"])
                         gp.destroy()
+                        # What bounds these two: the schedule, not the signal words.  The same 112 data ops linked by
+                        # DEPENDENCIES in the order the signalled form implies (an op behind its neighbour's op of the
+                        # step before, part by part, and behind its own rank's op of the step before, as a whole),
+                        # every op queueing its own entries; and without the in-rank order.
+                        ordered = [dict(o) for o in low]
+                        latest = {}
+                        for i, o in enumerate(ordered):
+                            rank = o["outs"][0][1]
+                            if rank in latest and latest[rank] not in o["deps"]:
+                                o["deps"] = list(o["deps"]) + [latest[rank]]
+                            latest[rank] = i
+                        by_deps = {}
+                        os.environ["PCCL_HIP_CHAINS"] = "0"
+                        try:
+                            for key, ops_k in (("the_same_order_as_dependencies", ordered), ("neighbour_dependencies_only", low)):
+                                for r in range(8):
+                                    rb["out"][r].zero_()
+                                gd = hip.Graph(lang.bind(ops_k, lambda b, r, e: rb[b][r].data_ptr() + 2 * e))
+                                td = event_times_us(torch, lambda: gd.run(stream), 20, 3)
+                                for r in range(8):
+                                    assert torch.equal(rb["out"][r], first)
+                                by_deps[key] = dict(stats(td), queue_entries=gd.info()["n_tiles"])
+                                gd.destroy()
+                        finally:
+                            del os.environ["PCCL_HIP_CHAINS"]
+                        full["8_ranks_x_%d_MiB" % per_rank_mib]["linked_by_signal_words_only"]["without_chains"] = by_deps
                     del rb
                 full["note"] = ("GBps_median counts the algorithmic bytes of the 112 ops; the 14 ops of a chunk run as one chain that keeps "
                                 "the value in registers and stores only what the chain does not overwrite itself: bytes_moved / GBps_moved_median.  "
-                                "No entry of these graphs waits for another, so they run as a wide launch (one short-lived workgroup per 16 KiB "
-                                "block of a chain); through_the_persistent_drain is the same graph with PCCL_HIP_WIDE=0")
+                                "No entry of these graphs waits for another, so they run as a wide launch (a launch of chains: one short-lived "
+                                "workgroup per 4 KiB of a chain); through_the_persistent_drain is the same graph with PCCL_HIP_WIDE=0")
                 extras["ring_allreduce_one_launch"] = full
 
                 # the same all-reduce as the one-exchange ("direct") schedule a fully connected node
