@@ -328,7 +328,7 @@ KNOBS = [("PCCL_HIP_PLAN_LAUNCHES", "0"), ("PCCL_HIP_ORDER_EDGES", "0"), ("PCCL_
          ("PCCL_HIP_CHAIN_BALANCE", "0"), ("PCCL_HIP_PART_DEPS", "0"), ("PCCL_HIP_FUSE_SIGNALS", "0"),
          ("PCCL_HIP_OWN_ENTRIES", "0"), ("PCCL_HIP_OWN_ENTRIES", "16"), ("PCCL_HIP_ORDER_BLOCK", "0"), ("PCCL_HIP_ORDER_BLOCK", "1"), ("PCCL_HIP_FOLD_COPIES", "0"),
          ("PCCL_HIP_LAST_LEVEL", "0"), ("PCCL_HIP_COUNT_ALL", "1"),
-         ("PCCL_HIP_WIDE", "0"), ("PCCL_HIP_CHAIN_LAUNCH", "0")]
+         ("PCCL_HIP_WIDE", "0"), ("PCCL_HIP_CHAIN_LAUNCH", "0"), ("PCCL_HIP_CHAIN_LAUNCH", "2")]
 
 
 @pytest.mark.parametrize("name,value", KNOBS, ids=["%s=%s" % kv for kv in KNOBS])
