@@ -74,7 +74,8 @@ __device__ __forceinline__ typename D::elem_t fold_head_elem(const typename D::e
   return D::template elem<Op, N>(w);
 }
 
-// MEM: kLaunchMemCached or kLaunchMemStreamWriteThrough (reduce_copy_kernel.h)
+// MEM (reduce_copy_kernel.h): kLaunchMemCached; kLaunchMemStreamWriteThrough (non-temporal loads, write-through
+// stores); kLaunchMemStream for launches of fan-out copies (cached loads, non-temporal stores)
 template <int DT, class Op, int MEM>
 __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch a) {
   typedef Dtype<DT> D;
@@ -84,8 +85,8 @@ __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch
   // (through the buffer instructions: the operands' addresses come out of memory, not out of the
   // kernel's pointer arguments, and a plain access through such an address would be a flat one; they
   // also take the operands that are only element-aligned)
-  constexpr int kLdPolicy = MEM == pccl_dev::kLaunchMemCached ? 0 : 2;             // nt
-  constexpr int kStPolicy = MEM == pccl_dev::kLaunchMemCached ? 0 : kCachePolicySc1;
+  constexpr int kLdPolicy = MEM == pccl_dev::kLaunchMemStreamWriteThrough ? 2 : 0;  // nt
+  constexpr int kStPolicy = MEM == pccl_dev::kLaunchMemCached ? 0 : MEM == pccl_dev::kLaunchMemStream ? 2 : kCachePolicySc1;
   const unsigned int b = blockIdx.x;
   int ci = 0;
 #pragma unroll
@@ -189,21 +190,24 @@ __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch
 }
 
 typedef void (*ChainsKernel)(const ChainsLaunch);
-// The instances of one dtype; defined in graph_chains_inst_<dtype>.hip.  mem: 0 cached, otherwise
-// non-temporal loads and write-through stores.
+// The instances of one dtype; defined in graph_chains_inst_<dtype>.hip.  mem: a kLaunchMem* value.
 template <int DT>
 ChainsKernel chains_for_compute(int compute, int mem);
 
-#define PCCL_DEFINE_CHAINS_FOR_COMPUTE(DT)                                                                                  \
-  template <>                                                                                                               \
-  ChainsKernel chains_for_compute<DT>(int compute, int mem) {                                                               \
-    constexpr int kC = pccl_dev::kLaunchMemCached, kW = pccl_dev::kLaunchMemStreamWriteThrough;                             \
-    switch (compute) {                                                                                                      \
-      case PCCL_SUM: return mem ? graph_chains_kernel<DT, OpSum, kW> : graph_chains_kernel<DT, OpSum, kC>;                  \
-      case PCCL_PROD: return mem ? graph_chains_kernel<DT, OpProd, kW> : graph_chains_kernel<DT, OpProd, kC>;               \
-      case PCCL_MIN: return mem ? graph_chains_kernel<DT, OpMin, kW> : graph_chains_kernel<DT, OpMin, kC>;                  \
-      default: return mem ? graph_chains_kernel<DT, OpMax, kW> : graph_chains_kernel<DT, OpMax, kC>;                        \
-    }                                                                                                                       \
+#define PCCL_CHAINS_KERNEL_OF(DT, OP)                                                             \
+  (mem == pccl_dev::kLaunchMemStreamWriteThrough ? graph_chains_kernel<DT, OP, pccl_dev::kLaunchMemStreamWriteThrough> \
+   : mem == pccl_dev::kLaunchMemStream           ? graph_chains_kernel<DT, OP, pccl_dev::kLaunchMemStream>             \
+                                                 : graph_chains_kernel<DT, OP, pccl_dev::kLaunchMemCached>)
+
+#define PCCL_DEFINE_CHAINS_FOR_COMPUTE(DT)                    \
+  template <>                                                 \
+  ChainsKernel chains_for_compute<DT>(int compute, int mem) { \
+    switch (compute) {                                        \
+      case PCCL_SUM: return PCCL_CHAINS_KERNEL_OF(DT, OpSum); \
+      case PCCL_PROD: return PCCL_CHAINS_KERNEL_OF(DT, OpProd); \
+      case PCCL_MIN: return PCCL_CHAINS_KERNEL_OF(DT, OpMin); \
+      default: return PCCL_CHAINS_KERNEL_OF(DT, OpMax);       \
+    }                                                         \
   }
 
 }  // namespace pccl_queue

@@ -777,18 +777,23 @@ int chain_launch_mode() {
 // final value (a chain through memory other than a copy stored by its producer; an output of a one-pass
 // chain that no later op overwrites although a later op still folds), more than kChainStreams inputs or
 // outputs, a fold in another dtype or compute op than the graph's kernel, an op of another element size.
-// *pays: every chain folds at least two inputs and walks at least four streams.  Eight independent ops of
+// *shape: kChainsFold if every chain folds at least two inputs and walks at least four streams, kChainsFanOut if
+// every chain is a copy to at least three outputs, else 0: where the launch is the better choice (fan-out
+// copies from 48 MiB in all, with the non-temporal stores a direct launch gives them).  Eight independent ops of
 // 1 / 4 / 16 / 32 MiB per stream, table-driven wide launch against this one, us: copies 1 -> 1 7.2 / 15 /
 // 44 / 81 against 7.8 / 17 / 53 / 103 and folds 2 -> 1 7.5 / 19 / 62 / 118 against 7.9 / 19 / 66 / 124, but
 // 2 -> 2 8 / 23 / 80 / 183 against 8.5 / 23 / 83 / 167, 4 -> 1 9 / 30 / 106 / 209 against 9.8 / 26 / 101 / 192,
 // 8 -> 1 15 / 56 / 222 / 440 against 14 / 53 / 189 / 368, 4 -> 4 15 / 47 / 205 / 401 against 14 / 45 / 178 / 340;
-// fan-out copies 1 -> 8 lose a fifth around 256 MiB in all (all-gather and broadcast over 8 ranks x 32 MiB:
-// 44 -> 54, 45 -> 53 us) although they gain beyond 1 GiB, so copies stay with the table.
+// fan-out copies with write-through stores lose a fifth around 256 MiB in all (1 -> 8 x 4 MiB 45 -> 55), with
+// non-temporal stores 1 -> 3 8.4 / 26 / 101 / 206 against 9.3 / 23 / 77 / 149, 1 -> 4 9.6 / 30 / 132 / 267 against
+// 10.5 / 28 / 95 / 188, 1 -> 8 14 / 45 / 240 / 510 against 14 / 45 / 166 / 355 (all-gather and broadcast over 8
+// ranks x 8 / 32 / 128 MiB: 14 / 44 / 235 against 14 / 44 / 167 us).
 // Which outputs survive depends on the operands' addresses, whether the graph fits does not, short of a
 // rebind that changes the chains themselves.  The caller has made sure that no queued op waits for anything.
+constexpr int kChainsFold = 1, kChainsFanOut = 2;
 bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<int> &words, int dtype, int compute,
-                      std::vector<LaunchChain> *rows, bool *pays) {
-  *pays = true;
+                      std::vector<LaunchChain> *rows, int *shape) {
+  *shape = kChainsFold | kChainsFanOut;
   const int n = (int)ops.size();
   std::vector<char> member(n, 0);
   for (int i = 0; i < n; ++i) {
@@ -860,7 +865,8 @@ bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<in
       ok = false;
     }
     if (!ok || c.n_out < 1) return false;
-    *pays = *pays && c.n_in >= 2 && c.n_in + c.n_out >= 4;
+    if (!(c.n_in >= 2 && c.n_in + c.n_out >= 4)) *shape &= ~kChainsFold;
+    if (!(c.n_in == 1 && c.n_out >= 3)) *shape &= ~kChainsFanOut;
     rows->push_back(c);
   }
   return !rows->empty();
@@ -1350,11 +1356,10 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
   // this traffic (reduce_copy.hip): streaming treatment and chunk rotation from 48 MiB in all, an
   // occupancy cap beyond the Infinity Cache.
   std::vector<LaunchChain> launch_rows;
-  bool launch_pays = false;
+  int launch_shape = 0;
   G->chains_launch = false;
   if (G->want_wide && !mixed && (G->fixed_chains ? G->fixed_chains->chains_launch : chain_launch_mode() != 0) &&
-      launch_chains_of(G->eff, G->chain_words, g_dtype, g_compute, &launch_rows, &launch_pays) &&
-      (launch_pays || G->fixed_chains || chain_launch_mode() == 2)) {
+      launch_chains_of(G->eff, G->chain_words, g_dtype, g_compute, &launch_rows, &launch_shape)) {
     ChainsLaunch &a = G->chains_args;
     memset(&a, 0, sizeof(a));
     long long blocks = 0, total_bytes = 0;
@@ -1372,11 +1377,13 @@ int build_graph(Graph *G, unsigned int run_number, char *reuse = nullptr, size_t
       streams = std::max(streams, c.n_in + c.n_out);
       folds = folds || c.n_in > 1;
     }
-    if (blocks < (1ll << 31)) {
+    const bool pays = (launch_shape & kChainsFold) || ((launch_shape & kChainsFanOut) && total_bytes >= (48ll << 20));
+    if (blocks < (1ll << 31) && (pays || G->fixed_chains || chain_launch_mode() == 2)) {
       G->chains_launch = true;
       G->chains_grid = (unsigned)blocks;
-      G->chains_mem = total_bytes >= (48ll << 20) ? 1 : 0;
-      a.rotate = G->chains_mem;
+      G->chains_mem = total_bytes >= (48ll << 20) ? (int)kLaunchMemStreamWriteThrough : (int)kLaunchMemCached;
+      if (G->chains_mem && (launch_shape & kChainsFanOut)) G->chains_mem = kLaunchMemStream;  // (as a direct launch treats a copy to three or more outputs)
+      a.rotate = G->chains_mem != 0;
       G->chains_lds = 0;
       if (total_bytes > (192ll << 20)) {
         int wgs = std::max(2, std::min(8, (20 + streams / 2) / streams));
@@ -1958,7 +1965,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
   // ... and so does which ops run as chains behind each other, and how (plan_chains).
   const std::vector<pccl_op_desc> eff_next = effective_of(G, next);
   std::vector<LaunchChain> rows_next;
-  bool pays_next = false;
+  int shape_next = 0;
   const std::vector<unsigned char> edges_after = classify_dependencies(eff_next, G->parts, G->topo, &G->part_eligible);
   if (edges_after != G->part_edge || plan_chains_of(G, eff_next, G->parts, edges_after, G->forward_capable ? G->kernel_elem_bytes : 0) != G->chain_words) {
     PCCL_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
@@ -2030,7 +2037,7 @@ int pccl_hip_graph_rebind(void *graph, const void *old_base, const void *new_bas
     if (old_dev != G->dev) PCCL_HIP_CHECK(hipFree(old_dev));
     return PCCL_OK;
   }
-  if (G->chains_launch && (!launch_chains_of(eff_next, G->chain_words, G->chains_dtype, G->chains_compute, &rows_next, &pays_next) ||
+  if (G->chains_launch && (!launch_chains_of(eff_next, G->chain_words, G->chains_dtype, G->chains_compute, &rows_next, &shape_next) ||
                            (int)rows_next.size() != G->chains_args.n_chains))
     return fail(PCCL_ERR_UNSUPPORTED, "graph_rebind: with these operands the graph no longer runs as the launch it was made for; create it again");
   G->descs.swap(next);

@@ -610,3 +610,28 @@ def test_other_collectives_over_resident_ranks_in_every_form(hip, oracle, monkey
                 H.assert_bits_equal(dev["out"][r].download(), host["out"][r], "%s as %s run %d rank %d" % (collective, want, it, r))
                 assert dev["out"][r].guards_intact()
         g.destroy()
+
+
+def test_large_fan_out_copies_run_as_a_launch_of_chains(hip, oracle):
+    """An all-gather over 8 resident ranks whose chains of copies move 72 MiB in all: from 48 MiB such a graph
+    runs as a launch of chains with non-temporal stores (what a direct launch gives a copy to many outputs).
+    Every rank's output is the concatenation of the ranks' chunks."""
+    import torch
+    from pccl_amd import lang
+    chunk = (1 << 19) + 24  # elements per chunk: 1 MiB and a few packs
+    ir, per_rank = lang.ring_all_gather(8, chunk, dtype="bf16")
+    low = ir.lower()
+    src = [H.gen("bf16", per_rank, 1600, r) for r in range(8)]
+    dev = {"in": [H.DevBuf(torch, "bf16", per_rank, 0, src=src[r]) for r in range(8)],
+           "out": [H.DevBuf(torch, "bf16", per_rank, 16 * (r % 2)) for r in range(8)]}
+    g = hip.Graph(lang.bind(low, lambda b, r, e: dev[b][r].ptr + 2 * e))
+    assert g.launch_kind() == "chains", g.launch_kind()
+    want = np.concatenate([src[r][r * chunk:(r + 1) * chunk] for r in range(8)])
+    for it in range(2):
+        for b in dev["out"]:
+            b.view().fill_(0xFF)
+        _run(torch, hip, g, len(low))
+        for r in range(8):
+            H.assert_bits_equal(dev["out"][r].download(), want, "all-gather run %d rank %d" % (it, r))
+            assert dev["out"][r].guards_intact()
+    g.destroy()
