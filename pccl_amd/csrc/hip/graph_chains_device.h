@@ -58,20 +58,63 @@ struct ChainsLaunch {
   int n_chains;
 };
 
-template <class D, class Op, int N>
-__device__ __forceinline__ u32x4 fold_head(const u32x4 *v) {
-  u32x4 w[N];
+// One workgroup's 4 KiB of a chain of NIN inputs (a count the compiler knows: a register array that is
+// written under run-time conditions costs the floating-point instances 244 registers and a wait behind
+// every load).  n_head is NIN (one op: all inputs folded as one reduction) or, for a one-pass chain, the
+// head op's 1 or 2, the other inputs then being folded in one after the other.
+template <class D, class Op, int NIN, int LD, int ST>
+__device__ __forceinline__ void chain_packs(const unsigned long long (&in)[kChainStreams], const unsigned long long (&out)[kChainStreams],
+                                            int n_head, int n_out, unsigned int fed, size_t wg_off, unsigned int lane_off) {
+  u32x4 v[NIN];
 #pragma unroll
-  for (int k = 0; k < N; ++k) w[k] = v[k];
-  return fold_pack<D, Op, N>(w);
+  for (int i = 0; i < NIN; ++i) v[i] = __builtin_amdgcn_raw_buffer_load_b128(whole_buffer((const char *)in[i] + wg_off), (int)lane_off, 0, LD);
+  u32x4 cur;
+  if (n_head == NIN) {
+    cur = fold_pack<D, Op, NIN>(v);
+  } else {
+    cur = v[0];
+    if constexpr (NIN >= 2) {
+      if (n_head == 2) cur = fold_two<D, Op>(v[0], v[1]);
+#pragma unroll
+      for (int i = 1; i < NIN; ++i)
+        if (i >= n_head) cur = ((fed >> i) & 1u) ? fold_two<D, Op>(v[i], cur) : fold_two<D, Op>(cur, v[i]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kChainStreams; ++j)
+    if (j < n_out) __builtin_amdgcn_raw_buffer_store_b128(cur, whole_buffer((char *)out[j] + wg_off), (int)lane_off, 0, ST);
 }
 
-template <class D, class Op, int N>
-__device__ __forceinline__ typename D::elem_t fold_head_elem(const typename D::elem_t *v) {
-  typename D::elem_t w[N];
+// ... and one of the few elements in front of the first and behind the last pack
+template <class D, class Op, int NIN>
+__device__ __forceinline__ void chain_elem(const unsigned long long (&in)[kChainStreams], const unsigned long long (&out)[kChainStreams],
+                                           int n_head, int n_out, unsigned int fed, long long i) {
+  typedef typename D::elem_t E;
+  E x[NIN];
 #pragma unroll
-  for (int k = 0; k < N; ++k) w[k] = v[k];
-  return D::template elem<Op, N>(w);
+  for (int s = 0; s < NIN; ++s) x[s] = ((const E *)in[s])[i];
+  E cur;
+  if (n_head == NIN) {
+    if constexpr (NIN == 1) cur = x[0];
+    else cur = D::template elem<Op, NIN>(x);
+  } else {
+    cur = x[0];
+    if constexpr (NIN >= 2) {
+      if (n_head == 2) {
+        const E two[2] = {x[0], x[1]};
+        cur = D::template elem<Op, 2>(two);
+      }
+#pragma unroll
+      for (int s = 1; s < NIN; ++s)
+        if (s >= n_head) {
+          const E two[2] = {((fed >> s) & 1u) ? x[s] : cur, ((fed >> s) & 1u) ? cur : x[s]};
+          cur = D::template elem<Op, 2>(two);
+        }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kChainStreams; ++j)
+    if (j < n_out) ((E *)out[j])[i] = cur;
 }
 
 // MEM (reduce_copy_kernel.h): kLaunchMemCached; kLaunchMemStreamWriteThrough (non-temporal loads, write-through
@@ -79,7 +122,6 @@ __device__ __forceinline__ typename D::elem_t fold_head_elem(const typename D::e
 template <int DT, class Op, int MEM>
 __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch a) {
   typedef Dtype<DT> D;
-  typedef typename D::elem_t E;
   constexpr int kEpp = 16 / D::kElemBytes;
   D::wave_init();
   // (through the buffer instructions: the operands' addresses come out of memory, not out of the
@@ -127,60 +169,38 @@ __global__ void __launch_bounds__(kBlock) graph_chains_kernel(const ChainsLaunch
   long long peel = (long long)((16 - (out[0] & 15)) & 15) / D::kElemBytes;
   if (peel > count) peel = count;
   const long long n_packs = (count - peel) / kEpp;
-  const size_t wg_off = (size_t)peel * D::kElemBytes + (size_t)chunk * (kBlock * 16);
+  // (read back into scalar registers: the compiler works this sum out on the vector unit, beside the lane's
+  // pack number, and every operand's address would follow it there: a vector register pair per address that
+  // each store then waits for the one before it to release)
+  const size_t wg_off = (size_t)uniform64((unsigned long long)peel * D::kElemBytes + (unsigned long long)chunk * (kBlock * 16));
   const unsigned int lane_off = threadIdx.x * 16u;
   if ((long long)chunk * kBlock + threadIdx.x < n_packs) {
-    u32x4 v[kChainStreams];
-#pragma unroll
-    for (int i = 0; i < kChainStreams; ++i)
-      if (i < n_in) v[i] = __builtin_amdgcn_raw_buffer_load_b128(whole_buffer((const char *)in[i] + wg_off), (int)lane_off, 0, kLdPolicy);
-    u32x4 cur;
-    switch (n_head) {
-      case 1: cur = v[0]; break;
-      case 2: cur = fold_head<D, Op, 2>(v); break;
-      case 3: cur = fold_head<D, Op, 3>(v); break;
-      case 4: cur = fold_head<D, Op, 4>(v); break;
-      case 5: cur = fold_head<D, Op, 5>(v); break;
-      case 6: cur = fold_head<D, Op, 6>(v); break;
-      case 7: cur = fold_head<D, Op, 7>(v); break;
-      default: cur = fold_head<D, Op, 8>(v); break;
+    switch (n_in) {
+      case 1: chain_packs<D, Op, 1, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 2: chain_packs<D, Op, 2, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 3: chain_packs<D, Op, 3, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 4: chain_packs<D, Op, 4, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 5: chain_packs<D, Op, 5, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 6: chain_packs<D, Op, 6, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      case 7: chain_packs<D, Op, 7, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
+      default: chain_packs<D, Op, 8, kLdPolicy, kStPolicy>(in, out, n_head, n_out, fed, wg_off, lane_off); break;
     }
-#pragma unroll
-    for (int i = 1; i < kChainStreams; ++i)
-      if (i >= n_head && i < n_in) cur = ((fed >> i) & 1u) ? fold_two<D, Op>(v[i], cur) : fold_two<D, Op>(cur, v[i]);
-#pragma unroll
-    for (int j = 0; j < kChainStreams; ++j)
-      if (j < n_out) __builtin_amdgcn_raw_buffer_store_b128(cur, whole_buffer((char *)out[j] + wg_off), (int)lane_off, 0, kStPolicy);
   }
   if (k == n_chunks - 1 && threadIdx.x >= kBlock - kWave) {  // fewer than two packs' worth of elements: one per lane
     const long long tail_begin = peel + n_packs * kEpp, n_edge = peel + (count - tail_begin);
     const long long e = (long long)threadIdx.x - (kBlock - kWave);
     if (e < n_edge) {
       const long long i = e < peel ? e : tail_begin + (e - peel);
-      E x[kChainStreams];
-#pragma unroll
-      for (int s = 0; s < kChainStreams; ++s)
-        if (s < n_in) x[s] = ((const E *)in[s])[i];
-      E cur;
-      switch (n_head) {
-        case 1: cur = x[0]; break;
-        case 2: cur = fold_head_elem<D, Op, 2>(x); break;
-        case 3: cur = fold_head_elem<D, Op, 3>(x); break;
-        case 4: cur = fold_head_elem<D, Op, 4>(x); break;
-        case 5: cur = fold_head_elem<D, Op, 5>(x); break;
-        case 6: cur = fold_head_elem<D, Op, 6>(x); break;
-        case 7: cur = fold_head_elem<D, Op, 7>(x); break;
-        default: cur = fold_head_elem<D, Op, 8>(x); break;
+      switch (n_in) {
+        case 1: chain_elem<D, Op, 1>(in, out, n_head, n_out, fed, i); break;
+        case 2: chain_elem<D, Op, 2>(in, out, n_head, n_out, fed, i); break;
+        case 3: chain_elem<D, Op, 3>(in, out, n_head, n_out, fed, i); break;
+        case 4: chain_elem<D, Op, 4>(in, out, n_head, n_out, fed, i); break;
+        case 5: chain_elem<D, Op, 5>(in, out, n_head, n_out, fed, i); break;
+        case 6: chain_elem<D, Op, 6>(in, out, n_head, n_out, fed, i); break;
+        case 7: chain_elem<D, Op, 7>(in, out, n_head, n_out, fed, i); break;
+        default: chain_elem<D, Op, 8>(in, out, n_head, n_out, fed, i); break;
       }
-#pragma unroll
-      for (int s = 1; s < kChainStreams; ++s)
-        if (s >= n_head && s < n_in) {
-          const E two[2] = {((fed >> s) & 1u) ? x[s] : cur, ((fed >> s) & 1u) ? cur : x[s]};
-          cur = D::template elem<Op, 2>(two);
-        }
-#pragma unroll
-      for (int j = 0; j < kChainStreams; ++j)
-        if (j < n_out) ((E *)out[j])[i] = cur;
     }
   }
   if (trace) {

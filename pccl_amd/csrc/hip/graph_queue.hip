@@ -836,6 +836,7 @@ bool launch_chains_of(const std::vector<pccl_op_desc> &ops, const std::vector<in
     if (steps.size() == 1) {
       for (int j = 0; j < head.n_out; ++j) add_out(head.outs[j]);
     } else if (forward == 1) {
+      if (head.n_in > 2) ok = false;  // (the kernel folds a chain's head as 1 or 2 inputs: plan_chains hands on nothing else)
       size_t last_fold = 0;  // the last op that changes the value
       for (size_t t = 1; t < steps.size() && ok; ++t) {
         const pccl_op_desc &o = ops[steps[t]];
