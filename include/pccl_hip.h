@@ -228,7 +228,7 @@ typedef struct pccl_op_desc {
  * the shape of a direct launch instead: a workgroup per 4 KiB of every stream of a chain, the chains'
  * operands in a small table of the arena that all workgroups of a chain share (ring all-reduce over 8
  * resident ranks x 1 / 32 / 64 MiB 9.6 / 84.5 / 200 -> 7 / 80-83 / 172 us, direct all-reduce 8 x 32 MiB
- * 88 -> 78-80 us = one 8 -> 8 launch).  graph_info then reports workgroups for n_tiles, graph_trace records
+ * 88 -> 79-81 us, within 3 % of one 8 -> 8 launch).  graph_info then reports workgroups for n_tiles, graph_trace records
  * one entry per workgroup.  A graph all of whose entries are copies to three or more outputs runs that way
  * from 48 MiB in all (all-gather or broadcast over 8 ranks x 128 MiB: 235 -> 167 us).  Other copies and folds
  * over fewer streams fit that launch too but are better off with the table (PCCL_HIP_CHAIN_LAUNCH=2 takes it
